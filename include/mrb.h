@@ -1,0 +1,147 @@
+/*
+ * mrb.h — C ABI of the MI355X (gfx950) replay-buffer library, libmrb.so.
+ *
+ * The library replaces the MindSpore primitives that the reference's replay
+ * buffer classes call into (the classes themselves hold no arithmetic):
+ *   - uniform FIFO buffer: P.BufferAppend / P.BufferGetItem / P.BufferSample
+ *     (mindspore_rl/core/uniform_replay_buffer.py:82-89, used at :114,:128,:139)
+ *   - prioritized buffer:  PriorityReplayBufferCreate/Push/Sample/Update/Destroy
+ *     (mindspore_rl/core/priority_replay_buffer.py:21-27, used at :62-76,:90,:106,:120)
+ *
+ * Conventions (the in-repo precedent for a C operator ABI is
+ * mindspore_rl/utils/mcts/cpu/cpu_mcts_ops.cc:25,51-97: plain pointers,
+ * a device stream argument, int status, int64 handles from a registry,
+ * mindspore_rl/utils/mcts/mcts_factory.h:32,39-82):
+ *   - every function returns 0 on success and a non-zero MRB_E* code on error;
+ *     mrb_last_error() returns a thread-local message for the last failure.
+ *     Nothing throws or aborts across this boundary.
+ *   - a buffer is an opaque int64 handle (> 0) owned by a process-wide
+ *     registry; the library owns row storage, trees and scratch in HBM.
+ *   - all row data pointers (src_fields, dst_fields, indices, priorities,
+ *     uniforms, outputs) are DEVICE pointers; the caller owns them and keeps
+ *     them alive until the work enqueued on `stream` has completed.
+ *   - `stream` is a hipStream_t (NULL = the null stream). All device work is
+ *     enqueued on it in program order; only create/destroy/state/check/
+ *     export_tree synchronise. Calls on one handle must be serialised by the
+ *     caller (the reference orders them with side_effect_io,
+ *     priority_replay_buffer.py:67-76); different handles are independent.
+ *   - storage is structure-of-arrays: field i is one [capacity, field_bytes[i]]
+ *     byte matrix (reference layout: uniform_replay_buffer.py:26-47).
+ */
+#ifndef MRB_H_
+#define MRB_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MRB_OK 0
+#define MRB_EINVAL 1   /* bad argument (size, count, NULL pointer, alignment) */
+#define MRB_EHANDLE 2  /* unknown or destroyed handle (cf. kErrorCode = 2, cpu_mcts_ops.cc:25) */
+#define MRB_EHIP 3     /* a HIP runtime call failed */
+#define MRB_ESTATE 4   /* operation not valid in the buffer's state (e.g. sample from empty) */
+#define MRB_EDEVICE 5  /* a kernel recorded a data error (see mrb_per_check) */
+
+#define MRB_MAX_FIELDS 16
+
+/* Bits of the device-side data-error word reported by mrb_per_check. */
+#define MRB_DERR_INDEX 1u     /* update_priorities: index outside [0, capacity) — entry skipped */
+#define MRB_DERR_PRIORITY 2u  /* update_priorities/push: negative or non-finite priority — entry skipped */
+#define MRB_DERR_TOTAL 4u     /* sample: tree total not finite or <= 0 */
+#define MRB_DERR_UNFILLED 8u  /* sample: descent ended on a slot >= size */
+
+/* ---- library ---------------------------------------------------------- */
+
+/* Message of the calling thread's last failed call ("" if none). */
+const char *mrb_last_error(void);
+/* 1 = HIP/gfx950. (There is no CPU backend in this library.) */
+int mrb_backend(void);
+/* ABI version of this header. */
+int mrb_version(void);
+/* Tuning knobs; unknown names return MRB_EINVAL.
+ *   "sample_path"  0 = choose by row size, 1 = force wide-row kernel, 2 = force LDS-top kernel
+ *   "row_split"    workgroups per sampled row in the wide-row kernel (0 = auto)
+ *   "lds_levels"   tree levels staged in LDS by the LDS-top kernel (0 = auto, max 12) */
+int mrb_set_option(const char *name, int64_t value);
+
+/* ---- uniform FIFO ring buffer ----------------------------------------- */
+
+/* Replaces UniformReplayBuffer.__init__ storage + count/head
+ * (uniform_replay_buffer.py:75-80). Storage is zero-filled. */
+int mrb_urb_create(int64_t capacity, int nfields, const int64_t *field_bytes, int64_t *out_handle);
+/* Replaces P.BufferAppend (uniform_replay_buffer.py:82,114): FIFO append of
+ * nrows rows; src_fields[i] is a contiguous [nrows, field_bytes[i]] matrix.
+ * nrows > capacity keeps the last `capacity` rows. */
+int mrb_urb_append(int64_t h, const void *const *src_fields, int64_t nrows, void *stream);
+/* Replaces P.BufferGetItem (uniform_replay_buffer.py:83,128): row at LOGICAL
+ * position (0 = oldest, negative counts back from the newest) copied to
+ * dst_fields[i] ([field_bytes[i]] each). */
+int mrb_urb_get_item(int64_t h, int64_t logical_index, void *const *dst_fields, void *stream);
+/* Gather half of P.BufferSample (uniform_replay_buffer.py:87-89,139):
+ * dst_fields[i][k] = storage_i[indices[k]] for k < n, indices being physical
+ * slot numbers in [0, count). Out-of-range indices are clamped into range and
+ * reported by mrb_urb_check. */
+int mrb_urb_gather(int64_t h, const int64_t *indices, int64_t n, void *const *dst_fields, void *stream);
+/* Whole P.BufferSample: draws n slots uniformly in [0, count) with replacement
+ * from the buffer's counter-based generator (seeded at create-time by
+ * mrb_urb_seed; each call advances the counter, so successive calls differ),
+ * optionally writes them to out_indices (may be NULL), and gathers. */
+int mrb_urb_sample(int64_t h, int64_t n, int64_t *out_indices, void *const *dst_fields, void *stream);
+int mrb_urb_seed(int64_t h, uint64_t seed);
+/* count / head as the reference's int32 Parameters (uniform_replay_buffer.py:78-79). */
+int mrb_urb_state(int64_t h, int32_t *count, int32_t *head);
+/* Replaces UniformReplayBuffer.reset (uniform_replay_buffer.py:141-150): count = 0, head untouched. */
+int mrb_urb_reset(int64_t h);
+/* Synchronises `stream` and returns the device error word (MRB_DERR_INDEX) since the last check. */
+int mrb_urb_check(int64_t h, uint32_t *flags, void *stream);
+/* Device pointer of field storage [capacity, field_bytes[field]] (backs the `.buffer` attribute,
+ * read directly by callers: mindspore_rl/core/msrl.py:550). */
+int mrb_urb_field_ptr(int64_t h, int field, void **dev_ptr);
+int mrb_urb_destroy(int64_t h);
+
+/* ---- prioritized replay buffer ---------------------------------------- */
+
+/* Replaces PriorityReplayBufferCreate (priority_replay_buffer.py:62-66).
+ * Trees have next_pow2(capacity) leaves; max priority starts at 1.0. */
+int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t *field_bytes,
+                   uint64_t seed, int64_t *out_handle);
+/* Replaces PriorityReplayBufferPush (priority_replay_buffer.py:67-69,90), batched:
+ * equals nrows sequential pushes. Row j goes to slot (pushes + j) mod capacity.
+ * opt_priorities == NULL: each new leaf takes the running max priority (not
+ * raised to alpha). Otherwise (device f32[nrows]) the push is followed by
+ * update_priorities(new slots, opt_priorities). */
+int mrb_per_push(int64_t h, const void *const *src_fields, int64_t nrows, const float *opt_priorities,
+                 void *stream);
+/* Replaces PriorityReplayBufferSample (priority_replay_buffer.py:70,106).
+ * Stratified proportional sampling of `batch` rows: seg = total / batch,
+ * mass_k = (k + u_k) * seg, sum-tree descent (go left when mass <= left sum),
+ * weight_k = (p_k / total * size)^-beta / (p_min / total * size)^-beta,
+ * then the row gather. `uniforms` is device f32[batch] in [0,1) supplied by
+ * the caller, or NULL to use the buffer's counter-based generator.
+ * Outputs: out_indices int64[batch], out_weights f32[batch],
+ * out_fields[i] = [batch, field_bytes[i]]. */
+int mrb_per_sample(int64_t h, int64_t batch, float beta, const float *uniforms, int64_t *out_indices,
+                   float *out_weights, void *const *out_fields, void *stream);
+/* Replaces PriorityReplayBufferUpdate (priority_replay_buffer.py:71-73,120):
+ * leaf[indices[j]] = priorities[j]^alpha for j in order (last write wins on
+ * duplicates), every ancestor of a touched leaf recomputed from its final
+ * children; max priority = max(old, all priorities[j]^alpha). */
+int mrb_per_update(int64_t h, const int64_t *indices, const float *priorities, int64_t n, void *stream);
+/* Parity hook: copies both trees in canonical heap order (root at 1, leaf i at
+ * leaves + i, element 0 unused) to HOST arrays of 2 * leaves floats each.
+ * Either pointer may be NULL. Synchronises `stream`. */
+int mrb_per_export_tree(int64_t h, float *sum_heap, float *min_heap, int64_t *leaves, void *stream);
+/* Synchronises `stream`; size, next slot (pushes mod capacity) and running max priority. */
+int mrb_per_state(int64_t h, int64_t *size, int64_t *head, float *max_priority, void *stream);
+/* Synchronises `stream` and returns (then clears) the device error word. */
+int mrb_per_check(int64_t h, uint32_t *flags, void *stream);
+int mrb_per_field_ptr(int64_t h, int field, void **dev_ptr);
+/* Replaces PriorityReplayBufferDestroy (priority_replay_buffer.py:74-76,138). */
+int mrb_per_destroy(int64_t h);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MRB_H_ */

@@ -1,0 +1,96 @@
+"""ctypes binding of libmrb.so (C ABI declared in include/mrb.h).
+
+There is no fallback: if the library has not been built, or a call fails, an
+exception is raised. Build with `python -m mindrl_amd.build`.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libmrb.so")
+
+MRB_OK, MRB_EINVAL, MRB_EHANDLE, MRB_EHIP, MRB_ESTATE, MRB_EDEVICE = 0, 1, 2, 3, 4, 5
+DERR_INDEX, DERR_PRIORITY, DERR_TOTAL, DERR_UNFILLED = 1, 2, 4, 8
+MAX_FIELDS = 16
+
+_vp, _i64, _u64, _f32, _int = C.c_void_p, C.c_int64, C.c_uint64, C.c_float, C.c_int
+_pvp = C.POINTER(C.c_void_p)
+_pi64 = C.POINTER(C.c_int64)
+
+# name -> argtypes; every function returns int except mrb_last_error
+SIGNATURES = {
+    "mrb_backend": [],
+    "mrb_version": [],
+    "mrb_set_option": [C.c_char_p, _i64],
+    "mrb_urb_create": [_i64, _int, _pi64, _pi64],
+    "mrb_urb_append": [_i64, _pvp, _i64, _vp],
+    "mrb_urb_get_item": [_i64, _i64, _pvp, _vp],
+    "mrb_urb_gather": [_i64, _vp, _i64, _pvp, _vp],
+    "mrb_urb_sample": [_i64, _i64, _vp, _pvp, _vp],
+    "mrb_urb_seed": [_i64, _u64],
+    "mrb_urb_state": [_i64, C.POINTER(C.c_int32), C.POINTER(C.c_int32)],
+    "mrb_urb_reset": [_i64],
+    "mrb_urb_check": [_i64, C.POINTER(C.c_uint32), _vp],
+    "mrb_urb_field_ptr": [_i64, _int, _pvp],
+    "mrb_urb_destroy": [_i64],
+    "mrb_per_create": [_i64, _f32, _int, _pi64, _u64, _pi64],
+    "mrb_per_push": [_i64, _pvp, _i64, _vp, _vp],
+    "mrb_per_sample": [_i64, _i64, _f32, _vp, _vp, _vp, _pvp, _vp],
+    "mrb_per_update": [_i64, _vp, _vp, _i64, _vp],
+    "mrb_per_export_tree": [_i64, _vp, _vp, _pi64, _vp],
+    "mrb_per_state": [_i64, _pi64, _pi64, C.POINTER(C.c_float), _vp],
+    "mrb_per_check": [_i64, C.POINTER(C.c_uint32), _vp],
+    "mrb_per_field_ptr": [_i64, _int, _pvp],
+    "mrb_per_destroy": [_i64],
+}
+
+_lib = None
+
+
+class MrbError(RuntimeError):
+    """A libmrb call returned a non-zero status."""
+
+    def __init__(self, code, message):
+        super().__init__("libmrb error %d: %s" % (code, message))
+        self.code = code
+
+
+def lib():
+    """Loads libmrb.so once. Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "libmrb.so is missing (%s): build the HIP library with `python -m mindrl_amd.build`; "
+            "there is no CPU fallback" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    L.mrb_last_error.restype = C.c_char_p
+    L.mrb_last_error.argtypes = []
+    for name, args in SIGNATURES.items():
+        fn = getattr(L, name)
+        fn.restype = C.c_int
+        fn.argtypes = args
+    _lib = L
+    return L
+
+
+def check(rc):
+    """Maps a status code to the exception the reference's runtime would raise."""
+    if rc == MRB_OK:
+        return
+    msg = lib().mrb_last_error().decode("utf-8", "replace")
+    if rc in (MRB_EINVAL, MRB_EHANDLE, MRB_ESTATE):
+        raise ValueError("libmrb: " + msg)
+    raise MrbError(rc, msg)
+
+
+def set_option(name, value):
+    check(lib().mrb_set_option(name.encode(), int(value)))
+
+
+def ptr_array(pointers):
+    arr = (C.c_void_p * len(pointers))()
+    for i, p in enumerate(pointers):
+        arr[i] = p
+    return arr

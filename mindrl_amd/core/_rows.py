@@ -1,0 +1,111 @@
+"""Host-side plumbing shared by both buffer classes: field layout, tensor
+marshalling to device pointers, and views over library-owned storage."""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from .. import _lib
+from ..dtype import as_torch_dtype
+
+
+def device():
+    if not torch.cuda.is_available():
+        raise RuntimeError("mindrl_amd buffers need a HIP device (torch.cuda.is_available() is False); "
+                           "there is no CPU fallback")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def stream_ptr():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class _DeviceView:
+    """Exposes library-owned device memory to torch through __cuda_array_interface__."""
+
+    def __init__(self, ptr, shape, typestr, owner):
+        self.owner = owner  # keeps the buffer object (and so the allocation) alive
+        self.__cuda_array_interface__ = {
+            "shape": tuple(shape), "typestr": typestr, "data": (int(ptr), False), "version": 2, "strides": None,
+        }
+
+
+_TYPESTR = {
+    torch.float16: "<f2", torch.float32: "<f4", torch.float64: "<f8", torch.int8: "|i1", torch.int16: "<i2",
+    torch.int32: "<i4", torch.int64: "<i8", torch.uint8: "|u1", torch.bool: "|b1",
+}
+
+
+def view_of(ptr, shape, dtype, owner, dev):
+    """torch tensor aliasing `ptr` (no copy)."""
+    if dtype == torch.bfloat16:
+        t = torch.as_tensor(_DeviceView(ptr, shape, "<i2", owner), device=dev)
+        return t.view(torch.bfloat16)
+    return torch.as_tensor(_DeviceView(ptr, shape, _TYPESTR[dtype], owner), device=dev)
+
+
+class FieldLayout:
+    """Shapes/dtypes of one buffer element, as given to the reference constructors
+    (`shapes`, `types`: mindspore_rl/core/uniform_replay_buffer.py:75)."""
+
+    def __init__(self, shapes, types):
+        if len(shapes) != len(types):
+            raise ValueError("shapes and types differ in length")
+        if not 0 < len(shapes) <= _lib.MAX_FIELDS:
+            raise ValueError("a buffer element has between 1 and %d tensors" % _lib.MAX_FIELDS)
+        self.shapes = []
+        for s in shapes:
+            if isinstance(s, (int, np.integer)):
+                s = (int(s),)
+            self.shapes.append(tuple(int(v) for v in s))
+        self.dtypes = [as_torch_dtype(t) for t in types]
+        self.numel = [int(np.prod(s, dtype=np.int64)) if len(s) else 1 for s in self.shapes]
+        self.bytes = [n * torch.empty((), dtype=d).element_size() for n, d in zip(self.numel, self.dtypes)]
+        self.c_bytes = (C.c_int64 * len(self.bytes))(*self.bytes)
+
+    def __len__(self):
+        return len(self.shapes)
+
+    def batch_of(self, fields):
+        """Number of rows in `fields` (each either shape_i or [n, *shape_i])."""
+        if len(fields) != len(self):
+            raise ValueError("expected %d tensors per element, got %d" % (len(self), len(fields)))
+        n = None
+        for f, numel in zip(fields, self.numel):
+            total = int(np.prod(tuple(f.shape), dtype=np.int64)) if len(f.shape) else 1
+            if total % numel:
+                raise ValueError("tensor of shape %s does not hold whole elements of %d values" % (tuple(f.shape), numel))
+            rows = total // numel
+            if n is None:
+                n = rows
+            elif rows != n:
+                raise ValueError("fields disagree on the number of rows (%d vs %d)" % (n, rows))
+        return n
+
+    def to_device(self, fields, dev):
+        """Contiguous device tensors of the declared dtypes (copies host data if needed)."""
+        out = []
+        for f, d in zip(fields, self.dtypes):
+            t = f if isinstance(f, torch.Tensor) else torch.as_tensor(np.asarray(f))
+            t = t.to(device=dev, dtype=d, non_blocking=False).contiguous()
+            out.append(t)
+        return out
+
+    def empty(self, n, dev):
+        """Output tensors [n, *shape_i] (or shape_i when n is None)."""
+        if n is None:
+            return [torch.empty(s, dtype=d, device=dev) for s, d in zip(self.shapes, self.dtypes)]
+        return [torch.empty((n,) + s, dtype=d, device=dev) for s, d in zip(self.shapes, self.dtypes)]
+
+    def check_out(self, out, n, dev):
+        if len(out) != len(self):
+            raise ValueError("out must hold %d tensors" % len(self))
+        for t, s, d in zip(out, self.shapes, self.dtypes):
+            want = ((n,) + s) if n is not None else s
+            if tuple(t.shape) != want or t.dtype != d or t.device != dev or not t.is_contiguous():
+                raise ValueError("out tensor must be contiguous %s %s on %s" % (want, d, dev))
+        return list(out)
+
+
+def pointers(tensors):
+    return _lib.ptr_array([t.data_ptr() for t in tensors])

@@ -1,0 +1,171 @@
+"""PriorityReplayBuffer with the interface of
+mindspore_rl/core/priority_replay_buffer.py:30-138, backed by libmrb.so."""
+import ctypes as C
+import os
+
+import numpy as np
+import torch
+
+from .. import _lib
+from ._rows import FieldLayout, device, pointers, stream_ptr, view_of
+
+
+class PriorityReplayBuffer:
+    """Proportional prioritized replay (Schaul et al.) resident in HBM: FIFO rows
+    plus a sum tree and a min tree over next_pow2(capacity) leaves.
+
+    Same constructor and methods as the reference class
+    (mindspore_rl/core/priority_replay_buffer.py:60-138).
+
+    Args:
+        alpha (float): priority exponent; 0 = uniform, 1 = fully prioritized.
+        capacity (int): number of rows kept.
+        sample_size (int): rows returned by sample().
+        shapes, types: shape / element type of each tensor of an element.
+        seed0, seed1 (int): generator seed; seed1 if non-zero, else seed0, else entropy.
+    """
+
+    def __init__(self, alpha, capacity, sample_size, shapes, types, seed0=0, seed1=0):
+        self._dev = device()
+        self._layout = FieldLayout(shapes, types)
+        self._capacity = int(capacity)
+        self._sample_size = int(sample_size)
+        self._alpha = float(alpha)
+        seed = int(seed1) or int(seed0) or int.from_bytes(os.urandom(8), "little")
+        h = C.c_int64(0)
+        _lib.check(_lib.lib().mrb_per_create(self._capacity, self._alpha, len(self._layout), self._layout.c_bytes,
+                                             seed & (2**64 - 1), C.byref(h)))
+        self._h = h.value
+        self._handle = torch.tensor([self._h], dtype=torch.int64)
+        self._keep = None
+
+    # -- reference methods ---------------------------------------------------
+    def insert(self, *transition, priorities=None):
+        """Pushes one transition (tensors of shape_i) or a batch ([n, *shape_i]); the
+        oldest row is replaced when full; new rows take the running max priority
+        (priority_replay_buffer.py:78-90). `priorities` (f32[n]), if given, are
+        applied to the new rows as update_priorities would. Returns the handle
+        tensor int64[1]."""
+        if len(transition) == 1 and isinstance(transition[0], (list, tuple)):
+            transition = tuple(transition[0])
+        n = self._layout.batch_of(transition)
+        src = self._layout.to_device(transition, self._dev)
+        pr = None
+        if priorities is not None:
+            pr = torch.as_tensor(priorities).to(device=self._dev, dtype=torch.float32).contiguous().reshape(-1)
+            if pr.numel() != n:
+                raise ValueError("priorities must hold one value per pushed row")
+        _lib.check(_lib.lib().mrb_per_push(self._h, pointers(src), n, pr.data_ptr() if pr is not None else None,
+                                           stream_ptr()))
+        self._keep = (src, pr)
+        return self._handle
+
+    # the reference's own test calls the method by this name (tests/st/test_priority_replay_buffer.py:46)
+    push = insert
+
+    def sample(self, beta, uniforms=None, out=None):
+        """Stratified proportional sample of `sample_size` rows
+        (priority_replay_buffer.py:92-106).
+
+        Returns (indices int64[B], weights f32[B], *transitions [B, *shape_i]).
+        `uniforms` (f32[B] in [0,1)) replaces the buffer's generator, stratum k
+        using uniforms[k]. `out` = (indices, weights, [fields]) reuses output tensors."""
+        n = self._sample_size
+        u = None
+        if uniforms is not None:
+            u = torch.as_tensor(uniforms).to(device=self._dev, dtype=torch.float32).contiguous().reshape(-1)
+            if u.numel() != n:
+                raise ValueError("uniforms must hold sample_size = %d values" % n)
+        if out is not None:
+            idx, w, fields = out
+            fields = self._layout.check_out(fields, n, self._dev)
+        else:
+            idx = torch.empty(n, dtype=torch.int64, device=self._dev)
+            w = torch.empty(n, dtype=torch.float32, device=self._dev)
+            fields = self._layout.empty(n, self._dev)
+        _lib.check(_lib.lib().mrb_per_sample(self._h, n, float(beta), u.data_ptr() if u is not None else None,
+                                             idx.data_ptr(), w.data_ptr(), pointers(fields), stream_ptr()))
+        self._keep = u
+        return (idx, w) + tuple(fields)
+
+    def update_priorities(self, indices, priorities):
+        """leaf[indices[j]] = priorities[j] ** alpha in order, last write wins
+        (priority_replay_buffer.py:108-120). Returns the handle tensor."""
+        idx = torch.as_tensor(indices).to(device=self._dev, dtype=torch.int64).contiguous().reshape(-1)
+        pr = torch.as_tensor(priorities).to(device=self._dev, dtype=torch.float32).contiguous().reshape(-1)
+        if idx.numel() != pr.numel():
+            raise ValueError("indices and priorities differ in length")
+        _lib.check(_lib.lib().mrb_per_update(self._h, idx.data_ptr(), pr.data_ptr(), idx.numel(), stream_ptr()))
+        self._keep = (idx, pr)
+        return self._handle
+
+    def full(self):
+        """Always False, as in the reference (priority_replay_buffer.py:122-124)."""
+        return torch.tensor(False)
+
+    def reset(self):
+        """Not supported, as in the reference (priority_replay_buffer.py:126-128)."""
+        raise ValueError("reset() is not supported by PriorityReplayBuffer.")
+
+    def destroy(self):
+        """Releases the native buffer (priority_replay_buffer.py:130-138)."""
+        if self._h:
+            h, self._h = self._h, 0
+            _lib.check(_lib.lib().mrb_per_destroy(h))
+        return self._handle
+
+    # -- extras ----------------------------------------------------------------
+    def size(self):
+        return self._state()[0]
+
+    @property
+    def max_priority(self):
+        return self._state(True)[2]
+
+    @property
+    def capacity(self):
+        return self._capacity
+
+    @property
+    def sample_size(self):
+        return self._sample_size
+
+    def _state(self, with_max=False):
+        s, hd, mp = C.c_int64(0), C.c_int64(0), C.c_float(0)
+        _lib.check(_lib.lib().mrb_per_state(self._h, C.byref(s), C.byref(hd), C.byref(mp) if with_max else None,
+                                            stream_ptr()))
+        return s.value, hd.value, mp.value
+
+    def export_tree(self):
+        """(sum_heap, min_heap) as numpy float32[2 * leaves], root at 1, leaf i at leaves + i."""
+        leaves = C.c_int64(0)
+        _lib.check(_lib.lib().mrb_per_export_tree(self._h, None, None, C.byref(leaves), stream_ptr()))
+        s = np.empty(2 * leaves.value, np.float32)
+        m = np.empty(2 * leaves.value, np.float32)
+        _lib.check(_lib.lib().mrb_per_export_tree(self._h, s.ctypes.data, m.ctypes.data, None, stream_ptr()))
+        return s, m
+
+    def storage(self):
+        """Views of the row storage, one [capacity, *shape_i] tensor per field."""
+        views = []
+        for i, (s, d) in enumerate(zip(self._layout.shapes, self._layout.dtypes)):
+            p = C.c_void_p()
+            _lib.check(_lib.lib().mrb_per_field_ptr(self._h, i, C.byref(p)))
+            views.append(view_of(p.value, (self._capacity,) + s, d, self, self._dev))
+        return tuple(views)
+
+    def check(self):
+        """Synchronises; raises if a kernel recorded a data error since the last check."""
+        flags = C.c_uint32(0)
+        _lib.check(_lib.lib().mrb_per_check(self._h, C.byref(flags), stream_ptr()))
+        f = flags.value
+        if f & _lib.DERR_INDEX:
+            raise IndexError("update_priorities: index outside [0, capacity)")
+        if f & _lib.DERR_PRIORITY:
+            raise ValueError("update_priorities: negative or non-finite priority")
+        if f & _lib.DERR_TOTAL:
+            raise ValueError("sample: total priority is not positive and finite")
+        return f
+
+    def __repr__(self):
+        return "PriorityReplayBuffer<>"

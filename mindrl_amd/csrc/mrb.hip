@@ -1,0 +1,607 @@
+// libmrb.so — C ABI (include/mrb.h) over the HIP kernels in mrb_kernels.h.
+// Host side: handle registry, ring/tree bookkeeping, argument checks, launches.
+// Nothing in this file computes a result on the CPU; without a HIP device every
+// entry point that touches a buffer fails with MRB_EHIP.
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <unordered_map>
+
+#include "mrb_kernels.h"
+
+namespace {
+
+using namespace mrb;
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                          \
+    do {                                                                                       \
+        hipError_t e_ = (expr);                                                                \
+        if (e_ != hipSuccess) return fail(MRB_EHIP, "%s: %s", #expr, hipGetErrorString(e_));    \
+    } while (0)
+
+#define LAUNCH_CHECK(name)                                                                     \
+    do {                                                                                       \
+        hipError_t e_ = hipGetLastError();                                                     \
+        if (e_ != hipSuccess) return fail(MRB_EHIP, "launch %s: %s", name, hipGetErrorString(e_)); \
+    } while (0)
+
+struct Options {
+    int64_t sample_path = 0;
+    int64_t row_split = 0;
+    int64_t lds_levels = 0;
+} g_opt;
+
+// Row storage: structure of arrays, field i = [capacity, bytes_i]
+// (reference layout: mindspore_rl/core/uniform_replay_buffer.py:26-47).
+struct RowStore {
+    int64_t capacity = 0;
+    int nfields = 0;
+    int64_t bytes[MRB_MAX_FIELDS] = {};
+    uint8_t* data[MRB_MAX_FIELDS] = {};
+    uint32_t vec_log2[MRB_MAX_FIELDS] = {};
+    uint32_t units[MRB_MAX_FIELDS] = {};
+
+    ~RowStore() {
+        for (int i = 0; i < nfields; ++i)
+            if (data[i]) (void)hipFree(data[i]);
+    }
+};
+
+int rows_alloc(RowStore& r, int64_t capacity, int nfields, const int64_t* field_bytes) {
+    if (capacity <= 0 || capacity > (1ll << 30)) return fail(MRB_EINVAL, "capacity %lld outside [1, 2^30]", (long long)capacity);
+    if (nfields <= 0 || nfields > MRB_MAX_FIELDS) return fail(MRB_EINVAL, "nfields %d outside [1, %d]", nfields, MRB_MAX_FIELDS);
+    if (!field_bytes) return fail(MRB_EINVAL, "field_bytes is NULL");
+    for (int i = 0; i < nfields; ++i)
+        if (field_bytes[i] <= 0 || field_bytes[i] > (1ll << 30))
+            return fail(MRB_EINVAL, "field_bytes[%d] = %lld outside [1, 2^30]", i, (long long)field_bytes[i]);
+    r.capacity = capacity;
+    for (int i = 0; i < nfields; ++i) {
+        r.bytes[i] = field_bytes[i];
+        uint32_t vl = 4;
+        while (vl > 0 && (field_bytes[i] & ((1ll << vl) - 1))) --vl;
+        r.vec_log2[i] = vl;
+        r.units[i] = (uint32_t)(field_bytes[i] >> vl);
+        const size_t total = (size_t)capacity * (size_t)field_bytes[i];
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&r.data[i]), total));
+        r.nfields = i + 1;  // so the destructor frees what exists
+        HIP_TRY(hipMemset(r.data[i], 0, total));
+    }
+    return MRB_OK;
+}
+
+// Builds the per-call field table. `io` pointers must honour each field's copy granule.
+int make_table(const RowStore& r, const void* const* io, int64_t n, IoTable& t) {
+    if (!io) return fail(MRB_EINVAL, "field pointer array is NULL");
+    t.nfields = r.nfields;
+    t.prefix[0] = 0;
+    for (int i = 0; i < r.nfields; ++i) {
+        if (!io[i]) return fail(MRB_EINVAL, "field %d pointer is NULL", i);
+        if (reinterpret_cast<uintptr_t>(io[i]) & ((1u << r.vec_log2[i]) - 1))
+            return fail(MRB_EINVAL, "field %d pointer %p is not %u-byte aligned", i, io[i], 1u << r.vec_log2[i]);
+        t.store[i] = r.data[i];
+        t.io[i] = const_cast<uint8_t*>(static_cast<const uint8_t*>(io[i]));
+        t.row_bytes[i] = (uint32_t)r.bytes[i];
+        t.units[i] = r.units[i];
+        t.vec_log2[i] = r.vec_log2[i];
+        t.prefix[i + 1] = t.prefix[i] + (uint64_t)n * r.units[i];
+    }
+    return MRB_OK;
+}
+
+uint32_t grid_for(uint64_t work, uint32_t per_thread = 1) {
+    uint64_t g = (work + (uint64_t)kWG * per_thread - 1) / ((uint64_t)kWG * per_thread);
+    if (g < 1) g = 1;
+    if (g > 16384) g = 16384;
+    return (uint32_t)g;
+}
+
+// One thread per entry, no grid-stride loop (n < 2^32, so the grid fits).
+uint32_t grid_exact(uint64_t n) { return (uint32_t)((n + kWG - 1) / kWG); }
+
+// Appends rows [skip, nrows) of the caller's matrices at ring position first_slot.
+int rows_put(const RowStore& r, const void* const* src, int64_t skip, int64_t n, int64_t first_slot, hipStream_t s) {
+    IoTable t;
+    const void* shifted[MRB_MAX_FIELDS];
+    if (!src) return fail(MRB_EINVAL, "field pointer array is NULL");
+    for (int i = 0; i < r.nfields; ++i) {
+        if (!src[i]) return fail(MRB_EINVAL, "field %d pointer is NULL", i);
+        shifted[i] = static_cast<const uint8_t*>(src[i]) + skip * r.bytes[i];
+    }
+    int rc = make_table(r, shifted, n, t);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_rows_put, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, r.capacity, first_slot);
+    LAUNCH_CHECK("k_rows_put");
+    return MRB_OK;
+}
+
+struct Urb {
+    RowStore rows;
+    int64_t count = 0, head = 0;
+    uint64_t seed = 0, calls = 0;
+    uint32_t* err = nullptr;
+    ~Urb() {
+        if (err) (void)hipFree(err);
+    }
+};
+
+struct Per {
+    RowStore rows;
+    int64_t leaves = 1;
+    int depth = 0;
+    int64_t size = 0, pushes = 0;
+    float alpha = 1.0f;
+    float* sum = nullptr;
+    float* mn = nullptr;
+    unsigned long long* stamp = nullptr;
+    float* maxp = nullptr;
+    uint32_t* err = nullptr;
+    uint32_t* dirty[4] = {};
+    int nrounds = 0;
+    int top_depth = 0;
+    uint64_t epoch = 0;
+    uint64_t seed = 0, calls = 0;
+    ~Per() {
+        if (sum) (void)hipFree(sum);
+        if (mn) (void)hipFree(mn);
+        if (stamp) (void)hipFree(stamp);
+        if (maxp) (void)hipFree(maxp);
+        if (err) (void)hipFree(err);
+        for (auto* d : dirty)
+            if (d) (void)hipFree(d);
+    }
+};
+
+std::mutex g_mu;
+int64_t g_next = 1;
+std::unordered_map<int64_t, std::shared_ptr<Urb>> g_urb;
+std::unordered_map<int64_t, std::shared_ptr<Per>> g_per;
+
+std::shared_ptr<Urb> find_urb(int64_t h) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_urb.find(h);
+    return it == g_urb.end() ? nullptr : it->second;
+}
+std::shared_ptr<Per> find_per(int64_t h) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_per.find(h);
+    return it == g_per.end() ? nullptr : it->second;
+}
+
+#define GET_URB(b, h)                                                              \
+    auto b = find_urb(h);                                                          \
+    if (!b) return fail(MRB_EHANDLE, "unknown uniform buffer handle %lld", (long long)(h))
+#define GET_PER(b, h)                                                              \
+    auto b = find_per(h);                                                          \
+    if (!b) return fail(MRB_EHANDLE, "unknown priority buffer handle %lld", (long long)(h))
+
+int read_and_clear_flags(uint32_t* d_err, uint32_t* flags, hipStream_t s) {
+    uint32_t v = 0;
+    HIP_TRY(hipMemcpyAsync(&v, d_err, sizeof(v), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    if (v) {
+        HIP_TRY(hipMemsetAsync(d_err, 0, sizeof(v), s));
+        HIP_TRY(hipStreamSynchronize(s));
+    }
+    if (flags) *flags = v;
+    return MRB_OK;
+}
+
+// Rebuilds every internal node above the leaves marked dirty in this epoch.
+int tree_rebuild(Per& b, hipStream_t s) {
+    const uint32_t epoch32 = (uint32_t)b.epoch;
+    for (int r = 0; r < b.nrounds; ++r) {
+        const int lo = b.depth - kRoundLevels * r;
+        const uint32_t nblocks = (1u << lo) / kBlockNodes;
+        hipLaunchKernelGGL(k_tree_round, dim3((nblocks + 3) / 4), dim3(kWG), 0, s, b.sum, b.mn, lo, b.dirty[r], epoch32);
+        LAUNCH_CHECK("k_tree_round");
+    }
+    if (b.top_depth > 0) {
+        hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, b.sum, b.mn, b.top_depth);
+        LAUNCH_CHECK("k_tree_top");
+    }
+    return MRB_OK;
+}
+
+// Starts a new tree-update epoch. Epochs tag stamps and dirty words so that
+// neither needs clearing between calls; when the 32-bit tag would wrap, both
+// are cleared once.
+int next_epoch(Per& b, hipStream_t s) {
+    b.epoch += 1;
+    if ((uint32_t)b.epoch == 0) {
+        HIP_TRY(hipMemsetAsync(b.stamp, 0, sizeof(unsigned long long) * (size_t)b.leaves, s));
+        for (int r = 0; r < b.nrounds; ++r) {
+            const size_t nblocks = ((size_t)1 << (b.depth - kRoundLevels * r)) / kBlockNodes;
+            HIP_TRY(hipMemsetAsync(b.dirty[r], 0, sizeof(uint32_t) * nblocks, s));
+        }
+        b.epoch += 1;
+    }
+    return MRB_OK;
+}
+
+UpdateArgs update_args(Per& b) {
+    UpdateArgs a{};
+    a.capacity = b.rows.capacity;
+    a.leaves = b.leaves;
+    a.alpha = b.alpha;
+    a.epoch = (uint32_t)b.epoch;
+    a.stamp = b.stamp;
+    a.sum = b.sum;
+    a.mn = b.mn;
+    a.maxp = b.maxp;
+    a.err = b.err;
+    for (int r = 0; r < 4; ++r) a.dirty[r] = b.dirty[r];
+    a.nrounds = b.nrounds;
+    return a;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mrb_last_error(void) { return g_err; }
+int mrb_backend(void) { return 1; }
+int mrb_version(void) { return 1; }
+
+int mrb_set_option(const char* name, int64_t value) {
+    if (!name) return fail(MRB_EINVAL, "option name is NULL");
+    if (!strcmp(name, "sample_path")) {
+        if (value < 0 || value > 2) return fail(MRB_EINVAL, "sample_path must be 0, 1 or 2");
+        g_opt.sample_path = value;
+    } else if (!strcmp(name, "row_split")) {
+        if (value < 0 || value > 64) return fail(MRB_EINVAL, "row_split must be in [0, 64]");
+        g_opt.row_split = value;
+    } else if (!strcmp(name, "lds_levels")) {
+        if (value < 0 || value > 12) return fail(MRB_EINVAL, "lds_levels must be in [0, 12]");
+        g_opt.lds_levels = value;
+    } else {
+        return fail(MRB_EINVAL, "unknown option '%s'", name);
+    }
+    return MRB_OK;
+}
+
+/* ---------------------------------------------------------------- uniform */
+
+int mrb_urb_create(int64_t capacity, int nfields, const int64_t* field_bytes, int64_t* out_handle) {
+    if (!out_handle) return fail(MRB_EINVAL, "out_handle is NULL");
+    if (capacity > 0x7fffffffll) return fail(MRB_EINVAL, "capacity %lld does not fit the int32 count", (long long)capacity);
+    auto b = std::make_shared<Urb>();
+    int rc = rows_alloc(b->rows, capacity, nfields, field_bytes);
+    if (rc) return rc;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16));
+    HIP_TRY(hipMemset(b->err, 0, 16));
+    std::lock_guard<std::mutex> lk(g_mu);
+    *out_handle = g_next++;
+    g_urb[*out_handle] = b;
+    return MRB_OK;
+}
+
+int mrb_urb_append(int64_t h, const void* const* src_fields, int64_t nrows, void* stream) {
+    GET_URB(b, h);
+    if (nrows <= 0) return fail(MRB_EINVAL, "nrows %lld must be positive", (long long)nrows);
+    const int64_t cap = b->rows.capacity;
+    // Write position: `count` while the buffer has never wrapped, else `head` (the oldest row).
+    const bool growing = b->count < cap && b->head == 0;
+    const int64_t w = growing ? b->count : b->head;
+    // More rows than slots: only the last `cap` survive, at the positions a row-by-row append leaves them.
+    const int64_t skip = nrows > cap ? nrows - cap : 0;
+    const int64_t first = (w + skip) % cap;
+    int rc = rows_put(b->rows, src_fields, skip, nrows - skip, first, static_cast<hipStream_t>(stream));
+    if (rc) return rc;
+    if (growing) {
+        const int64_t room = cap - b->count;
+        if (nrows <= room) {
+            b->count += nrows;
+        } else {
+            b->count = cap;
+            b->head = (nrows - room) % cap;
+        }
+    } else {
+        b->head = (b->head + nrows) % cap;
+        b->count = b->count + nrows < cap ? b->count + nrows : cap;
+    }
+    return MRB_OK;
+}
+
+static int urb_gather_impl(Urb& b, const int64_t* indices, int64_t fixed_slot, int64_t n, int64_t* out_indices,
+                           void* const* dst_fields, hipStream_t s) {
+    IoTable t;
+    int rc = make_table(b.rows, dst_fields, n, t);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, b.rows.capacity,
+                       b.count, indices, fixed_slot, b.seed, b.calls, out_indices, b.err);
+    LAUNCH_CHECK("k_rows_gather");
+    return MRB_OK;
+}
+
+int mrb_urb_get_item(int64_t h, int64_t logical_index, void* const* dst_fields, void* stream) {
+    GET_URB(b, h);
+    int64_t i = logical_index;
+    if (i < 0) i += b->count;
+    if (i < 0 || i >= b->count)
+        return fail(MRB_EINVAL, "index %lld outside the %lld stored rows", (long long)logical_index, (long long)b->count);
+    const int64_t t = b->count - b->head;
+    const int64_t slot = i < t ? i + b->head : i - t;
+    return urb_gather_impl(*b, nullptr, slot, 1, nullptr, dst_fields, static_cast<hipStream_t>(stream));
+}
+
+int mrb_urb_gather(int64_t h, const int64_t* indices, int64_t n, void* const* dst_fields, void* stream) {
+    GET_URB(b, h);
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (!indices) return fail(MRB_EINVAL, "indices is NULL");
+    if (b->count <= 0) return fail(MRB_ESTATE, "gather from an empty buffer");
+    return urb_gather_impl(*b, indices, -1, n, nullptr, dst_fields, static_cast<hipStream_t>(stream));
+}
+
+int mrb_urb_sample(int64_t h, int64_t n, int64_t* out_indices, void* const* dst_fields, void* stream) {
+    GET_URB(b, h);
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (n > b->count)
+        return fail(MRB_ESTATE, "sample size %lld exceeds the %lld stored rows", (long long)n, (long long)b->count);
+    int rc = urb_gather_impl(*b, nullptr, -1, n, out_indices, dst_fields, static_cast<hipStream_t>(stream));
+    if (rc) return rc;
+    b->calls += 1;
+    return MRB_OK;
+}
+
+int mrb_urb_seed(int64_t h, uint64_t seed) {
+    GET_URB(b, h);
+    b->seed = seed;
+    b->calls = 0;
+    return MRB_OK;
+}
+
+int mrb_urb_state(int64_t h, int32_t* count, int32_t* head) {
+    GET_URB(b, h);
+    if (count) *count = (int32_t)b->count;
+    if (head) *head = (int32_t)b->head;
+    return MRB_OK;
+}
+
+int mrb_urb_reset(int64_t h) {
+    GET_URB(b, h);
+    b->count = 0;
+    return MRB_OK;
+}
+
+int mrb_urb_check(int64_t h, uint32_t* flags, void* stream) {
+    GET_URB(b, h);
+    return read_and_clear_flags(b->err, flags, static_cast<hipStream_t>(stream));
+}
+
+int mrb_urb_field_ptr(int64_t h, int field, void** dev_ptr) {
+    GET_URB(b, h);
+    if (field < 0 || field >= b->rows.nfields || !dev_ptr) return fail(MRB_EINVAL, "bad field %d", field);
+    *dev_ptr = b->rows.data[field];
+    return MRB_OK;
+}
+
+int mrb_urb_destroy(int64_t h) {
+    std::shared_ptr<Urb> b;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        auto it = g_urb.find(h);
+        if (it == g_urb.end()) return fail(MRB_EHANDLE, "unknown uniform buffer handle %lld", (long long)h);
+        b = it->second;
+        g_urb.erase(it);
+    }
+    HIP_TRY(hipDeviceSynchronize());
+    return MRB_OK;
+}
+
+/* ------------------------------------------------------------ prioritized */
+
+int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* field_bytes, uint64_t seed,
+                   int64_t* out_handle) {
+    if (!out_handle) return fail(MRB_EINVAL, "out_handle is NULL");
+    if (!(alpha >= 0.0f) || alpha > 16.0f) return fail(MRB_EINVAL, "alpha %g outside [0, 16]", (double)alpha);
+    auto b = std::make_shared<Per>();
+    int rc = rows_alloc(b->rows, capacity, nfields, field_bytes);
+    if (rc) return rc;
+    while (b->leaves < capacity) {
+        b->leaves <<= 1;
+        b->depth += 1;
+    }
+    b->alpha = alpha;
+    b->seed = seed;
+    b->nrounds = b->depth > kTopMaxDepth ? (b->depth - kTopMaxDepth + kRoundLevels - 1) / kRoundLevels : 0;
+    b->top_depth = b->depth - kRoundLevels * b->nrounds;
+    const size_t nodes = 2 * (size_t)b->leaves;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->sum), nodes * sizeof(float)));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->mn), nodes * sizeof(float)));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->stamp), (size_t)b->leaves * sizeof(unsigned long long)));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->maxp), 16));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16));
+    HIP_TRY(hipMemset(b->sum, 0, nodes * sizeof(float)));
+    HIP_TRY(hipMemset(b->stamp, 0, (size_t)b->leaves * sizeof(unsigned long long)));
+    HIP_TRY(hipMemset(b->err, 0, 16));
+    for (int r = 0; r < b->nrounds; ++r) {
+        const size_t nblocks = ((size_t)1 << (b->depth - kRoundLevels * r)) / kBlockNodes;
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->dirty[r]), nblocks * sizeof(uint32_t)));
+        HIP_TRY(hipMemset(b->dirty[r], 0, nblocks * sizeof(uint32_t)));
+    }
+    hipLaunchKernelGGL(k_fill_f32, dim3(grid_for(nodes)), dim3(kWG), 0, nullptr, b->mn, FLT_MAX, (uint64_t)nodes);
+    LAUNCH_CHECK("k_fill_f32");
+    const float one = 1.0f;
+    HIP_TRY(hipMemcpy(b->maxp, &one, sizeof(one), hipMemcpyHostToDevice));
+    HIP_TRY(hipDeviceSynchronize());
+    std::lock_guard<std::mutex> lk(g_mu);
+    *out_handle = g_next++;
+    g_per[*out_handle] = b;
+    return MRB_OK;
+}
+
+int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const float* opt_priorities, void* stream) {
+    GET_PER(b, h);
+    if (nrows <= 0) return fail(MRB_EINVAL, "nrows %lld must be positive", (long long)nrows);
+    if (nrows > 0x7fffffffll) return fail(MRB_EINVAL, "nrows %lld exceeds 2^31 - 1 rows per call", (long long)nrows);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t cap = b->rows.capacity;
+    const int64_t skip = nrows > cap ? nrows - cap : 0;  // rows overwritten within this very call
+    const int64_t n = nrows - skip;
+    const int64_t first = (b->pushes + skip) % cap;
+    int rc = rows_put(b->rows, src_fields, skip, n, first, s);
+    if (rc) return rc;
+    rc = next_epoch(*b, s);
+    if (rc) return rc;
+    UpdateArgs a = update_args(*b);
+    a.first_slot = first;
+    a.n = n;
+    if (opt_priorities) {
+        // push-then-update: the running max sees every priority of the call, surviving or not
+        a.priorities = opt_priorities;
+        a.stamp = nullptr;
+        a.n = nrows;
+        a.first_slot = b->pushes % cap;
+        hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)nrows)), dim3(kWG), 0, s, a);
+        LAUNCH_CHECK("k_update_stamp");
+        a.priorities = opt_priorities + skip;
+        a.n = n;
+        a.first_slot = first;
+        a.stamp = b->stamp;
+    }
+    hipLaunchKernelGGL(k_update_leaves, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
+    LAUNCH_CHECK("k_update_leaves");
+    rc = tree_rebuild(*b, s);
+    if (rc) return rc;
+    b->pushes += nrows;
+    b->size = b->size + nrows < cap ? b->size + nrows : cap;
+    return MRB_OK;
+}
+
+int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, int64_t n, void* stream) {
+    GET_PER(b, h);
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (n > 0xffffffffll) return fail(MRB_EINVAL, "n %lld exceeds 2^32 - 1 entries per call", (long long)n);
+    if (!indices || !priorities) return fail(MRB_EINVAL, "indices or priorities is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rc = next_epoch(*b, s);
+    if (rc) return rc;
+    UpdateArgs a = update_args(*b);
+    a.indices = indices;
+    a.priorities = priorities;
+    a.n = n;
+    hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
+    LAUNCH_CHECK("k_update_stamp");
+    hipLaunchKernelGGL(k_update_leaves, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
+    LAUNCH_CHECK("k_update_leaves");
+    return tree_rebuild(*b, s);
+}
+
+int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, int64_t* out_indices,
+                   float* out_weights, void* const* out_fields, void* stream) {
+    GET_PER(b, h);
+    if (batch <= 0 || batch > (1ll << 24)) return fail(MRB_EINVAL, "batch %lld outside [1, 2^24]", (long long)batch);
+    if (!out_indices || !out_weights) return fail(MRB_EINVAL, "out_indices or out_weights is NULL");
+    if (b->size <= 0) return fail(MRB_ESTATE, "sample from an empty buffer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    IoTable t;
+    int rc = make_table(b->rows, out_fields, batch, t);
+    if (rc) return rc;
+    SampleArgs a{};
+    a.sum = b->sum;
+    a.mn = b->mn;
+    a.depth = b->depth;
+    a.leaves = b->leaves;
+    a.capacity = b->rows.capacity;
+    a.size = b->size;
+    a.batch = batch;
+    a.beta = beta;
+    a.uniforms = uniforms;
+    a.seed = b->seed;
+    a.calls = b->calls;
+    a.out_idx = out_indices;
+    a.out_w = out_weights;
+    a.err = b->err;
+    uint32_t max_units = 0;
+    int64_t max_bytes = 0;
+    for (int i = 0; i < b->rows.nfields; ++i) {
+        if (b->rows.units[i] > max_units) max_units = b->rows.units[i];
+        if (b->rows.bytes[i] > max_bytes) max_bytes = b->rows.bytes[i];
+    }
+    int path = (int)g_opt.sample_path;
+    if (path == 0) path = (batch >= 8192 && max_bytes <= 256) ? 2 : 1;
+    if (path == 1) {
+        int split = (int)g_opt.row_split;
+        if (split <= 0) {
+            split = (int)((max_units + 2 * kWG - 1) / (2 * kWG));  // about two granules per thread
+            if (split < 1) split = 1;
+            if (split > 16) split = 16;
+        }
+        hipLaunchKernelGGL(k_per_sample_wide, dim3((uint32_t)(batch * split)), dim3(kWG), 0, s, t, a, split);
+        LAUNCH_CHECK("k_per_sample_wide");
+    } else {
+        int levels = g_opt.lds_levels > 0 ? (int)g_opt.lds_levels : 12;
+        if (levels > b->depth) levels = b->depth;
+        const uint32_t ntop = (2u << levels) < 4 ? 4 : (2u << levels);
+        const size_t lds = ntop * sizeof(float) + kWG * sizeof(int64_t);
+        hipLaunchKernelGGL(k_per_sample_lds, dim3((uint32_t)((batch + kWG - 1) / kWG)), dim3(kWG), lds, s, t, a, levels);
+        LAUNCH_CHECK("k_per_sample_lds");
+    }
+    if (!uniforms) b->calls += 1;
+    return MRB_OK;
+}
+
+int mrb_per_export_tree(int64_t h, float* sum_heap, float* min_heap, int64_t* leaves, void* stream) {
+    GET_PER(b, h);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t bytes = 2 * (size_t)b->leaves * sizeof(float);
+    HIP_TRY(hipStreamSynchronize(s));
+    if (sum_heap) HIP_TRY(hipMemcpy(sum_heap, b->sum, bytes, hipMemcpyDeviceToHost));
+    if (min_heap) HIP_TRY(hipMemcpy(min_heap, b->mn, bytes, hipMemcpyDeviceToHost));
+    if (leaves) *leaves = b->leaves;
+    return MRB_OK;
+}
+
+int mrb_per_state(int64_t h, int64_t* size, int64_t* head, float* max_priority, void* stream) {
+    GET_PER(b, h);
+    if (size) *size = b->size;
+    if (head) *head = b->pushes % b->rows.capacity;
+    if (max_priority) {
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        HIP_TRY(hipMemcpyAsync(max_priority, b->maxp, sizeof(float), hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+    }
+    return MRB_OK;
+}
+
+int mrb_per_check(int64_t h, uint32_t* flags, void* stream) {
+    GET_PER(b, h);
+    return read_and_clear_flags(b->err, flags, static_cast<hipStream_t>(stream));
+}
+
+int mrb_per_field_ptr(int64_t h, int field, void** dev_ptr) {
+    GET_PER(b, h);
+    if (field < 0 || field >= b->rows.nfields || !dev_ptr) return fail(MRB_EINVAL, "bad field %d", field);
+    *dev_ptr = b->rows.data[field];
+    return MRB_OK;
+}
+
+int mrb_per_destroy(int64_t h) {
+    std::shared_ptr<Per> b;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        auto it = g_per.find(h);
+        if (it == g_per.end()) return fail(MRB_EHANDLE, "unknown priority buffer handle %lld", (long long)h);
+        b = it->second;
+        g_per.erase(it);
+    }
+    HIP_TRY(hipDeviceSynchronize());
+    return MRB_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,455 @@
+// HIP kernels of the replay-buffer library (gfx950, wave64). No MFMA: nothing
+// here is a dense contraction; the row kernels are HBM copies and the tree
+// kernels are latency/LDS work.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mrb.h"
+#include "mrb_device.h"
+
+namespace mrb {
+
+constexpr int kWG = 256;          // threads per workgroup of the row and sample kernels
+constexpr int kRoundLevels = 8;   // tree levels rebuilt by one pass of k_tree_round
+constexpr int kBlockNodes = 256;  // nodes per wave in k_tree_round (float4 per lane)
+constexpr int kTopMaxDepth = 12;  // deepest level k_tree_top starts from (4096 nodes)
+
+// Per-call table of the fields of a row, passed to kernels by value.
+// `store` is the buffer's [capacity, row_bytes] matrix, `io` the caller's
+// contiguous [n, row_bytes] matrix (source of an append, destination of a gather).
+struct IoTable {
+    int nfields;
+    uint8_t* store[MRB_MAX_FIELDS];
+    uint8_t* io[MRB_MAX_FIELDS];
+    uint32_t row_bytes[MRB_MAX_FIELDS];
+    uint32_t units[MRB_MAX_FIELDS];     // row_bytes >> vec_log2
+    uint32_t vec_log2[MRB_MAX_FIELDS];  // copy granule: 16, 8, 4, 2 or 1 bytes
+    uint64_t prefix[MRB_MAX_FIELDS + 1];  // running sum of n * units over fields
+};
+
+// One granule of 1 << vl bytes. Rows are read once and written once, so both
+// sides bypass the caches' retention (non-temporal).
+__device__ __forceinline__ void copy_granule(uint8_t* dst, const uint8_t* src, uint32_t vl) {
+    switch (vl) {
+        case 4: {
+            using v4 = __attribute__((ext_vector_type(4))) uint32_t;
+            v4 t = __builtin_nontemporal_load(reinterpret_cast<const v4*>(src));
+            __builtin_nontemporal_store(t, reinterpret_cast<v4*>(dst));
+            break;
+        }
+        case 3: {
+            using v2 = __attribute__((ext_vector_type(2))) uint32_t;
+            v2 t = __builtin_nontemporal_load(reinterpret_cast<const v2*>(src));
+            __builtin_nontemporal_store(t, reinterpret_cast<v2*>(dst));
+            break;
+        }
+        case 2:
+            *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(src);
+            break;
+        case 1:
+            *reinterpret_cast<uint16_t*>(dst) = *reinterpret_cast<const uint16_t*>(src);
+            break;
+        default:
+            *dst = *src;
+            break;
+    }
+}
+
+__device__ __forceinline__ int field_of(const IoTable& t, uint64_t w) {
+    int f = 0;
+    while (f + 1 < t.nfields && w >= t.prefix[f + 1]) ++f;
+    return f;
+}
+
+__device__ __forceinline__ void split_work(uint64_t local, uint32_t units, uint64_t& row, uint32_t& unit) {
+    if (local <= 0xffffffffull) {
+        const uint32_t l32 = (uint32_t)local;
+        const uint32_t r = l32 / units;
+        row = r;
+        unit = l32 - r * units;
+    } else {
+        row = local / units;
+        unit = (uint32_t)(local - row * units);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Ring append: rows [0, nrows) of each io matrix go to slots
+// (first_slot + row) mod capacity. Replaces P.BufferAppend
+// (mindspore_rl/core/uniform_replay_buffer.py:82,114) and the row copy of
+// PriorityReplayBufferPush (mindspore_rl/core/priority_replay_buffer.py:67-69).
+// The host guarantees nrows <= capacity, so no two rows share a slot.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kWG) void k_rows_put(IoTable t, int64_t capacity, int64_t first_slot) {
+    const uint64_t total = t.prefix[t.nfields];
+    const uint64_t stride = (uint64_t)gridDim.x * kWG;
+    for (uint64_t w = (uint64_t)blockIdx.x * kWG + threadIdx.x; w < total; w += stride) {
+        const int f = field_of(t, w);
+        uint64_t row;
+        uint32_t unit;
+        split_work(w - t.prefix[f], t.units[f], row, unit);
+        int64_t slot = first_slot + (int64_t)row;
+        if (slot >= capacity) slot -= capacity;
+        const uint32_t vl = t.vec_log2[f];
+        const uint64_t off = (uint64_t)unit << vl;
+        copy_granule(t.store[f] + (uint64_t)slot * t.row_bytes[f] + off, t.io[f] + row * t.row_bytes[f] + off, vl);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Gather: io_f[k] = store_f[slot_k]. slot_k is `fixed_slot` when that is >= 0
+// (single-row read), else comes from `indices` or, when that is NULL, from the
+// counter-based generator (uniform in [0, count), with replacement). Replaces P.BufferSample / P.BufferGetItem
+// (mindspore_rl/core/uniform_replay_buffer.py:83-89,128,139).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kWG) void k_rows_gather(IoTable t, int64_t capacity, int64_t count,
+                                                     const int64_t* __restrict__ indices, int64_t fixed_slot,
+                                                     uint64_t seed, uint64_t calls,
+                                                     int64_t* __restrict__ out_indices,
+                                                     uint32_t* __restrict__ err) {
+    const uint64_t total = t.prefix[t.nfields];
+    const uint64_t stride = (uint64_t)gridDim.x * kWG;
+    for (uint64_t w = (uint64_t)blockIdx.x * kWG + threadIdx.x; w < total; w += stride) {
+        const int f = field_of(t, w);
+        uint64_t row;
+        uint32_t unit;
+        split_work(w - t.prefix[f], t.units[f], row, unit);
+        int64_t slot = fixed_slot >= 0 ? fixed_slot : indices ? indices[row] : rng_below(seed, calls, row, count);
+        if (slot < 0 || slot >= count) {
+            if (f == 0 && unit == 0) atomicOr(err, MRB_DERR_INDEX);
+            slot = slot < 0 ? 0 : (count > 0 ? count - 1 : 0);
+            if (slot >= capacity) slot = capacity - 1;
+        }
+        if (out_indices && f == 0 && unit == 0) out_indices[row] = slot;
+        const uint32_t vl = t.vec_log2[f];
+        const uint64_t off = (uint64_t)unit << vl;
+        copy_granule(t.io[f] + row * t.row_bytes[f] + off, t.store[f] + (uint64_t)slot * t.row_bytes[f] + off, vl);
+    }
+}
+
+// Arguments common to both sample kernels.
+struct SampleArgs {
+    const float* sum;   // sum tree, heap order
+    const float* mn;    // min tree, heap order
+    int depth;          // log2(leaves)
+    int64_t leaves;
+    int64_t capacity;
+    int64_t size;
+    int64_t batch;
+    float beta;
+    const float* uniforms;  // f32[batch] or NULL -> generator
+    uint64_t seed, calls;
+    int64_t* out_idx;
+    float* out_w;
+    uint32_t* err;
+};
+
+// mass of stratum k: (u + k) * (total / batch), each operation rounded once.
+__device__ __forceinline__ float stratum_mass(const SampleArgs& a, float total, int64_t k) {
+    const float u = a.uniforms ? a.uniforms[k] : rng_uniform(a.seed, a.calls, (uint64_t)k);
+    const float seg = total / (float)a.batch;
+    return (u + (float)k) * seg;
+}
+
+// w = (p / total * size)^-beta / (pmin / total * size)^-beta
+__device__ __forceinline__ float is_weight(float p, float total, float pmin, float fsize, float beta) {
+    const float max_w = powf_det(pmin / total * fsize, -beta);
+    return powf_det(p / total * fsize, -beta) / max_w;
+}
+
+__device__ __forceinline__ void sample_flags(const SampleArgs& a, float total, int64_t idx) {
+    if (!(total > 0.0f) || total > 3.0e38f) atomicOr(a.err, MRB_DERR_TOTAL);
+    if (idx >= a.size) atomicOr(a.err, MRB_DERR_UNFILLED);
+}
+
+// ---------------------------------------------------------------------------
+// PER sample, wide rows: `split` workgroups per sampled row. Wave 0 of every
+// workgroup walks the sum tree for its stratum with descend_group (one
+// dependent load per 8 levels), publishes the slot through LDS, then the whole
+// workgroup copies its share of the row with 16-byte granules. Index and
+// importance weight are written by the row's first workgroup. Replaces
+// PriorityReplayBufferSample (mindspore_rl/core/priority_replay_buffer.py:70,92-106).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kWG) void k_per_sample_wide(IoTable t, SampleArgs a, int split) {
+    __shared__ int64_t s_idx;
+    const int64_t k = blockIdx.x / (uint32_t)split;
+    const uint32_t part = blockIdx.x % (uint32_t)split;
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const float total = a.sum[1];
+        float mass = stratum_mass(a, total, k);
+        uint32_t node = 1;
+        float picked = total;
+        int g = a.depth % kRoundLevels ? a.depth % kRoundLevels : kRoundLevels;
+        for (int d = 0; d < a.depth; d += g, g = kRoundLevels) node = descend_group(a.sum, node, g, mass, picked, lane);
+        const int64_t idx = (int64_t)node - a.leaves;
+        if (lane == 0) {
+            s_idx = idx;
+            if (part == 0) {
+                a.out_idx[k] = idx;
+                a.out_w[k] = is_weight(picked, total, a.mn[1], (float)a.size, a.beta);
+                sample_flags(a, total, idx);
+            }
+        }
+    }
+    __syncthreads();
+    int64_t slot = s_idx;
+    if (slot >= a.capacity) slot = a.capacity - 1;
+    for (int f = 0; f < t.nfields; ++f) {
+        const uint32_t units = t.units[f];
+        const uint32_t per = (units + split - 1) / split;
+        const uint32_t lo = part * per;
+        const uint32_t hi = lo + per < units ? lo + per : units;
+        const uint32_t vl = t.vec_log2[f];
+        const uint8_t* src = t.store[f] + (uint64_t)slot * t.row_bytes[f];
+        uint8_t* dst = t.io[f] + (uint64_t)k * t.row_bytes[f];
+        for (uint32_t u = lo + threadIdx.x; u < hi; u += kWG) {
+            const uint64_t off = (uint64_t)u << vl;
+            copy_granule(dst + off, src + off, vl);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// PER sample, many narrow rows: one workgroup per 256 strata. The top
+// `lds_levels` levels of the sum tree (nodes [1, 2 << lds_levels)) are staged
+// in LDS once per workgroup, so each thread's descent reads HBM/L2 only for
+// the levels below; then the workgroup gathers its 256 rows with coalesced
+// writes. Same outputs, bit for bit, as k_per_sample_wide.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kWG) void k_per_sample_lds(IoTable t, SampleArgs a, int lds_levels) {
+    extern __shared__ float s_top[];  // [2 << lds_levels] floats, then kWG int64 slots
+    const uint32_t ntop = 2u << lds_levels;
+    int64_t* s_slot = reinterpret_cast<int64_t*>(s_top + (ntop < 4 ? 4 : ntop));
+    if (ntop >= 4) {
+        for (uint32_t i = threadIdx.x * 4; i < ntop; i += kWG * 4)
+            *reinterpret_cast<float4*>(s_top + i) = *reinterpret_cast<const float4*>(a.sum + i);
+    } else if (threadIdx.x < ntop) {
+        s_top[threadIdx.x] = a.sum[threadIdx.x];
+    }
+    __syncthreads();
+    const int64_t k0 = (int64_t)blockIdx.x * kWG;
+    const int64_t k = k0 + threadIdx.x;
+    if (k < a.batch) {
+        const float total = s_top[1];
+        float mass = stratum_mass(a, total, k);
+        uint32_t node = 1;
+        int d = 0;
+        for (; d < lds_levels; ++d) {
+            const float left = s_top[2 * node];
+            if (mass <= left) {
+                node = 2 * node;
+            } else {
+                mass -= left;
+                node = 2 * node + 1;
+            }
+        }
+        for (; d < a.depth; ++d) {
+            const float left = a.sum[2 * node];
+            if (mass <= left) {
+                node = 2 * node;
+            } else {
+                mass -= left;
+                node = 2 * node + 1;
+            }
+        }
+        const float picked = a.depth <= lds_levels ? s_top[node] : a.sum[node];
+        const int64_t idx = (int64_t)node - a.leaves;
+        a.out_idx[k] = idx;
+        a.out_w[k] = is_weight(picked, total, a.mn[1], (float)a.size, a.beta);
+        sample_flags(a, total, idx);
+        s_slot[threadIdx.x] = idx < a.capacity ? idx : a.capacity - 1;
+    }
+    __syncthreads();
+    const uint32_t rows = (uint32_t)((a.batch - k0) < kWG ? (a.batch - k0) : kWG);
+    for (int f = 0; f < t.nfields; ++f) {
+        const uint32_t units = t.units[f];
+        const uint32_t vl = t.vec_log2[f];
+        const uint64_t work = (uint64_t)rows * units;
+        for (uint64_t w = threadIdx.x; w < work; w += kWG) {
+            uint64_t r;
+            uint32_t u;
+            split_work(w, units, r, u);
+            const uint64_t off = (uint64_t)u << vl;
+            copy_granule(t.io[f] + (uint64_t)(k0 + (int64_t)r) * t.row_bytes[f] + off,
+                         t.store[f] + (uint64_t)s_slot[r] * t.row_bytes[f] + off, vl);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// update_priorities, pass 1 (PriorityReplayBufferUpdate,
+// mindspore_rl/core/priority_replay_buffer.py:71-73,108-120): every valid
+// entry j raises stamp[index_j] to (epoch << 32 | j) with an integer max, so
+// after the pass the stamp names the LAST entry of this call that targets the
+// leaf (last write wins). The running max priority takes an integer max of the
+// float bits (order-preserving for non-negative floats). No float is summed
+// atomically anywhere.
+//   indices == NULL: entry j targets slot (first_slot + j) mod capacity
+//   stamp   == NULL: only the running max is updated
+// ---------------------------------------------------------------------------
+struct UpdateArgs {
+    const int64_t* indices;
+    const float* priorities;  // NULL: every entry takes the running max priority as it is
+    int64_t n;
+    int64_t capacity;
+    int64_t first_slot;
+    int64_t leaves;
+    float alpha;
+    uint32_t epoch;
+    unsigned long long* stamp;  // [leaves]
+    float* sum;
+    float* mn;
+    float* maxp;    // running max priority (device scalar)
+    uint32_t* err;
+    uint32_t* dirty[4];  // per rebuild round: one word per 256-node block
+    int nrounds;
+};
+
+__device__ __forceinline__ bool update_entry(const UpdateArgs& a, int64_t j, int64_t& idx, float& q, bool report) {
+    if (a.indices) {
+        idx = a.indices[j];
+        if (idx < 0 || idx >= a.capacity) {
+            if (report) atomicOr(a.err, MRB_DERR_INDEX);
+            return false;
+        }
+    } else {
+        idx = a.first_slot + j;
+        if (idx >= a.capacity) idx -= a.capacity;
+    }
+    const float p = a.priorities[j];
+    if (!(p >= 0.0f) || p > 3.0e38f) {
+        if (report) atomicOr(a.err, MRB_DERR_PRIORITY);
+        return false;
+    }
+    q = powf_det(p, a.alpha);
+    return true;
+}
+
+__global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
+    const int64_t j = (int64_t)blockIdx.x * kWG + threadIdx.x;
+    float q = 0.0f;
+    if (j < a.n) {
+        int64_t idx;
+        float qq;
+        if (update_entry(a, j, idx, qq, true)) {
+            q = qq;
+            if (a.stamp) atomicMax(&a.stamp[idx], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
+        }
+    }
+    // wave max, then one integer atomic per wave
+    for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+    if ((threadIdx.x & 63) == 0 && q > 0.0f) atomicMax(reinterpret_cast<unsigned int*>(a.maxp), __float_as_uint(q));
+}
+
+__device__ __forceinline__ void mark_dirty(const UpdateArgs& a, int64_t idx) {
+    for (int r = 0; r < a.nrounds; ++r) a.dirty[r][idx >> (kRoundLevels * (r + 1))] = a.epoch;
+}
+
+// Pass 2: the winning entry of each leaf writes it (sum and min trees) and
+// marks the 256-node blocks above it dirty for the rebuild rounds.
+//   indices given:            winner = entry named by the stamp
+//   indices NULL, priorities: slots are distinct, every entry writes
+//   indices NULL, no priorities: every slot takes the running max priority
+__global__ __launch_bounds__(kWG) void k_update_leaves(UpdateArgs a) {
+    const int64_t j = (int64_t)blockIdx.x * kWG + threadIdx.x;
+    if (j >= a.n) return;
+    int64_t idx;
+    float q;
+    if (a.priorities && a.indices) {
+        if (!update_entry(a, j, idx, q, false)) return;
+        if (a.stamp[idx] != (((unsigned long long)a.epoch << 32) | (unsigned long long)j)) return;
+    } else if (a.priorities) {
+        // freshly pushed slot: an invalid priority leaves it at the running max, as a plain push would
+        if (!update_entry(a, j, idx, q, false)) q = *a.maxp;
+    } else {
+        idx = a.first_slot + j;
+        if (idx >= a.capacity) idx -= a.capacity;
+        q = *a.maxp;
+    }
+    a.sum[a.leaves + idx] = q;
+    a.mn[a.leaves + idx] = q;
+    mark_dirty(a, idx);
+}
+
+// ---------------------------------------------------------------------------
+// Rebuild round: one wave per block of 256 consecutive nodes at depth
+// `lo_depth`. A block whose dirty word carries this call's epoch recomputes
+// the 8 levels above it from those 256 nodes (float4 per lane, then wave
+// shuffles), each parent as the single rounded sum / min of its two children
+// — the same operation, on the same operands, as a leaf-to-root walk performs.
+// Recomputing a clean node reproduces its bits, so only values that a
+// sequential update would have changed change.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kWG) void k_tree_round(float* __restrict__ sum, float* __restrict__ mn, int lo_depth,
+                                                    const uint32_t* __restrict__ dirty, uint32_t epoch) {
+    const uint32_t block = blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
+    const uint32_t nblocks = (1u << lo_depth) / kBlockNodes;
+    if (block >= nblocks) return;
+    if (dirty[block] != epoch) return;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t first = (1u << lo_depth) + block * kBlockNodes;  // heap index of the block's first node
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        float* tree = which ? mn : sum;
+        const float4 v = *reinterpret_cast<const float4*>(tree + first + 4 * lane);
+        float a0, a1, c;
+        if (which) {
+            a0 = fminf(v.x, v.y);
+            a1 = fminf(v.z, v.w);
+            c = fminf(a0, a1);
+        } else {
+            a0 = v.x + v.y;
+            a1 = v.z + v.w;
+            c = a0 + a1;
+        }
+        // level lo_depth-1: 128 nodes, two per lane; level lo_depth-2: 64 nodes, one per lane
+        *reinterpret_cast<float2*>(tree + (first >> 1) + 2 * lane) = make_float2(a0, a1);
+        tree[(first >> 2) + lane] = c;
+        // levels lo_depth-3 .. lo_depth-8: 32, 16, 8, 4, 2, 1 nodes
+#pragma unroll
+        for (int s = 0; s < 6; ++s) {
+            const float o = __shfl_xor(c, 1 << s);
+            c = which ? fminf(c, o) : c + o;
+            if ((lane & ((2u << s) - 1)) == 0) tree[(first >> (3 + s)) + (lane >> (s + 1))] = c;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Top of the tree: one workgroup loads the 2^top_depth (<= 4096) nodes at
+// depth `top_depth` into LDS, rebuilds every level above them and writes
+// nodes [1, 2^top_depth) back.
+// ---------------------------------------------------------------------------
+constexpr int kTopWG = 1024;
+__global__ __launch_bounds__(kTopWG) void k_tree_top(float* __restrict__ sum, float* __restrict__ mn, int top_depth) {
+    __shared__ float s_sum[2 << kTopMaxDepth];
+    __shared__ float s_min[2 << kTopMaxDepth];
+    const uint32_t n = 1u << top_depth;
+    for (uint32_t i = n + threadIdx.x; i < 2 * n; i += kTopWG) {
+        s_sum[i] = sum[i];
+        s_min[i] = mn[i];
+    }
+    __syncthreads();
+    for (int d = top_depth - 1; d >= 0; --d) {
+        const uint32_t lo = 1u << d;
+        for (uint32_t i = lo + threadIdx.x; i < 2 * lo; i += kTopWG) {
+            s_sum[i] = s_sum[2 * i] + s_sum[2 * i + 1];
+            s_min[i] = fminf(s_min[2 * i], s_min[2 * i + 1]);
+        }
+        __syncthreads();
+    }
+    for (uint32_t i = 1 + threadIdx.x; i < n; i += kTopWG) {
+        sum[i] = s_sum[i];
+        mn[i] = s_min[i];
+    }
+}
+
+// Fills a float array with one value (tree initialisation: sums 0, mins FLT_MAX).
+__global__ __launch_bounds__(kWG) void k_fill_f32(float* p, float v, uint64_t n) {
+    const uint64_t stride = (uint64_t)gridDim.x * kWG;
+    for (uint64_t i = (uint64_t)blockIdx.x * kWG + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+
+}  // namespace mrb

@@ -1,0 +1,251 @@
+"""ctypes binding of the CPU oracle (oracle/mrb_oracle.c).
+
+Test infrastructure: imported only by tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py. Works on numpy arrays in host memory.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libmrb_oracle.so")
+
+
+def build(force=False):
+    """Compile the oracle with gcc (see oracle/Makefile)."""
+    if force and os.path.exists(_SO):
+        os.remove(_SO)
+    subprocess.run(["make", "-s", "-C", _HERE], check=True)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_SO):
+        build()
+    L = C.CDLL(_SO)
+    vp, i64, u64, f32 = C.c_void_p, C.c_int64, C.c_uint64, C.c_float
+    pvp = C.POINTER(C.c_void_p)
+    sig = {
+        "orc_powf": (f32, [f32, f32]),
+        "orc_powf_n": (None, [vp, f32, vp, i64]),
+        "orc_rng_u64": (u64, [u64, u64, u64]),
+        "orc_rng_uniform": (f32, [u64, u64, u64]),
+        "orc_rng_below": (i64, [u64, u64, u64, i64]),
+        "orc_urb_create": (vp, [i64, C.c_int, vp]),
+        "orc_urb_destroy": (None, [vp]),
+        "orc_urb_seed": (None, [vp, u64]),
+        "orc_urb_append": (C.c_int, [vp, pvp, i64]),
+        "orc_urb_get_item": (C.c_int, [vp, i64, pvp]),
+        "orc_urb_gather": (C.c_int, [vp, vp, i64, pvp]),
+        "orc_urb_sample": (C.c_int, [vp, i64, vp, pvp]),
+        "orc_urb_reset": (None, [vp]),
+        "orc_urb_count": (i64, [vp]),
+        "orc_urb_head": (i64, [vp]),
+        "orc_urb_field": (vp, [vp, C.c_int]),
+        "orc_per_create": (vp, [i64, f32, C.c_int, vp, u64]),
+        "orc_per_destroy": (None, [vp]),
+        "orc_per_update": (C.c_int, [vp, vp, vp, i64]),
+        "orc_per_push": (C.c_int, [vp, pvp, i64, vp]),
+        "orc_per_sample": (C.c_int, [vp, i64, f32, vp, vp, vp, pvp]),
+        "orc_per_export_tree": (None, [vp, vp, vp]),
+        "orc_per_leaves": (i64, [vp]),
+        "orc_per_size": (i64, [vp]),
+        "orc_per_head": (i64, [vp]),
+        "orc_per_max_priority": (f32, [vp]),
+        "orc_per_field": (vp, [vp, C.c_int]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = L
+    return L
+
+
+def powf(x, a):
+    return lib().orc_powf(float(np.float32(x)), float(np.float32(a)))
+
+
+def powf_array(x, a):
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty_like(x)
+    lib().orc_powf_n(x.ctypes.data, float(np.float32(a)), out.ctypes.data, x.size)
+    return out
+
+
+def rng_uniform(seed, counter, n):
+    L = lib()
+    return np.array([L.orc_rng_uniform(seed, counter, k) for k in range(n)], np.float32)
+
+
+def _field_bytes(shapes, dtypes):
+    return [int(np.prod(s, dtype=np.int64)) * np.dtype(d).itemsize for s, d in zip(shapes, dtypes)]
+
+
+def _ptr_array(arrays):
+    arr = (C.c_void_p * len(arrays))()
+    for i, a in enumerate(arrays):
+        arr[i] = a.ctypes.data
+    return arr
+
+
+class _Rows:
+    def __init__(self, shapes, dtypes):
+        self.shapes = [tuple(int(v) for v in s) for s in shapes]
+        self.dtypes = [np.dtype(d) for d in dtypes]
+        self.bytes = _field_bytes(self.shapes, self.dtypes)
+        self._fb = (C.c_int64 * len(self.bytes))(*self.bytes)
+
+    def _src(self, fields, nrows):
+        keep = []
+        for f, s, d in zip(fields, self.shapes, self.dtypes):
+            a = np.ascontiguousarray(np.asarray(f, dtype=d).reshape((nrows,) + s))
+            keep.append(a)
+        return keep
+
+    def _dst(self, n):
+        if n is None:
+            return [np.empty(s, d) for s, d in zip(self.shapes, self.dtypes)]
+        return [np.empty((n,) + s, d) for s, d in zip(self.shapes, self.dtypes)]
+
+
+class OracleUniform(_Rows):
+    """CPU twin of UniformReplayBuffer (mindspore_rl/core/uniform_replay_buffer.py:50-172)."""
+
+    def __init__(self, capacity, shapes, dtypes, seed=0):
+        super().__init__(shapes, dtypes)
+        self.capacity = int(capacity)
+        self.h = lib().orc_urb_create(self.capacity, len(self.bytes), self._fb)
+        if not self.h:
+            raise ValueError("orc_urb_create failed")
+        lib().orc_urb_seed(self.h, seed)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_urb_destroy(self.h)
+            self.h = None
+
+    def append(self, fields, nrows):
+        src = self._src(fields, nrows)
+        if lib().orc_urb_append(self.h, _ptr_array(src), nrows):
+            raise ValueError("orc_urb_append failed")
+
+    def get_item(self, index):
+        dst = self._dst(None)
+        if lib().orc_urb_get_item(self.h, int(index), _ptr_array(dst)):
+            raise IndexError(index)
+        return dst
+
+    def gather(self, indices):
+        idx = np.ascontiguousarray(indices, np.int64)
+        dst = self._dst(idx.size)
+        if lib().orc_urb_gather(self.h, idx.ctypes.data, idx.size, _ptr_array(dst)):
+            raise IndexError("orc_urb_gather: index out of range")
+        return dst
+
+    def sample(self, n):
+        idx = np.empty(n, np.int64)
+        dst = self._dst(n)
+        if lib().orc_urb_sample(self.h, n, idx.ctypes.data, _ptr_array(dst)):
+            raise ValueError("orc_urb_sample failed")
+        return idx, dst
+
+    def reset(self):
+        lib().orc_urb_reset(self.h)
+
+    @property
+    def count(self):
+        return lib().orc_urb_count(self.h)
+
+    @property
+    def head(self):
+        return lib().orc_urb_head(self.h)
+
+    def field(self, i):
+        n = self.capacity * self.bytes[i]
+        raw = (C.c_ubyte * n).from_address(lib().orc_urb_field(self.h, i))
+        return np.frombuffer(raw, np.uint8).view(self.dtypes[i]).reshape((self.capacity,) + self.shapes[i]).copy()
+
+
+class OraclePER(_Rows):
+    """CPU twin of PriorityReplayBuffer (mindspore_rl/core/priority_replay_buffer.py:30-138)."""
+
+    def __init__(self, alpha, capacity, shapes, dtypes, seed=0):
+        super().__init__(shapes, dtypes)
+        self.capacity = int(capacity)
+        self.h = lib().orc_per_create(self.capacity, float(alpha), len(self.bytes), self._fb, seed)
+        if not self.h:
+            raise ValueError("orc_per_create failed")
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_per_destroy(self.h)
+            self.h = None
+
+    def push(self, fields, nrows, priorities=None):
+        src = self._src(fields, nrows)
+        pr = None
+        if priorities is not None:
+            pr = np.ascontiguousarray(priorities, np.float32)
+            assert pr.size == nrows
+        rc = lib().orc_per_push(self.h, _ptr_array(src), nrows, pr.ctypes.data if pr is not None else None)
+        if rc:
+            raise ValueError("orc_per_push failed rc=%d" % rc)
+
+    def update(self, indices, priorities):
+        idx = np.ascontiguousarray(indices, np.int64)
+        pr = np.ascontiguousarray(priorities, np.float32)
+        assert idx.size == pr.size
+        rc = lib().orc_per_update(self.h, idx.ctypes.data, pr.ctypes.data, idx.size)
+        if rc:
+            raise ValueError("orc_per_update failed rc=%d" % rc)
+
+    def sample(self, batch, beta, uniforms=None, gather=True):
+        idx = np.empty(batch, np.int64)
+        w = np.empty(batch, np.float32)
+        dst = self._dst(batch) if gather else None
+        u = None
+        if uniforms is not None:
+            u = np.ascontiguousarray(uniforms, np.float32)
+            assert u.size == batch
+        rc = lib().orc_per_sample(self.h, batch, float(beta), u.ctypes.data if u is not None else None,
+                                  idx.ctypes.data, w.ctypes.data, _ptr_array(dst) if gather else None)
+        if rc:
+            raise ValueError("orc_per_sample failed rc=%d" % rc)
+        return idx, w, dst
+
+    def export_tree(self):
+        n = 2 * self.leaves
+        s = np.empty(n, np.float32)
+        m = np.empty(n, np.float32)
+        lib().orc_per_export_tree(self.h, s.ctypes.data, m.ctypes.data)
+        return s, m
+
+    @property
+    def leaves(self):
+        return lib().orc_per_leaves(self.h)
+
+    @property
+    def size(self):
+        return lib().orc_per_size(self.h)
+
+    @property
+    def head(self):
+        return lib().orc_per_head(self.h)
+
+    @property
+    def max_priority(self):
+        return lib().orc_per_max_priority(self.h)
+
+    def field(self, i):
+        n = self.capacity * self.bytes[i]
+        raw = (C.c_ubyte * n).from_address(lib().orc_per_field(self.h, i))
+        return np.frombuffer(raw, np.uint8).view(self.dtypes[i]).reshape((self.capacity,) + self.shapes[i]).copy()

@@ -1,0 +1,370 @@
+"""GPU parity: the HIP library (through ctypes and the C ABI) against the CPU
+oracle on identical seeded inputs. Bar: indices, gathered rows, ring contents
+and both trees bit-exact; importance weights within 1e-6 relative (fp32)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import (assert_sample_equal, assert_tree_equal, bits, random_rows, t2n, to_dev, torch_types)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mrb():
+    if not torch.cuda.is_available():
+        pytest.fail("no HIP device: the GPU parity tests cannot run (there is no CPU fallback)")
+    from mindrl_amd import _lib
+    from mindrl_amd.core import PriorityReplayBuffer, UniformReplayBuffer
+    _lib.lib()
+
+    class NS:
+        pass
+
+    ns = NS()
+    ns.lib, ns.PER, ns.URB = _lib, PriorityReplayBuffer, UniformReplayBuffer
+    yield ns
+    _lib.set_option("sample_path", 0)
+    _lib.set_option("row_split", 0)
+    _lib.set_option("lds_levels", 0)
+
+
+# ------------------------------------------------------------------ uniform
+URB_LAYOUTS = [
+    ([(4,), (1,), (1,), (4,), (1,)], [np.float32, np.int32, np.float32, np.float32, np.bool_]),   # 41 B row
+    ([(17,), (6,), (1,), (17,), (1,)], [np.float32, np.float32, np.float32, np.float32, np.bool_]),  # 165 B row
+    ([(3, 5), (2,), (7,)], [np.float16, np.int64, np.uint8]),
+    ([(64,), (1,)], [np.float32, np.int16]),
+]
+
+
+@pytest.mark.parametrize("layout", range(len(URB_LAYOUTS)))
+@pytest.mark.parametrize("cap", [1, 7, 64, 1000])
+def test_uniform_ring_random_ops(mrb, orc, layout, cap):
+    shapes, dtypes = URB_LAYOUTS[layout]
+    rng = np.random.default_rng(100 * layout + cap)
+    g = mrb.URB(8, cap, shapes, torch_types(dtypes), seed=77)
+    c = orc.OracleUniform(cap, shapes, dtypes, seed=77)
+    for step in range(25):
+        n = int(rng.integers(1, 2 * cap + 3)) if step % 5 else 1
+        rows = random_rows(rng, n, shapes, dtypes)
+        if n == 1 and step % 2:
+            g.insert([torch.from_numpy(r[0]).cuda() for r in rows])  # single element, shape_i
+        else:
+            g.insert(to_dev(rows))
+        c.append(rows, n)
+        assert int(g.count) == c.count and int(g.head) == c.head
+        assert int(g.size()) == c.count and bool(g.full()[0]) == (c.count >= cap)
+        for f in range(len(shapes)):  # raw storage, slot by slot
+            assert np.array_equal(t2n(g.buffer[f]).view(np.uint8), c.field(f).view(np.uint8)), (step, f)
+        j = int(rng.integers(-c.count, c.count))
+        for a, b in zip(g.get_item(j), c.get_item(j)):
+            assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+        idx = rng.integers(0, c.count, 33)
+        for a, b in zip(g.sample(indices=torch.from_numpy(idx).cuda()), c.gather(idx)):
+            assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+        if c.count >= 8:
+            gi, gf = g.sample_with_indices()
+            ci, cf = c.sample(8)
+            assert np.array_equal(t2n(gi), ci)
+            for a, b in zip(gf, cf):
+                assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+        if step == 12:
+            g.reset()
+            c.reset()
+    g.check()
+    g.destroy()
+
+
+def test_uniform_successive_samples_differ_and_errors(mrb):
+    g = mrb.URB(32, 200, [(1,)], [torch.int32], seed=5)
+    with pytest.raises(ValueError):
+        g.sample()  # batch > count (empty)
+    g.insert([torch.arange(200, dtype=torch.int32).reshape(200, 1).cuda()])
+    a = t2n(g.sample()[0])
+    b = t2n(g.sample()[0])
+    assert not np.array_equal(a, b) and a.min() >= 0 and a.max() < 200  # rows hold their own slot number
+    with pytest.raises(ValueError):
+        g.get_item(200)
+    g.sample(indices=torch.tensor([0, 500, -3]).cuda())
+    with pytest.raises(IndexError):
+        g.check()
+    g.check()  # flags cleared by the failing check
+    g.destroy()
+    with pytest.raises(ValueError):
+        g._state()  # destroyed handle
+    with pytest.raises(ValueError):
+        mrb.URB(1, 0, [(1,)], [torch.int32])
+
+
+# ---------------------------------------------------------------------- PER
+PER_SHAPES = [(3,), (1,)]
+PER_DTYPES = [np.float32, np.int32]
+
+
+def id_rows(n, start=0):
+    ids = np.arange(start, start + n)
+    return [np.repeat(ids[:, None], 3, 1).astype(np.float32), ids.astype(np.int32)[:, None]]
+
+
+def make_pair(mrb, orc, alpha, cap, batch, seed=9, shapes=PER_SHAPES, dtypes=PER_DTYPES):
+    g = mrb.PER(alpha, cap, batch, shapes, torch_types(dtypes), seed0=seed)
+    c = orc.OraclePER(alpha, cap, shapes, dtypes, seed=seed)
+    return g, c
+
+
+@pytest.mark.parametrize("path", [1, 2])
+@pytest.mark.parametrize("cap", [1, 2, 5, 100, 200, 4096, 5000, 10000, 70000])
+def test_per_random_ops_bit_exact(mrb, orc, cap, path):
+    """Random pushes (plain / with priorities / larger than capacity), updates with
+    duplicates and samples; after every step both trees, indices, rows, size, head and
+    running max are compared. Capacities cover tree depths 0..17, i.e. the top kernel
+    alone (<= 4096 leaves) and one rebuild round."""
+    mrb.lib.set_option("sample_path", path)
+    rng = np.random.default_rng(cap + path)
+    batch = 32
+    g, c = make_pair(mrb, orc, 0.6, cap, batch)
+    serial, exact_w = 0, 0
+    for step in range(12):
+        n = int(rng.integers(1, min(2 * cap + 3, 3000)))
+        rows = id_rows(n, serial)
+        serial += n
+        if step % 3 == 2:
+            pr = (np.abs(rng.normal(size=n)) + 1e-6).astype(np.float32)
+            g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda())
+            c.push(rows, n, pr)
+        else:
+            g.insert(*to_dev(rows))
+            c.push(rows, n)
+        k = int(rng.integers(1, min(2 * cap + 2, 2500)))
+        idx = rng.integers(0, cap, k)
+        pr = rng.pareto(1.5, k).astype(np.float32) + np.float32(1e-6)
+        g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda())
+        c.update(idx, pr)
+        assert_tree_equal(g, c, "cap %d step %d" % (cap, step))
+        assert g.size() == c.size and g._state()[1] == c.head
+        assert np.float32(g.max_priority) == np.float32(c.max_priority)
+        u = rng.random(batch).astype(np.float32)
+        beta = float(rng.uniform(0, 1))
+        exact_w += assert_sample_equal(g.sample(beta, uniforms=torch.from_numpy(u).cuda()), c.sample(batch, beta, u),
+                                       "cap %d step %d" % (cap, step))
+        # generator-driven draw: both sides advance the same counter-based stream
+        exact_w += assert_sample_equal(g.sample(beta), c.sample(batch, beta), "cap %d step %d rng" % (cap, step))
+        for f, (a, b) in enumerate(zip(g.storage(), [c.field(0), c.field(1)])):
+            assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8)), (step, f)
+    assert g.check() in (0, 8)
+    assert exact_w == 24, "importance weights not bit-identical in %d of 24 draws" % (24 - exact_w)
+    g.destroy()
+
+
+@pytest.mark.parametrize("alpha", [0.0, 0.4, 0.6, 1.0, 1.7])
+def test_device_powf_bit_exact(mrb, orc, alpha):
+    """priorities ** alpha computed on the device equals the oracle's deterministic powf bit for bit."""
+    n = 1 << 16
+    rng = np.random.default_rng(int(alpha * 10))
+    pr = np.exp(rng.uniform(-60, 40, n)).astype(np.float32)
+    pr[:8] = [0.0, 1.0, 1e-38, 1e-45, 3e38, 2.0, 0.5, 1e-7]
+    g = mrb.PER(alpha, n, 4, [(1,)], [torch.int32], seed0=1)
+    g.insert(torch.zeros(n, 1, dtype=torch.int32).cuda())
+    g.update_priorities(torch.arange(n).cuda(), torch.from_numpy(pr).cuda())
+    s, _ = g.export_tree()
+    want = orc.powf_array(pr, alpha)
+    bad = np.nonzero(bits(s[n:]) != bits(want))[0]
+    assert bad.size == 0, (pr[bad[:5]], s[n:][bad[:5]], want[bad[:5]])
+    g.destroy()
+
+
+def test_reference_scenario(mrb):
+    """tests/st/test_priority_replay_buffer.py:34-66 on the HIP buffer, through the
+    method names that test uses (push / sample / update_priorities)."""
+    capacity, batch_size = 200, 32
+    prb = mrb.PER(1., capacity, batch_size, ((17,), (6,)), (torch.float32, torch.int32), seed0=0, seed1=42)
+    for i in range(100):
+        prb.push(torch.ones(17) * i, (torch.ones(6) * i).to(torch.int32))
+    indices, weights, states, actions = prb.sample(1.)
+    ind = t2n(indices)
+    assert np.all(ind < 100) and weights.shape == (32,) and weights.dtype == torch.float32
+    assert np.allclose(t2n(states), np.broadcast_to(ind.reshape(-1, 1), states.shape))
+    assert np.allclose(t2n(actions), np.broadcast_to(ind.reshape(-1, 1), actions.shape))
+    prb.update_priorities(indices, torch.ones(32) * 1e-7)
+    indices_new, _, states_new, actions_new = prb.sample(1.)
+    ind2 = t2n(indices_new)
+    assert np.all(ind2 < 100) and np.all(ind != ind2)
+    assert np.allclose(t2n(states_new), np.broadcast_to(ind2.reshape(-1, 1), states_new.shape))
+    assert np.allclose(t2n(actions_new), np.broadcast_to(ind2.reshape(-1, 1), actions_new.shape))
+    assert bool(prb.full()) is False
+    with pytest.raises(ValueError):
+        prb.reset()
+    h = prb.destroy()
+    assert h.dtype == torch.int64 and tuple(h.shape) == (1,)
+
+
+def test_per_error_paths(mrb):
+    L = mrb.lib.lib()
+    assert L.mrb_backend() == 1
+    g = mrb.PER(0.6, 16, 4, [(1,)], [torch.int32], seed0=3)
+    with pytest.raises(ValueError):
+        g.sample(0.4)  # empty
+    g.insert(torch.zeros(16, 1, dtype=torch.int32).cuda())
+    g.update_priorities(torch.tensor([3, 99, -1]).cuda(), torch.tensor([2.0, 1.0, 1.0]).cuda())
+    with pytest.raises(IndexError):
+        g.check()
+    g.update_priorities(torch.tensor([3, 4, 5]).cuda(), torch.tensor([-2.0, float("nan"), float("inf")]).cuda())
+    with pytest.raises(ValueError):
+        g.check()
+    s, _ = g.export_tree()
+    assert abs(s[16 + 3] - 2.0 ** 0.6) < 1e-6
+    assert s[16 + 4] == 1.0 and s[16 + 5] == 1.0  # invalid entries skipped
+    assert L.mrb_per_update(C.c_int64(987654), None, None, 1, None) == mrb.lib.MRB_EHANDLE
+    assert L.mrb_per_update(C.c_int64(g._h), None, None, 1, None) == mrb.lib.MRB_EINVAL
+    assert b"NULL" in L.mrb_last_error()
+    g.destroy()
+    with pytest.raises(ValueError):
+        g.size()
+    with pytest.raises(ValueError):
+        mrb.PER(0.6, -5, 4, [(1,)], [torch.int32])
+
+
+# ------------------------------------------------- BASELINE.json configurations
+def test_config1_dqn_per_cartpole_full_loop(mrb, orc):
+    """Config 1: capacity 10 000, alpha .6, beta .4, eps 1e-6; fill, then 1000 x
+    {sample 64, update with |N(0,1)|+eps, insert 1}. Every step compared."""
+    shapes = [(4,), (1,), (1,), (4,), (1,)]
+    dtypes = [np.float32, np.int32, np.float32, np.float32, np.bool_]
+    rng = np.random.default_rng(1001)
+    cap, batch = 10_000, 64
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=1001, shapes=shapes, dtypes=dtypes)
+
+    def transitions(n):
+        return [rng.uniform(-2.4, 2.4, (n, 4)).astype(np.float32), rng.integers(0, 2, (n, 1)).astype(np.int32),
+                np.ones((n, 1), np.float32), rng.uniform(-2.4, 2.4, (n, 4)).astype(np.float32),
+                rng.random((n, 1)) < 0.05]
+
+    rows = transitions(cap)
+    g.insert(*to_dev(rows))
+    c.push(rows, cap)
+    exact = 0
+    for step in range(1000):
+        u = rng.random(batch).astype(np.float32)
+        out = g.sample(0.4, uniforms=torch.from_numpy(u).cuda())
+        ref = c.sample(batch, 0.4, u)
+        exact += assert_sample_equal(out, ref, "step %d" % step)
+        td = (np.abs(rng.normal(size=batch)) + 1e-6).astype(np.float32)
+        g.update_priorities(out[0], torch.from_numpy(td).cuda())
+        c.update(ref[0], td)
+        one = transitions(1)
+        g.insert(*[torch.from_numpy(r[0]).cuda() for r in one])
+        c.push(one, 1)
+        if step % 50 == 0 or step == 999:
+            assert_tree_equal(g, c, "step %d" % step)
+    assert exact == 1000
+    assert g.check() == 0
+    g.destroy()
+
+
+def test_config4_apex_high_churn(mrb, orc):
+    """Config 4 at its real shape: capacity 2^21, 521-byte rows, per step insert 4096
+    with actor priorities, update 2048 (~10% duplicates, Pareto(1.5)), sample 1024."""
+    shapes = [(64,), (1,), (1,), (64,), (1,)]
+    dtypes = [np.float32, np.int32, np.float32, np.float32, np.bool_]
+    rng = np.random.default_rng(1004)
+    cap, batch = 1 << 21, 1024
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=1004, shapes=shapes, dtypes=dtypes)
+    for step in range(6):
+        n = 4096 if step else 65536
+        rows = random_rows(rng, n, shapes, dtypes)
+        pr = (np.abs(rng.normal(size=n)) + 1e-6).astype(np.float32)
+        g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda())
+        c.push(rows, n, pr)
+        idx = rng.integers(0, c.size, 2048)
+        idx[rng.integers(0, 2048, 205)] = idx[rng.integers(0, 2048, 205)]
+        up = rng.pareto(1.5, 2048).astype(np.float32) + np.float32(1e-6)
+        g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(up).cuda())
+        c.update(idx, up)
+        u = rng.random(batch).astype(np.float32)
+        for path in (1, 2):
+            mrb.lib.set_option("sample_path", path)
+            assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(batch, 0.5, u),
+                                "step %d path %d" % (step, path))
+        mrb.lib.set_option("sample_path", 0)
+    assert_tree_equal(g, c, "config 4")
+    assert g.check() == 0
+    g.destroy()
+
+
+def test_config5_tree_descent_stress(mrb, orc):
+    """Config 5 at full size: 2^24 leaves, 8-byte rows, heavy-tailed priorities,
+    batch 65 536 stratified, update 65 536 random indices per step."""
+    shapes, dtypes = [(1,), (1,)], [np.int32, np.float32]
+    rng = np.random.default_rng(1005)
+    cap, batch = 1 << 24, 65536
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=1005, shapes=shapes, dtypes=dtypes)
+    rows = [np.arange(cap, dtype=np.int32)[:, None], rng.normal(size=(cap, 1)).astype(np.float32)]
+    pr = np.where(rng.random(cap) < 0.99, rng.uniform(0, 1e-3, cap), rng.uniform(1, 100, cap)).astype(np.float32)
+    g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda())
+    c.push(rows, cap)
+    c.update(np.arange(cap), pr)
+    for step in range(3):
+        idx = rng.integers(0, cap, batch)
+        up = np.where(rng.random(batch) < 0.99, rng.uniform(0, 1e-3, batch), rng.uniform(1, 100, batch)).astype(np.float32)
+        g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(up).cuda())
+        c.update(idx, up)
+        u = rng.random(batch).astype(np.float32)
+        for path in (2, 1):
+            mrb.lib.set_option("sample_path", path)
+            out = g.sample(0.7, uniforms=torch.from_numpy(u).cuda())
+            assert_sample_equal(out, c.sample(batch, 0.7, u), "step %d path %d" % (step, path))
+            assert np.array_equal(t2n(out[2])[:, 0], t2n(out[0]))  # row k holds its own slot number
+        mrb.lib.set_option("sample_path", 0)
+    assert_tree_equal(g, c, "config 5")
+    assert g.check() == 0
+    g.destroy()
+
+
+def test_config3_atari_shape_properties(mrb, orc):
+    """Config 3's row shape (u8[84,84,4] + next_idx i64 + action i32 + reward f32 + done
+    bool = 28 241 stored bytes) at capacity 2^17 (3.7 GB) instead of 10^6: the tree logic
+    does not depend on row content, so indices/weights/trees are compared with an oracle
+    holding only the four small fields, and the image field is checked against torch's own
+    index_select of the storage."""
+    shapes = [(84, 84, 4), (1,), (1,), (1,), (1,)]
+    dtypes = [np.uint8, np.int64, np.int32, np.float32, np.bool_]
+    rng = np.random.default_rng(1003)
+    cap, batch = 1 << 17, 512
+    g = mrb.PER(0.6, cap, batch, shapes, torch_types(dtypes), seed0=1003)
+    c = orc.OraclePER(0.6, cap, shapes[1:], dtypes[1:], seed=1003)
+    gen = torch.Generator(device="cuda").manual_seed(1003)
+    chunk = 4096
+    for start in range(0, cap, chunk):
+        small = [np.arange(start + 1, start + chunk + 1, dtype=np.int64)[:, None] % cap,
+                 rng.integers(0, 18, (chunk, 1)).astype(np.int32),
+                 rng.integers(-1, 2, (chunk, 1)).astype(np.float32), rng.random((chunk, 1)) < 0.01]
+        obs = torch.randint(0, 256, (chunk, 84, 84, 4), dtype=torch.uint8, device="cuda", generator=gen)
+        g.insert(obs, *to_dev(small))
+        c.push(small, chunk)
+    pr = rng.lognormal(0, 1, cap).astype(np.float32)
+    g.update_priorities(torch.arange(cap).cuda(), torch.from_numpy(pr).cuda())
+    c.update(np.arange(cap), pr)
+    store = g.storage()
+    for step in range(8):
+        beta = 0.4 + 0.6 * step / 7
+        u = rng.random(batch).astype(np.float32)
+        out = g.sample(beta, uniforms=torch.from_numpy(u).cuda())
+        ci, cw, cf = c.sample(batch, beta, u)
+        assert_sample_equal((out[0], out[1]) + tuple(out[3:]), (ci, cw, cf), "step %d" % step)
+        assert torch.equal(out[2], store[0].index_select(0, out[0]))
+        td = (np.abs(rng.normal(size=batch)) + 1e-6).astype(np.float32)
+        g.update_priorities(out[0], torch.from_numpy(td).cuda())
+        c.update(ci, td)
+        four = [np.arange(4, dtype=np.int64)[:, None], rng.integers(0, 18, (4, 1)).astype(np.int32),
+                rng.integers(-1, 2, (4, 1)).astype(np.float32), rng.random((4, 1)) < 0.01]
+        obs4 = torch.randint(0, 256, (4, 84, 84, 4), dtype=torch.uint8, device="cuda", generator=gen)
+        head = g._state()[1]
+        g.insert(obs4, *to_dev(four))
+        c.push(four, 4)
+        assert torch.equal(store[0][head:head + 4], obs4)
+    assert_tree_equal(g, c, "config 3 shape")
+    assert g.check() == 0
+    g.destroy()

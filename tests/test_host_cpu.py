@@ -1,0 +1,82 @@
+"""CPU-only checks of the product's host side: the C-ABI library loads and
+exports every symbol include/mrb.h declares, argument validation that needs no
+device, and the Python-side layout logic. No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from mindrl_amd import _lib
+from mindrl_amd.core._rows import FieldLayout
+from mindrl_amd.dtype import as_torch_dtype
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mrb.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mrb_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_symbols()
+    assert len(names) == 24
+    L = _lib.lib()
+    for n in names:
+        assert hasattr(L, n), "libmrb.so does not export %s" % n
+    assert set(_lib.SIGNATURES) | {"mrb_last_error"} == set(names)
+    assert L.mrb_backend() == 1 and L.mrb_version() == 1
+
+
+def test_status_codes_without_a_device():
+    L = _lib.lib()
+    assert L.mrb_urb_state(123456, None, None) == _lib.MRB_EHANDLE
+    assert b"123456" in L.mrb_last_error()
+    assert L.mrb_per_destroy(42) == _lib.MRB_EHANDLE
+    assert L.mrb_set_option(b"no_such_option", 1) == _lib.MRB_EINVAL
+    assert L.mrb_set_option(b"row_split", 1000) == _lib.MRB_EINVAL
+    assert L.mrb_set_option(b"row_split", 0) == _lib.MRB_OK
+    h = C.c_int64(0)
+    fb = (C.c_int64 * 1)(4)
+    assert L.mrb_urb_create(0, 1, fb, C.byref(h)) == _lib.MRB_EINVAL
+    assert L.mrb_urb_create(10, 0, fb, C.byref(h)) == _lib.MRB_EINVAL
+    assert L.mrb_urb_create(10, 17, fb, C.byref(h)) == _lib.MRB_EINVAL
+    assert L.mrb_per_create(10, C.c_float(-1.0), 1, fb, 0, C.byref(h)) == _lib.MRB_EINVAL
+    with pytest.raises(ValueError):
+        _lib.check(_lib.MRB_EINVAL)
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-device failure mode")
+def test_buffers_fail_loudly_without_a_device():
+    from mindrl_amd.core import PriorityReplayBuffer, UniformReplayBuffer
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        UniformReplayBuffer(4, 10, [(1,)], [torch.float32])
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        PriorityReplayBuffer(0.6, 10, 4, [(1,)], [torch.float32])
+
+
+def test_missing_library_is_an_error(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmrb.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.lib()
+
+
+def test_field_layout():
+    lay = FieldLayout([(84, 84, 4), (1,), 1, (1,), (1,)], [np.uint8, "int64", torch.int32, "mindspore.float32", bool])
+    assert lay.bytes == [28224, 8, 4, 4, 1] and sum(lay.bytes) == 28241
+    assert lay.dtypes == [torch.uint8, torch.int64, torch.int32, torch.float32, torch.bool]
+    assert lay.batch_of([torch.zeros(84, 84, 4), torch.zeros(1), torch.zeros(1), torch.zeros(1), torch.zeros(1)]) == 1
+    assert lay.batch_of([torch.zeros(5, 84, 84, 4)] + [torch.zeros(5, 1)] * 4) == 5
+    with pytest.raises(ValueError):
+        lay.batch_of([torch.zeros(5, 84, 84, 4)] + [torch.zeros(4, 1)] * 4)
+    with pytest.raises(ValueError):
+        lay.batch_of([torch.zeros(1)])
+    with pytest.raises(ValueError):
+        FieldLayout([(1,)] * 17, [np.float32] * 17)
+    with pytest.raises(TypeError):
+        as_torch_dtype("complex64")
