@@ -1,0 +1,275 @@
+#!/usr/bin/env python3
+"""Replay-buffer hot-path benchmark on one MI355X.
+
+A step is one pass of the hot path over one batch: PriorityReplayBuffer.sample
+(stratified sum-tree descent + importance weights + row gather) on the
+Atari-shaped buffer of capacity 1,000,000 (28,241 stored bytes per row, batch
+512). Inputs are synthetic and resident in HBM before the timed region; the
+sampling uniforms are drawn on the host beforehand, one set per step.
+
+Prints ONE JSON line. `roofline` prices the sample kernel's algorithmic bytes
+against the HBM peak; `cpu_baseline` is the CPU oracle timed on this machine's
+host cores on a bounded sample of the same workload (rank 0, N = 1 only).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (capacity, batch, shapes, numpy dtypes, update n, insert n, description)
+    "c3": (1_000_000, 512, [(84, 84, 4), (1,), (1,), (1,), (1,)], ["uint8", "int64", "int32", "float32", "bool"],
+           512, 4, "config 3: Atari-shaped PriorityReplayBuffer, capacity 1,000,000, 28,241 B stored rows "
+                   "(obs u8[84,84,4] + next_idx i64 + action i32 + reward f32 + done bool), batch 512"),
+    "c4": (1 << 21, 1024, [(64,), (1,), (1,), (64,), (1,)], ["float32", "int32", "float32", "float32", "bool"],
+           2048, 4096, "config 4: Ape-X PriorityReplayBuffer, capacity 2,097,152, 521 B rows, batch 1024"),
+    "c5": (1 << 24, 65536, [(1,), (1,)], ["int32", "float32"], 65536, 4096,
+           "config 5: tree-descent stress, capacity 16,777,216, 8 B rows, batch 65,536"),
+}
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=2000)
+    p.add_argument("--warmup", type=int, default=200)
+    p.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    p.add_argument("--capacity", type=int, default=0, help="override the workload's capacity (for quick trials)")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--graph", action="store_true", help="replay the timed steps as one captured HIP graph")
+    p.add_argument("--row-split", type=int, default=0, help="workgroups per sampled row (0 = library default)")
+    p.add_argument("--sample-path", type=int, default=0, help="0 auto, 1 wide-row kernel, 2 LDS-top kernel")
+    p.add_argument("--extras", action="store_true", help="also time update_priorities, insert and the full loop")
+    return p.parse_args()
+
+
+def fill_per(buf, torch, capacity, shapes, np_dtypes, seed):
+    """Prefill to capacity in chunks (rows generated on the device), then set lognormal priorities."""
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    row_bytes = sum(int(np.prod(s)) * np.dtype(d).itemsize for s, d in zip(shapes, np_dtypes))
+    chunk = max(1, min(capacity, (256 << 20) // row_bytes))
+    done = 0
+    while done < capacity:
+        n = min(chunk, capacity - done)
+        fields = []
+        for s, d in zip(shapes, np_dtypes):
+            d = np.dtype(d)
+            if d == np.uint8:
+                fields.append(torch.randint(0, 256, (n,) + tuple(s), dtype=torch.uint8, device="cuda", generator=gen))
+            elif d == np.bool_:
+                fields.append(torch.rand((n,) + tuple(s), device="cuda", generator=gen) < 0.01)
+            elif d.kind == "f":
+                fields.append(torch.randn((n,) + tuple(s), device="cuda", generator=gen))
+            elif d == np.int64:
+                fields.append(((torch.arange(done, done + n, device="cuda") + 1) % capacity).reshape((n,) + tuple(s)))
+            else:
+                fields.append(torch.randint(0, 18, (n,) + tuple(s), dtype=torch.int32, device="cuda", generator=gen))
+        buf.insert(*fields)
+        done += n
+    rng = np.random.default_rng(seed)
+    pr = rng.lognormal(0.0, 1.0, capacity).astype(np.float32)
+    buf.update_priorities(torch.arange(capacity, device="cuda"), torch.from_numpy(pr).cuda())
+    torch.cuda.synchronize()
+    return pr
+
+
+def cpu_baseline(workload, shapes, np_dtypes, batch, seed):
+    """The CPU oracle (sequential C restatement of the reference path) on this host:
+    same row shape and batch, capacity cut to 131,072 rows to bound memory and time."""
+    from oracle import orc
+    cap = min(WORKLOADS[workload][0], 1 << 17)
+    rng = np.random.default_rng(seed)
+    per = orc.OraclePER(0.6, cap, shapes, np_dtypes, seed=seed)
+    chunk = 2048
+    rows = []
+    for s, d in zip(shapes, np_dtypes):
+        d = np.dtype(d)
+        if d == np.uint8:
+            rows.append(rng.integers(0, 256, (chunk,) + tuple(s), dtype=np.uint8))
+        elif d == np.bool_:
+            rows.append(rng.random((chunk,) + tuple(s)) < 0.01)
+        else:
+            rows.append(rng.integers(0, 3, (chunk,) + tuple(s)).astype(d))
+    for start in range(0, cap, chunk):
+        per.push(rows, min(chunk, cap - start))
+    per.update(np.arange(cap), rng.lognormal(0, 1, cap).astype(np.float32))
+    L = orc.lib()
+    idx = np.empty(batch, np.int64)
+    w = np.empty(batch, np.float32)
+    dst = per._dst(batch)
+    dptr = orc._ptr_array(dst)
+    calls, t_end = 0, time.perf_counter() + 12.0
+    u_all = rng.random((64, batch)).astype(np.float32)
+    t0 = time.perf_counter()
+    while time.perf_counter() < t_end:
+        u = u_all[calls % 64]
+        rc = L.orc_per_sample(per.h, batch, 0.4, u.ctypes.data, idx.ctypes.data, w.ctypes.data, dptr)
+        assert rc == 0
+        calls += 1
+    dt = time.perf_counter() - t0
+    return {
+        "value": calls * batch / dt, "unit": "transitions/s", "cores": 1, "kind": "port",
+        "sample": "%d sample calls (batch %d, same row shape) in %.1f s on a capacity-%d buffer, 1 thread" % (
+            calls, batch, dt, cap),
+    }
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this benchmark measures one GPU; --gpus %d is not supported (every box here has one GPU)"
+              % a.gpus, file=sys.stderr)
+        return 2
+    import torch
+
+    from mindrl_amd import _lib
+    from mindrl_amd.core import PriorityReplayBuffer
+    from mindrl_amd.core._rows import pointers
+
+    assert torch.cuda.is_available(), "bench.py needs a HIP device"
+    torch.cuda.set_device(0)
+    capacity, batch, shapes, np_dtypes, upd_n, ins_n, desc = WORKLOADS[a.workload]
+    _lib.set_option("row_split", a.row_split)
+    _lib.set_option("sample_path", a.sample_path)
+    if a.capacity:
+        capacity = a.capacity
+        desc += " [capacity overridden to %d]" % capacity
+    seed = 1000 + int(a.workload[1])
+    t_types = [getattr(torch, d) for d in np_dtypes]
+    buf = PriorityReplayBuffer(0.6, capacity, batch, shapes, t_types, seed0=seed)
+    t0 = time.perf_counter()
+    fill_per(buf, torch, capacity, shapes, np_dtypes, seed)
+    fill_s = time.perf_counter() - t0
+
+    K, W = a.steps, a.warmup
+    rng = np.random.default_rng(seed + 1)
+    uniforms = torch.from_numpy(rng.random((K + W, batch)).astype(np.float32)).cuda()
+    betas = np.linspace(0.4, 1.0, K + W).astype(np.float32)
+    idx = torch.empty(batch, dtype=torch.int64, device="cuda")
+    wts = torch.empty(batch, dtype=torch.float32, device="cuda")
+    fields = buf._layout.empty(batch, buf._dev)
+    fptr = pointers(fields)
+    L = _lib.lib()
+    stream = torch.cuda.current_stream()
+    sp = C.c_void_p(stream.cuda_stream)
+    h = buf._h
+    ubase, ustride = uniforms.data_ptr(), batch * 4
+    ip, wp = idx.data_ptr(), wts.data_ptr()
+
+    def step(i):
+        rc = L.mrb_per_sample(h, batch, float(betas[i]), ubase + i * ustride, ip, wp, fptr, sp)
+        if rc:
+            _lib.check(rc)
+
+    for i in range(W):
+        step(i)
+    torch.cuda.synchronize()
+
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    graph = None
+    if a.graph:
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            sp_side = C.c_void_p(side.cuda_stream)
+            graph.capture_begin()
+            for i in range(W, W + K):
+                rc = L.mrb_per_sample(h, batch, float(betas[i]), ubase + i * ustride, ip, wp, fptr, sp_side)
+                if rc:
+                    _lib.check(rc)
+            graph.capture_end()
+        torch.cuda.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    if graph is not None:
+        graph.replay()
+    else:
+        for i in range(W, W + K):
+            step(i)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = ev0.elapsed_time(ev1)
+    flags = buf.check()
+
+    row_bytes = sum(buf._layout.bytes)
+    algo_bytes = batch * (2 * row_bytes + 12)  # rows read + rows written + index (8) + weight (4)
+    kern_s = dev_ms * 1e-3 / K
+    achieved = algo_bytes / kern_s / 1e9
+    out = {
+        "metric": "sampled transitions/sec (sample+IS+gather) at cap 1M; HBM GB/s vs peak",
+        "value": K * batch / wall,
+        "unit": "transitions/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": wall * 1e3 / K,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": desc, "capacity": capacity, "batch": batch, "row_bytes": row_bytes,
+                   "alpha": 0.6, "beta": "0.4->1.0", "launch": "hip graph replay" if a.graph else "eager C-ABI calls",
+                   "prefill_s": round(fill_s, 2), "device_flags": flags},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "k_per_sample_wide", "algorithmic_bytes_per_launch": algo_bytes,
+                     "avg_launch_us": kern_s * 1e6},
+    }
+
+    if a.extras:
+        extras = {}
+        uidx = torch.from_numpy(rng.integers(0, capacity, (64, upd_n))).cuda()
+        upr = torch.from_numpy((np.abs(rng.normal(size=(64, upd_n))) + 1e-6).astype(np.float32)).cuda()
+        n_it = 300
+        for i in range(20):
+            L.mrb_per_update(h, uidx[i % 64].data_ptr(), upr[i % 64].data_ptr(), upd_n, sp)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n_it):
+            L.mrb_per_update(h, uidx[i % 64].data_ptr(), upr[i % 64].data_ptr(), upd_n, sp)
+        torch.cuda.synchronize()
+        extras["updates_per_s"] = n_it * upd_n / (time.perf_counter() - t0)
+        src = [f[:ins_n].contiguous() if f.shape[0] >= ins_n else f.repeat((ins_n + f.shape[0] - 1) // f.shape[0],
+               *([1] * (f.dim() - 1)))[:ins_n].contiguous() for f in fields]
+        sptr = pointers(src)
+        for i in range(20):
+            L.mrb_per_push(h, sptr, ins_n, None, sp)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n_it):
+            L.mrb_per_push(h, sptr, ins_n, None, sp)
+        torch.cuda.synchronize()
+        extras["inserts_per_s"] = n_it * ins_n / (time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        for i in range(n_it):
+            step(W + (i % K))
+            L.mrb_per_update(h, ip, upr[i % 64].data_ptr(), min(upd_n, batch), sp)
+            L.mrb_per_push(h, sptr, ins_n, None, sp)
+        torch.cuda.synchronize()
+        extras["loop_steps_per_s"] = n_it / (time.perf_counter() - t0)
+        out["extras"] = extras
+
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(a.workload, shapes, np_dtypes, batch, seed)
+    else:
+        out["cpu_baseline"] = None
+    buf.destroy()
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -542,7 +542,10 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, 
             if (split < 1) split = 1;
             if (split > 16) split = 16;
         }
-        hipLaunchKernelGGL(k_per_sample_wide, dim3((uint32_t)(batch * split)), dim3(kWG), 0, s, t, a, split);
+        SplitPlan plan{};
+        plan.split = split;
+        for (int i = 0; i < b->rows.nfields; ++i) plan.per[i] = (b->rows.units[i] + split - 1) / split;
+        hipLaunchKernelGGL(k_per_sample_wide, dim3((uint32_t)(batch * split)), dim3(kWG), 0, s, t, a, plan);
         LAUNCH_CHECK("k_per_sample_wide");
     } else {
         int levels = g_opt.lds_levels > 0 ? (int)g_opt.lds_levels : 12;

@@ -87,68 +87,106 @@ __device__ __forceinline__ int64_t rng_below(uint64_t seed, uint64_t counter, ui
 }
 
 // ---------------------------------------------------------------------------
-// Wave-cooperative descent of `g` (1..8) sum-tree levels.
+// Wave-cooperative descent of up to 10 sum-tree levels per memory round trip.
 //
 // The tree is a heap (root 1, children 2i and 2i+1), each level contiguous.
 // The 2^g descendants of `node` that lie g levels below it are the contiguous
-// run [node << g, (node + 1) << g): one coalesced load of at most 1 KB
-// (float4 per lane). Every node between is, by construction of the tree, the
-// single rounded sum of its two children, so the wave rebuilds those g-1
-// levels in registers with the same additions (a + b == b + a bitwise) and
-// walks them without further memory traffic. The walk is the reference's
-// prefix-sum descent: go left when mass <= left sum, otherwise subtract it
-// and go right.
+// run [node << g, (node + 1) << g): at most 4 KB, loaded as up to four float4
+// per lane (lane l holds 16 consecutive nodes). Every node between is, by
+// construction of the tree, the single rounded sum of its two children, so the
+// wave rebuilds those levels in registers with the same additions
+// (a + b == b + a bitwise): four levels inside each lane, six across lanes.
+// The walk then needs no further memory traffic. It is the reference's
+// prefix-sum descent: go left when mass <= left sum, otherwise subtract the
+// left sum and go right.
 //
-// All 64 lanes must call this together; every lane returns the same result.
-// `picked` receives the value of the node reached.
+// Loading and walking are separate so that a group whose address is already
+// known (the one under the root) can be in flight before the mass is.
+// All 64 lanes must call these together; every lane obtains the same result.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ uint32_t descend_group(const float* __restrict__ sum, uint32_t node, int g,
-                                                  float& mass, float& picked, int lane) {
+constexpr int kGroupMaxLevels = 10;
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+struct NodeGroup {
+    f32x16 v;  // this lane's 16 consecutive bottom nodes (0 where the group is narrower)
+};
+
+__device__ __forceinline__ void group_load(const float* __restrict__ sum, uint32_t node, int g, int lane,
+                                           NodeGroup& n) {
     const uint32_t base = node << g;
     const uint32_t width = 1u << g;
-    float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
+    f32x4 t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
     if (g >= 2) {
-        if ((uint32_t)(4 * lane) < width) {
-            const float4 t = *reinterpret_cast<const float4*>(sum + base + 4 * lane);
-            v0 = t.x;
-            v1 = t.y;
-            v2 = t.z;
-            v3 = t.w;
-        }
+        const uint32_t off = 16u * lane;
+        const f32x4* src = reinterpret_cast<const f32x4*>(sum + base + off);
+        if (off + 0 < width) t0 = src[0];
+        if (off + 4 < width) t1 = src[1];
+        if (off + 8 < width) t2 = src[2];
+        if (off + 12 < width) t3 = src[3];
     } else if (lane == 0) {
-        v0 = sum[base];
-        v1 = sum[base + 1];
+        t0.x = sum[base];
+        if (g == 1) t0.y = sum[base + 1];
     }
-    const float a0 = v0 + v1;
-    const float a1 = v2 + v3;
-    const float c0 = a0 + a1;
+    n.v = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
+                                  __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8,
+                                  9, 10, 11, 12, 13, 14, 15);
+}
+
+__device__ __forceinline__ float lane_value(float x, uint32_t src_lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)src_lane));
+}
+
+// Walks the g levels held in `n`, starting at the group's root with `mass`.
+// Returns the offset of the node reached among the group's 2^g bottom nodes;
+// `mass` is left as the remainder, `picked` receives that node's value.
+// The position is kept wave-uniform (scalar), so element selection inside a
+// lane is a register-indexed move, not a memory access.
+__device__ __forceinline__ uint32_t group_walk(const NodeGroup& n, int g, float& mass, float& picked) {
+    const f32x8 q8 = __builtin_shufflevector(n.v, n.v, 0, 2, 4, 6, 8, 10, 12, 14) +
+                     __builtin_shufflevector(n.v, n.v, 1, 3, 5, 7, 9, 11, 13, 15);
+    const f32x4 q4 = __builtin_shufflevector(q8, q8, 0, 2, 4, 6) + __builtin_shufflevector(q8, q8, 1, 3, 5, 7);
+    const float q2a = q4.x + q4.y;
+    const float q2b = q4.z + q4.w;
+    const float c0 = q2a + q2b;
     const float c1 = c0 + __shfl_xor(c0, 1);
     const float c2 = c1 + __shfl_xor(c1, 2);
     const float c3 = c2 + __shfl_xor(c2, 4);
     const float c4 = c3 + __shfl_xor(c3, 8);
     const float c5 = c4 + __shfl_xor(c4, 16);
-    uint32_t p = 0;  // offset among the `width` bottom nodes
+    uint32_t p = 0;
     for (int sl = g - 1; sl >= 0; --sl) {
+        const uint32_t in = p & 15u;
         float cand;
         switch (sl) {
-            case 7: cand = c5; break;
-            case 6: cand = c4; break;
-            case 5: cand = c3; break;
-            case 4: cand = c2; break;
-            case 3: cand = c1; break;
-            case 2: cand = c0; break;
-            case 1: cand = (p & 2u) ? a1 : a0; break;
-            default: cand = (p & 2u) ? ((p & 1u) ? v3 : v2) : ((p & 1u) ? v1 : v0); break;
+            case 9: cand = c5; break;
+            case 8: cand = c4; break;
+            case 7: cand = c3; break;
+            case 6: cand = c2; break;
+            case 5: cand = c1; break;
+            case 4: cand = c0; break;
+            case 3: cand = q2a; break;
+            case 2: cand = q4[in >> 2]; break;
+            case 1: cand = q8[in >> 1]; break;
+            default: cand = n.v[in]; break;
         }
-        const float left = __shfl(cand, (int)(p >> 2));
+        const float left = lane_value(cand, p >> 4);
         if (!(mass <= left)) {
             mass -= left;
             p += 1u << sl;
         }
+        p = (uint32_t)__builtin_amdgcn_readfirstlane((int)p);
     }
-    const float mine = (p & 2u) ? ((p & 1u) ? v3 : v2) : ((p & 1u) ? v1 : v0);
-    picked = __shfl(mine, (int)(p >> 2));
-    return base + p;
+    picked = lane_value(n.v[p & 15u], p >> 4);
+    return p;
+}
+
+// Number of round trips and the levels taken by each for a tree of `depth` levels.
+__device__ __forceinline__ int group_count(int depth) { return (depth + kGroupMaxLevels - 1) / kGroupMaxLevels; }
+__device__ __forceinline__ int group_levels(int depth, int count, int i) {
+    return depth / count + (i < depth % count ? 1 : 0);
 }
 
 }  // namespace mrb

@@ -28,30 +28,92 @@ struct IoTable {
     uint64_t prefix[MRB_MAX_FIELDS + 1];  // running sum of n * units over fields
 };
 
+// Row pointers reach the kernels inside by-value tables, where the compiler cannot
+// see that they point to global memory; the qualified type makes every row access a
+// global_load/global_store rather than a flat one.
+using gbyte = __attribute__((address_space(1))) uint8_t;
+__device__ __forceinline__ gbyte* as_global(uint8_t* p) { return (gbyte*)p; }
+__device__ __forceinline__ const gbyte* as_global(const uint8_t* p) { return (const gbyte*)p; }
+
 // One granule of 1 << vl bytes. Rows are read once and written once, so both
 // sides bypass the caches' retention (non-temporal).
-__device__ __forceinline__ void copy_granule(uint8_t* dst, const uint8_t* src, uint32_t vl) {
+__device__ __forceinline__ void copy_granule(gbyte* dst, const gbyte* src, uint32_t vl) {
     switch (vl) {
         case 4: {
             using v4 = __attribute__((ext_vector_type(4))) uint32_t;
-            v4 t = __builtin_nontemporal_load(reinterpret_cast<const v4*>(src));
-            __builtin_nontemporal_store(t, reinterpret_cast<v4*>(dst));
+            v4 t = __builtin_nontemporal_load((const __attribute__((address_space(1))) v4*)src);
+            __builtin_nontemporal_store(t, (__attribute__((address_space(1))) v4*)dst);
             break;
         }
         case 3: {
             using v2 = __attribute__((ext_vector_type(2))) uint32_t;
-            v2 t = __builtin_nontemporal_load(reinterpret_cast<const v2*>(src));
-            __builtin_nontemporal_store(t, reinterpret_cast<v2*>(dst));
+            v2 t = __builtin_nontemporal_load((const __attribute__((address_space(1))) v2*)src);
+            __builtin_nontemporal_store(t, (__attribute__((address_space(1))) v2*)dst);
             break;
         }
         case 2:
-            *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(src);
+            *(__attribute__((address_space(1))) uint32_t*)dst = *(const __attribute__((address_space(1))) uint32_t*)src;
             break;
         case 1:
-            *reinterpret_cast<uint16_t*>(dst) = *reinterpret_cast<const uint16_t*>(src);
+            *(__attribute__((address_space(1))) uint16_t*)dst = *(const __attribute__((address_space(1))) uint16_t*)src;
             break;
         default:
             *dst = *src;
+            break;
+    }
+}
+
+using granule_t = __attribute__((ext_vector_type(4))) uint32_t;
+
+// Load / store halves of copy_granule, for kernels that keep several granules
+// in flight per thread (all loads issued before the first store).
+__device__ __forceinline__ granule_t load_granule(const gbyte* src, uint32_t vl) {
+    granule_t r = 0;
+    switch (vl) {
+        case 4:
+            r = __builtin_nontemporal_load((const __attribute__((address_space(1))) granule_t*)src);
+            break;
+        case 3: {
+            using v2 = __attribute__((ext_vector_type(2))) uint32_t;
+            const v2 t = __builtin_nontemporal_load((const __attribute__((address_space(1))) v2*)src);
+            r.x = t.x;
+            r.y = t.y;
+            break;
+        }
+        case 2:
+            r.x = *(const __attribute__((address_space(1))) uint32_t*)src;
+            break;
+        case 1:
+            r.x = *(const __attribute__((address_space(1))) uint16_t*)src;
+            break;
+        default:
+            r.x = *src;
+            break;
+    }
+    return r;
+}
+
+__device__ __forceinline__ void store_granule(gbyte* dst, granule_t r, uint32_t vl) {
+    switch (vl) {
+        case 4:
+            __builtin_nontemporal_store(r, (__attribute__((address_space(1))) granule_t*)dst);
+            break;
+        case 3: {
+            using v2 = __attribute__((ext_vector_type(2))) uint32_t;
+            v2 t;
+            t.x = r.x;
+            t.y = r.y;
+            __builtin_nontemporal_store(t, (__attribute__((address_space(1))) v2*)dst);
+            break;
+        }
+        case 2:
+            *(__attribute__((address_space(1))) uint32_t*)dst = r.x;
+            break;
+        case 1:
+            *(__attribute__((address_space(1))) uint16_t*)dst = (uint16_t)r.x;
+            break;
+        default:
+            *dst = (uint8_t)r.x;
             break;
     }
 }
@@ -93,7 +155,7 @@ __global__ __launch_bounds__(kWG) void k_rows_put(IoTable t, int64_t capacity, i
         if (slot >= capacity) slot -= capacity;
         const uint32_t vl = t.vec_log2[f];
         const uint64_t off = (uint64_t)unit << vl;
-        copy_granule(t.store[f] + (uint64_t)slot * t.row_bytes[f] + off, t.io[f] + row * t.row_bytes[f] + off, vl);
+        copy_granule(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f] + off, as_global(t.io[f]) + row * t.row_bytes[f] + off, vl);
     }
 }
 
@@ -116,7 +178,8 @@ __global__ __launch_bounds__(kWG) void k_rows_gather(IoTable t, int64_t capacity
         uint32_t unit;
         split_work(w - t.prefix[f], t.units[f], row, unit);
         int64_t slot = fixed_slot >= 0 ? fixed_slot : indices ? indices[row] : rng_below(seed, calls, row, count);
-        if (slot < 0 || slot >= count) {
+        // a fixed slot was range-checked by the host against the ring (it may lie above `count` after a reset)
+        if (fixed_slot < 0 && (slot < 0 || slot >= count)) {
             if (f == 0 && unit == 0) atomicOr(err, MRB_DERR_INDEX);
             slot = slot < 0 ? 0 : (count > 0 ? count - 1 : 0);
             if (slot >= capacity) slot = capacity - 1;
@@ -124,7 +187,7 @@ __global__ __launch_bounds__(kWG) void k_rows_gather(IoTable t, int64_t capacity
         if (out_indices && f == 0 && unit == 0) out_indices[row] = slot;
         const uint32_t vl = t.vec_log2[f];
         const uint64_t off = (uint64_t)unit << vl;
-        copy_granule(t.io[f] + row * t.row_bytes[f] + off, t.store[f] + (uint64_t)slot * t.row_bytes[f] + off, vl);
+        copy_granule(as_global(t.io[f]) + row * t.row_bytes[f] + off, as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f] + off, vl);
     }
 }
 
@@ -163,52 +226,175 @@ __device__ __forceinline__ void sample_flags(const SampleArgs& a, float total, i
     if (idx >= a.size) atomicOr(a.err, MRB_DERR_UNFILLED);
 }
 
+// How the wide-row sample kernel divides a row among `split` workgroups:
+// workgroup `part` copies granules [part * per[f], (part + 1) * per[f]) of field f.
+struct SplitPlan {
+    int split;
+    uint32_t per[MRB_MAX_FIELDS];
+};
+
+constexpr int kInFlight = 4;  // granules a thread holds between its loads and its stores
+
 // ---------------------------------------------------------------------------
 // PER sample, wide rows: `split` workgroups per sampled row. Wave 0 of every
-// workgroup walks the sum tree for its stratum with descend_group (one
-// dependent load per 8 levels), publishes the slot through LDS, then the whole
-// workgroup copies its share of the row with 16-byte granules. Index and
-// importance weight are written by the row's first workgroup. Replaces
-// PriorityReplayBufferSample (mindspore_rl/core/priority_replay_buffer.py:70,92-106).
+// workgroup walks the sum tree for its stratum with group_load/group_walk (one
+// dependent load per 10 levels; the first group sits under the root, so its
+// load is issued together with the total and the uniform draw) and publishes
+// the slot through LDS. The workgroup's share of the row — granules of all
+// fields, numbered consecutively — is then copied with every load issued
+// before the first store, so a row costs one memory round trip, not one per
+// field. The row's first workgroup computes the importance weight while its
+// loads are in flight (the two powers in two lanes of one instruction stream).
+// Replaces PriorityReplayBufferSample
+// (mindspore_rl/core/priority_replay_buffer.py:70,92-106).
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kWG) void k_per_sample_wide(IoTable t, SampleArgs a, int split) {
+__global__ __launch_bounds__(kWG) void k_per_sample_wide(IoTable t, SampleArgs a, SplitPlan plan) {
     __shared__ int64_t s_idx;
-    const int64_t k = blockIdx.x / (uint32_t)split;
-    const uint32_t part = blockIdx.x % (uint32_t)split;
+    __shared__ float s_picked;
+    // this workgroup's share of each field, filled by wave 1 while wave 0 walks the tree
+    __shared__ const gbyte* s_src[MRB_MAX_FIELDS];  // store_f + first granule's byte offset
+    __shared__ gbyte* s_dst[MRB_MAX_FIELDS];          // io_f + k * row_bytes + the same offset
+    __shared__ uint32_t s_wide[MRB_MAX_FIELDS];       // 16-byte granules of field f copied here
+    __shared__ uint32_t s_narrow[MRB_MAX_FIELDS];     // smaller granules (field rows not a multiple of 16 bytes)
+    __shared__ uint32_t s_vl[MRB_MAX_FIELDS];
+    __shared__ uint32_t s_rb[MRB_MAX_FIELDS];
+    const uint32_t split = (uint32_t)plan.split;
+    const int64_t k = blockIdx.x / split;
+    const uint32_t part = blockIdx.x % split;
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
+        const int ngroups = group_count(a.depth);
+        NodeGroup grp;
+        int g = ngroups ? group_levels(a.depth, ngroups, 0) : 0;
+        if (ngroups) group_load(a.sum, 1u, g, lane, grp);
         const float total = a.sum[1];
         float mass = stratum_mass(a, total, k);
         uint32_t node = 1;
         float picked = total;
-        int g = a.depth % kRoundLevels ? a.depth % kRoundLevels : kRoundLevels;
-        for (int d = 0; d < a.depth; d += g, g = kRoundLevels) node = descend_group(a.sum, node, g, mass, picked, lane);
-        const int64_t idx = (int64_t)node - a.leaves;
+        for (int i = 0; i < ngroups; ++i) {
+            if (i) {
+                g = group_levels(a.depth, ngroups, i);
+                group_load(a.sum, node, g, lane, grp);
+            }
+            node = (node << g) + group_walk(grp, g, mass, picked);
+        }
         if (lane == 0) {
-            s_idx = idx;
-            if (part == 0) {
+            s_idx = (int64_t)node - a.leaves;
+            s_picked = picked;
+        }
+    } else if (threadIdx.x < 64 + MRB_MAX_FIELDS) {
+        const int f = threadIdx.x - 64;
+        uint32_t cnt = 0, vl = 0;
+        if (f < t.nfields) {
+            const uint32_t lo = part * plan.per[f];
+            vl = t.vec_log2[f];
+            const uint64_t off = (uint64_t)lo << vl;
+            cnt = lo < t.units[f] ? min(plan.per[f], t.units[f] - lo) : 0u;
+            s_vl[f] = vl;
+            s_rb[f] = t.row_bytes[f];
+            s_src[f] = as_global(t.store[f]) + off;
+            s_dst[f] = as_global(t.io[f]) + (uint64_t)k * t.row_bytes[f] + off;
+        }
+        s_wide[f] = vl == 4 ? cnt : 0u;
+        s_narrow[f] = vl == 4 ? 0u : cnt;
+    }
+    __syncthreads();
+    const int64_t idx = s_idx;
+    const uint64_t slot = (uint64_t)(idx < a.capacity ? idx : a.capacity - 1);
+    // This workgroup's granules, numbered consecutively over the fields: 16-byte ones
+    // ("wide") and the granules of fields whose rows are not multiples of 16 bytes ("narrow").
+    uint32_t wide_items = 0, narrow_items = 0;
+#pragma unroll
+    for (int f = 0; f < MRB_MAX_FIELDS; ++f) {
+        wide_items += s_wide[f];
+        narrow_items += s_narrow[f];
+    }
+    using g16 = __attribute__((address_space(1))) granule_t;
+    uint32_t wfirst = 0, nfirst = 0;
+    do {
+        // ---- addresses first. A thread without a granule in this pass re-reads granule 0
+        // (a valid address) and skips the store, so that the loads below are unconditional
+        // and can all be in flight together.
+        const g16* wsrc[kInFlight];
+        g16* wdst[kInFlight];
+        bool wlive[kInFlight];
+#pragma unroll
+        for (int j = 0; j < kInFlight; ++j) {
+            uint32_t it = wfirst + j * kWG + threadIdx.x;
+            wlive[j] = it < wide_items;
+            if (!wlive[j]) it = 0;
+            int f = 0;
+            if (wide_items) {
+                uint32_t cnt = s_wide[0];
+                while (it >= cnt) {
+                    it -= cnt;
+                    cnt = s_wide[++f];
+                }
+            }
+            const uint64_t off = (uint64_t)it << 4;
+            wsrc[j] = (const g16*)(s_src[f] + slot * s_rb[f] + off);
+            wdst[j] = (g16*)(s_dst[f] + off);
+        }
+        const gbyte* nsrc;
+        gbyte* ndst;
+        uint32_t nbytes;
+        bool nlive;
+        {
+            uint32_t it = nfirst + threadIdx.x;
+            nlive = it < narrow_items;
+            if (!nlive) it = 0;
+            int f = 0;
+            if (narrow_items) {
+                uint32_t cnt = s_narrow[0];
+                while (it >= cnt) {
+                    it -= cnt;
+                    cnt = s_narrow[++f];
+                }
+            }
+            const uint32_t vl = s_vl[f];
+            const uint64_t off = (uint64_t)it << vl;
+            nsrc = s_src[f] + slot * s_rb[f] + off;
+            ndst = s_dst[f] + off;
+            nbytes = 1u << vl;
+        }
+        // ---- loads
+        granule_t held[kInFlight];
+        uint8_t nb[8];
+        if (wide_items) {
+#pragma unroll
+            for (int j = 0; j < kInFlight; ++j) held[j] = __builtin_nontemporal_load(wsrc[j]);
+        }
+        if (narrow_items) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) nb[i] = nsrc[(uint32_t)i < nbytes ? i : 0];
+        }
+        // ---- importance weight, computed while the loads are in flight
+        if (wfirst == 0 && part == 0 && threadIdx.x < 2) {
+            // lane 0: (p / total * size)^-beta, lane 1: (pmin / total * size)^-beta
+            const float total = a.sum[1];
+            const float x = threadIdx.x == 0 ? s_picked : a.mn[1];
+            const float r = powf_det(x / total * (float)a.size, -a.beta);
+            const float max_w = __shfl(r, 1);
+            if (threadIdx.x == 0) {
                 a.out_idx[k] = idx;
-                a.out_w[k] = is_weight(picked, total, a.mn[1], (float)a.size, a.beta);
+                a.out_w[k] = r / max_w;
                 sample_flags(a, total, idx);
             }
         }
-    }
-    __syncthreads();
-    int64_t slot = s_idx;
-    if (slot >= a.capacity) slot = a.capacity - 1;
-    for (int f = 0; f < t.nfields; ++f) {
-        const uint32_t units = t.units[f];
-        const uint32_t per = (units + split - 1) / split;
-        const uint32_t lo = part * per;
-        const uint32_t hi = lo + per < units ? lo + per : units;
-        const uint32_t vl = t.vec_log2[f];
-        const uint8_t* src = t.store[f] + (uint64_t)slot * t.row_bytes[f];
-        uint8_t* dst = t.io[f] + (uint64_t)k * t.row_bytes[f];
-        for (uint32_t u = lo + threadIdx.x; u < hi; u += kWG) {
-            const uint64_t off = (uint64_t)u << vl;
-            copy_granule(dst + off, src + off, vl);
+        // ---- stores
+        if (wide_items) {
+#pragma unroll
+            for (int j = 0; j < kInFlight; ++j)
+                if (wlive[j]) __builtin_nontemporal_store(held[j], wdst[j]);
         }
-    }
+        if (narrow_items && nlive) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if ((uint32_t)i < nbytes) ndst[i] = nb[i];
+        }
+        wfirst += kWG * kInFlight;
+        nfirst += kWG;
+    } while (wfirst < wide_items || nfirst < narrow_items);
 }
 
 // ---------------------------------------------------------------------------
@@ -272,8 +458,8 @@ __global__ __launch_bounds__(kWG) void k_per_sample_lds(IoTable t, SampleArgs a,
             uint32_t u;
             split_work(w, units, r, u);
             const uint64_t off = (uint64_t)u << vl;
-            copy_granule(t.io[f] + (uint64_t)(k0 + (int64_t)r) * t.row_bytes[f] + off,
-                         t.store[f] + (uint64_t)s_slot[r] * t.row_bytes[f] + off, vl);
+            copy_granule(as_global(t.io[f]) + (uint64_t)(k0 + (int64_t)r) * t.row_bytes[f] + off,
+                         as_global(t.store[f]) + (uint64_t)s_slot[r] * t.row_bytes[f] + off, vl);
         }
     }
 }

@@ -198,21 +198,26 @@ void orc_urb_seed(orc_urb *b, uint64_t seed) {
     b->calls = 0;
 }
 
-/* insert(): uniform_replay_buffer.py:101-115. One row at a time, in order:
- * while the buffer has never been full it grows at `count`; afterwards the
- * write position is `head` (the oldest row), which then advances. */
+/* insert(): uniform_replay_buffer.py:101-115. The write position is chosen
+ * once per call: `count` while the buffer has never been full (count <
+ * capacity and head == 0), otherwise `head` (the oldest row). Rows then go to
+ * consecutive slots modulo capacity, later rows overwriting earlier ones. */
 int orc_urb_append(orc_urb *b, const void *const *src, int64_t nrows) {
     if (nrows <= 0) return 1;
     int64_t cap = b->rows.capacity;
-    for (int64_t j = 0; j < nrows; ++j) {
-        if (b->count < cap && b->head == 0) {
-            rows_put(&b->rows, b->count, src, j);
-            b->count += 1;
+    int growing = b->count < cap && b->head == 0;
+    int64_t w = growing ? b->count : b->head;
+    for (int64_t j = 0; j < nrows; ++j) rows_put(&b->rows, (w + j) % cap, src, j);
+    if (growing) {
+        if (b->count + nrows <= cap) {
+            b->count += nrows;
         } else {
-            rows_put(&b->rows, b->head, src, j);
-            b->head = (b->head + 1) % cap;
-            if (b->count < cap) b->count += 1;
+            b->head = (b->count + nrows) % cap; /* wrapped: the slot after the newest row holds the oldest */
+            b->count = cap;
         }
+    } else {
+        b->head = (b->head + nrows) % cap;
+        b->count = b->count + nrows < cap ? b->count + nrows : cap;
     }
     return 0;
 }
