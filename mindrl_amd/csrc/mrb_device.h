@@ -114,36 +114,69 @@ struct NodeGroup {
     f32x16 v;  // this lane's 16 consecutive bottom nodes (0 where the group is narrower)
 };
 
-__device__ __forceinline__ void group_load(const float* __restrict__ sum, uint32_t node, int g, int lane,
-                                           NodeGroup& n) {
+// Requests the 2^g (2 <= g <= 10) nodes that lie g levels below `node`: four float4
+// per lane, unconditional (lanes past the group re-read its first granule, discarded
+// later by group_finish), issued back to back. Nothing here uses the loaded values, so
+// the caller can put further independent loads behind these before the first wait.
+struct NodeGroupRaw {
+    f32x4 r0, r1, r2, r3;
+    bool in0, in1, in2, in3;
+};
+
+__device__ __forceinline__ void group_request(const float* __restrict__ sum, uint32_t node, int g, int lane,
+                                              NodeGroupRaw& raw) {
     const uint32_t base = node << g;
     const uint32_t width = 1u << g;
-    f32x4 t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
-    if (g >= 2) {
-        const uint32_t off = 16u * lane;
-        const f32x4* src = reinterpret_cast<const f32x4*>(sum + base + off);
-        if (off + 0 < width) t0 = src[0];
-        if (off + 4 < width) t1 = src[1];
-        if (off + 8 < width) t2 = src[2];
-        if (off + 12 < width) t3 = src[3];
-    } else if (lane == 0) {
-        t0.x = sum[base];
-        if (g == 1) t0.y = sum[base + 1];
-    }
+    const uint32_t off = 16u * lane;
+    const f32x4* src = reinterpret_cast<const f32x4*>(sum + base);
+    raw.in0 = off + 0 < width;
+    raw.in1 = off + 4 < width;
+    raw.in2 = off + 8 < width;
+    raw.in3 = off + 12 < width;
+    raw.r0 = src[raw.in0 ? (off >> 2) + 0 : 0];
+    raw.r1 = src[raw.in1 ? (off >> 2) + 1 : 0];
+    raw.r2 = src[raw.in2 ? (off >> 2) + 2 : 0];
+    raw.r3 = src[raw.in3 ? (off >> 2) + 3 : 0];
+}
+
+__device__ __forceinline__ void group_finish(const NodeGroupRaw& raw, NodeGroup& n) {
+    const f32x4 zero = 0.0f;
+    const f32x4 t0 = raw.in0 ? raw.r0 : zero, t1 = raw.in1 ? raw.r1 : zero;
+    const f32x4 t2 = raw.in2 ? raw.r2 : zero, t3 = raw.in3 ? raw.r3 : zero;
     n.v = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
                                   __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8,
                                   9, 10, 11, 12, 13, 14, 15);
+}
+
+// A group of g < 2 levels (trees of fewer than four leaves): scalar loads by lane 0.
+__device__ __forceinline__ void group_load_tiny(const float* __restrict__ sum, uint32_t node, int g, int lane,
+                                                NodeGroup& n) {
+    n.v = 0.0f;
+    if (lane == 0 && g == 1) {
+        n.v[0] = sum[2 * node];
+        n.v[1] = sum[2 * node + 1];
+    }
 }
 
 __device__ __forceinline__ float lane_value(float x, uint32_t src_lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)src_lane));
 }
 
+// One step of the walk: `left` is the sum of the `1 << SL` bottom nodes starting at p.
+template <int SL>
+__device__ __forceinline__ void walk_step(float cand, uint32_t& p, float& mass) {
+    const float left = lane_value(cand, p >> 4);
+    const bool right = !(mass <= left);
+    mass = right ? mass - left : mass;
+    p = (uint32_t)__builtin_amdgcn_readfirstlane((int)(right ? p + (1u << SL) : p));
+}
+
 // Walks the g levels held in `n`, starting at the group's root with `mass`.
 // Returns the offset of the node reached among the group's 2^g bottom nodes;
 // `mass` is left as the remainder, `picked` receives that node's value.
 // The position is kept wave-uniform (scalar), so element selection inside a
-// lane is a register-indexed move, not a memory access.
+// lane is a register-indexed move, not a memory access; the level tests are
+// scalar branches over straight-line steps.
 __device__ __forceinline__ uint32_t group_walk(const NodeGroup& n, int g, float& mass, float& picked) {
     const f32x8 q8 = __builtin_shufflevector(n.v, n.v, 0, 2, 4, 6, 8, 10, 12, 14) +
                      __builtin_shufflevector(n.v, n.v, 1, 3, 5, 7, 9, 11, 13, 15);
@@ -157,28 +190,16 @@ __device__ __forceinline__ uint32_t group_walk(const NodeGroup& n, int g, float&
     const float c4 = c3 + __shfl_xor(c3, 8);
     const float c5 = c4 + __shfl_xor(c4, 16);
     uint32_t p = 0;
-    for (int sl = g - 1; sl >= 0; --sl) {
-        const uint32_t in = p & 15u;
-        float cand;
-        switch (sl) {
-            case 9: cand = c5; break;
-            case 8: cand = c4; break;
-            case 7: cand = c3; break;
-            case 6: cand = c2; break;
-            case 5: cand = c1; break;
-            case 4: cand = c0; break;
-            case 3: cand = q2a; break;
-            case 2: cand = q4[in >> 2]; break;
-            case 1: cand = q8[in >> 1]; break;
-            default: cand = n.v[in]; break;
-        }
-        const float left = lane_value(cand, p >> 4);
-        if (!(mass <= left)) {
-            mass -= left;
-            p += 1u << sl;
-        }
-        p = (uint32_t)__builtin_amdgcn_readfirstlane((int)p);
-    }
+    if (g > 9) walk_step<9>(c5, p, mass);
+    if (g > 8) walk_step<8>(c4, p, mass);
+    if (g > 7) walk_step<7>(c3, p, mass);
+    if (g > 6) walk_step<6>(c2, p, mass);
+    if (g > 5) walk_step<5>(c1, p, mass);
+    if (g > 4) walk_step<4>(c0, p, mass);
+    if (g > 3) walk_step<3>(q2a, p, mass);
+    if (g > 2) walk_step<2>(q4[(p & 15u) >> 2], p, mass);
+    if (g > 1) walk_step<1>(q8[(p & 15u) >> 1], p, mass);
+    if (g > 0) walk_step<0>(n.v[p & 15u], p, mass);
     picked = lane_value(n.v[p & 15u], p >> 4);
     return p;
 }

@@ -209,10 +209,12 @@ struct SampleArgs {
 };
 
 // mass of stratum k: (u + k) * (total / batch), each operation rounded once.
-__device__ __forceinline__ float stratum_mass(const SampleArgs& a, float total, int64_t k) {
-    const float u = a.uniforms ? a.uniforms[k] : rng_uniform(a.seed, a.calls, (uint64_t)k);
+__device__ __forceinline__ float stratum_mass(const SampleArgs& a, float total, int64_t k, float u) {
     const float seg = total / (float)a.batch;
     return (u + (float)k) * seg;
+}
+__device__ __forceinline__ float stratum_mass(const SampleArgs& a, float total, int64_t k) {
+    return stratum_mass(a, total, k, a.uniforms ? a.uniforms[k] : rng_uniform(a.seed, a.calls, (uint64_t)k));
 }
 
 // w = (p / total * size)^-beta / (pmin / total * size)^-beta
@@ -264,18 +266,29 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(IoTable t, SampleArgs a
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
         const int ngroups = group_count(a.depth);
-        NodeGroup grp;
         int g = ngroups ? group_levels(a.depth, ngroups, 0) : 0;
-        if (ngroups) group_load(a.sum, 1u, g, lane, grp);
+        // The first group hangs under the root: its address is known, so it is requested
+        // together with the total and the draw; the scheduling barrier keeps every request
+        // ahead of the first use.
+        NodeGroup grp;
+        NodeGroupRaw raw;
+        if (g >= 2) group_request(a.sum, 1u, g, lane, raw);
         const float total = a.sum[1];
-        float mass = stratum_mass(a, total, k);
-        uint32_t node = 1;
+        const float u = a.uniforms ? a.uniforms[k] : rng_uniform(a.seed, a.calls, (uint64_t)k);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g >= 2) {
+            group_finish(raw, grp);
+        } else {
+            group_load_tiny(a.sum, 1u, g, lane, grp);
+        }
+        float mass = stratum_mass(a, total, k, u);
         float picked = total;
-        for (int i = 0; i < ngroups; ++i) {
-            if (i) {
-                g = group_levels(a.depth, ngroups, i);
-                group_load(a.sum, node, g, lane, grp);
-            }
+        uint32_t node = (1u << g) + (g ? group_walk(grp, g, mass, picked) : 0u);
+        for (int i = 1; i < ngroups; ++i) {
+            g = group_levels(a.depth, ngroups, i);  // >= 5 once there are two groups
+            group_request(a.sum, node, g, lane, raw);
+            __builtin_amdgcn_sched_barrier(0);
+            group_finish(raw, grp);
             node = (node << g) + group_walk(grp, g, mass, picked);
         }
         if (lane == 0) {
