@@ -545,14 +545,15 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, 
         SplitPlan plan{};
         plan.split = split;
         for (int i = 0; i < b->rows.nfields; ++i) plan.per[i] = (b->rows.units[i] + split - 1) / split;
-        hipLaunchKernelGGL(k_per_sample_wide, dim3((uint32_t)(batch * split)), dim3(kWG), 0, s, t, a, plan);
+        hipLaunchKernelGGL(k_per_sample_wide, dim3((uint32_t)(batch * split)), dim3(kWG), 0, s, a.sum, a.uniforms,
+                           a.depth, split, a.batch, a.seed, a.calls, a, t, plan);
         LAUNCH_CHECK("k_per_sample_wide");
     } else {
         int levels = g_opt.lds_levels > 0 ? (int)g_opt.lds_levels : 12;
         if (levels > b->depth) levels = b->depth;
         const uint32_t ntop = (2u << levels) < 4 ? 4 : (2u << levels);
         const size_t lds = ntop * sizeof(float) + kWG * sizeof(int64_t);
-        hipLaunchKernelGGL(k_per_sample_lds, dim3((uint32_t)((batch + kWG - 1) / kWG)), dim3(kWG), lds, s, t, a, levels);
+        hipLaunchKernelGGL(k_per_sample_lds, dim3((uint32_t)((batch + kWG - 1) / kWG)), dim3(kWG), lds, s, a, t, levels);
         LAUNCH_CHECK("k_per_sample_lds");
     }
     if (!uniforms) b->calls += 1;

@@ -110,52 +110,43 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-struct NodeGroup {
-    f32x16 v;  // this lane's 16 consecutive bottom nodes (0 where the group is narrower)
-};
-
 // Requests the 2^g (2 <= g <= 10) nodes that lie g levels below `node`: four float4
 // per lane, unconditional (lanes past the group re-read its first granule, discarded
 // later by group_finish), issued back to back. Nothing here uses the loaded values, so
 // the caller can put further independent loads behind these before the first wait.
-struct NodeGroupRaw {
-    f32x4 r0, r1, r2, r3;
-    bool in0, in1, in2, in3;
-};
-
+// Everything is passed in registers (plain vector values, no aggregates in memory).
 __device__ __forceinline__ void group_request(const float* __restrict__ sum, uint32_t node, int g, int lane,
-                                              NodeGroupRaw& raw) {
+                                              f32x4& r0, f32x4& r1, f32x4& r2, f32x4& r3) {
     const uint32_t base = node << g;
     const uint32_t width = 1u << g;
     const uint32_t off = 16u * lane;
     const f32x4* src = reinterpret_cast<const f32x4*>(sum + base);
-    raw.in0 = off + 0 < width;
-    raw.in1 = off + 4 < width;
-    raw.in2 = off + 8 < width;
-    raw.in3 = off + 12 < width;
-    raw.r0 = src[raw.in0 ? (off >> 2) + 0 : 0];
-    raw.r1 = src[raw.in1 ? (off >> 2) + 1 : 0];
-    raw.r2 = src[raw.in2 ? (off >> 2) + 2 : 0];
-    raw.r3 = src[raw.in3 ? (off >> 2) + 3 : 0];
+    r0 = src[off + 0 < width ? (off >> 2) + 0 : 0];
+    r1 = src[off + 4 < width ? (off >> 2) + 1 : 0];
+    r2 = src[off + 8 < width ? (off >> 2) + 2 : 0];
+    r3 = src[off + 12 < width ? (off >> 2) + 3 : 0];
 }
 
-__device__ __forceinline__ void group_finish(const NodeGroupRaw& raw, NodeGroup& n) {
+// The lane's 16 consecutive bottom nodes, 0 where the group is narrower.
+__device__ __forceinline__ f32x16 group_finish(int g, int lane, f32x4 r0, f32x4 r1, f32x4 r2, f32x4 r3) {
+    const uint32_t width = 1u << g;
+    const uint32_t off = 16u * lane;
     const f32x4 zero = 0.0f;
-    const f32x4 t0 = raw.in0 ? raw.r0 : zero, t1 = raw.in1 ? raw.r1 : zero;
-    const f32x4 t2 = raw.in2 ? raw.r2 : zero, t3 = raw.in3 ? raw.r3 : zero;
-    n.v = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
-                                  __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8,
-                                  9, 10, 11, 12, 13, 14, 15);
+    const f32x4 t0 = off + 0 < width ? r0 : zero, t1 = off + 4 < width ? r1 : zero;
+    const f32x4 t2 = off + 8 < width ? r2 : zero, t3 = off + 12 < width ? r3 : zero;
+    return __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
+                                   __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8,
+                                   9, 10, 11, 12, 13, 14, 15);
 }
 
 // A group of g < 2 levels (trees of fewer than four leaves): scalar loads by lane 0.
-__device__ __forceinline__ void group_load_tiny(const float* __restrict__ sum, uint32_t node, int g, int lane,
-                                                NodeGroup& n) {
-    n.v = 0.0f;
+__device__ __forceinline__ f32x16 group_load_tiny(const float* __restrict__ sum, uint32_t node, int g, int lane) {
+    f32x16 v = 0.0f;
     if (lane == 0 && g == 1) {
-        n.v[0] = sum[2 * node];
-        n.v[1] = sum[2 * node + 1];
+        v.s0 = sum[2 * node];
+        v.s1 = sum[2 * node + 1];
     }
+    return v;
 }
 
 __device__ __forceinline__ float lane_value(float x, uint32_t src_lane) {
@@ -171,15 +162,15 @@ __device__ __forceinline__ void walk_step(float cand, uint32_t& p, float& mass) 
     p = (uint32_t)__builtin_amdgcn_readfirstlane((int)(right ? p + (1u << SL) : p));
 }
 
-// Walks the g levels held in `n`, starting at the group's root with `mass`.
+// Walks the g levels held in `v`, starting at the group's root with `mass`.
 // Returns the offset of the node reached among the group's 2^g bottom nodes;
 // `mass` is left as the remainder, `picked` receives that node's value.
 // The position is kept wave-uniform (scalar), so element selection inside a
 // lane is a register-indexed move, not a memory access; the level tests are
 // scalar branches over straight-line steps.
-__device__ __forceinline__ uint32_t group_walk(const NodeGroup& n, int g, float& mass, float& picked) {
-    const f32x8 q8 = __builtin_shufflevector(n.v, n.v, 0, 2, 4, 6, 8, 10, 12, 14) +
-                     __builtin_shufflevector(n.v, n.v, 1, 3, 5, 7, 9, 11, 13, 15);
+__device__ __forceinline__ uint32_t group_walk(f32x16 v, int g, float& mass, float& picked) {
+    const f32x8 q8 = __builtin_shufflevector(v, v, 0, 2, 4, 6, 8, 10, 12, 14) +
+                     __builtin_shufflevector(v, v, 1, 3, 5, 7, 9, 11, 13, 15);
     const f32x4 q4 = __builtin_shufflevector(q8, q8, 0, 2, 4, 6) + __builtin_shufflevector(q8, q8, 1, 3, 5, 7);
     const float q2a = q4.x + q4.y;
     const float q2b = q4.z + q4.w;
@@ -199,8 +190,8 @@ __device__ __forceinline__ uint32_t group_walk(const NodeGroup& n, int g, float&
     if (g > 3) walk_step<3>(q2a, p, mass);
     if (g > 2) walk_step<2>(q4[(p & 15u) >> 2], p, mass);
     if (g > 1) walk_step<1>(q8[(p & 15u) >> 1], p, mass);
-    if (g > 0) walk_step<0>(n.v[p & 15u], p, mass);
-    picked = lane_value(n.v[p & 15u], p >> 4);
+    if (g > 0) walk_step<0>(v[p & 15u], p, mass);
+    picked = lane_value(v[p & 15u], p >> 4);
     return p;
 }
 

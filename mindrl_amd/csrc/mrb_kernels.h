@@ -191,18 +191,20 @@ __global__ __launch_bounds__(kWG) void k_rows_gather(IoTable t, int64_t capacity
     }
 }
 
-// Arguments common to both sample kernels.
+// Arguments common to both sample kernels. Passed first, with the fields that the
+// tree descent needs at the front: the leading kernel-argument dwords are preloaded
+// into scalar registers at wave launch, which saves a dependent fetch.
 struct SampleArgs {
-    const float* sum;   // sum tree, heap order
-    const float* mn;    // min tree, heap order
-    int depth;          // log2(leaves)
+    const float* sum;       // sum tree, heap order
+    const float* uniforms;  // f32[batch] or NULL -> generator
+    int64_t batch;
+    int depth;              // log2(leaves)
+    float beta;
+    uint64_t seed, calls;
     int64_t leaves;
     int64_t capacity;
     int64_t size;
-    int64_t batch;
-    float beta;
-    const float* uniforms;  // f32[batch] or NULL -> generator
-    uint64_t seed, calls;
+    const float* mn;        // min tree, heap order
     int64_t* out_idx;
     float* out_w;
     uint32_t* err;
@@ -250,7 +252,9 @@ constexpr int kInFlight = 4;  // granules a thread holds between its loads and i
 // Replaces PriorityReplayBufferSample
 // (mindspore_rl/core/priority_replay_buffer.py:70,92-106).
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kWG) void k_per_sample_wide(IoTable t, SampleArgs a, SplitPlan plan) {
+__global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict__ sum, const float* __restrict__ uniforms,
+                                                         int depth, int split_arg, int64_t batch, uint64_t seed,
+                                                         uint64_t calls, SampleArgs a, IoTable t, SplitPlan plan) {
     __shared__ int64_t s_idx;
     __shared__ float s_picked;
     // this workgroup's share of each field, filled by wave 1 while wave 0 walks the tree
@@ -260,36 +264,40 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(IoTable t, SampleArgs a
     __shared__ uint32_t s_narrow[MRB_MAX_FIELDS];     // smaller granules (field rows not a multiple of 16 bytes)
     __shared__ uint32_t s_vl[MRB_MAX_FIELDS];
     __shared__ uint32_t s_rb[MRB_MAX_FIELDS];
-    const uint32_t split = (uint32_t)plan.split;
+    // sum, uniforms, depth, split, batch, seed and calls repeat fields of `a` and `plan` as plain
+    // leading parameters: those are preloaded into scalar registers when the wave starts.
+    const uint32_t split = (uint32_t)split_arg;
     const int64_t k = blockIdx.x / split;
     const uint32_t part = blockIdx.x % split;
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
-        const int ngroups = group_count(a.depth);
-        int g = ngroups ? group_levels(a.depth, ngroups, 0) : 0;
-        // The first group hangs under the root: its address is known, so it is requested
-        // together with the total and the draw; the scheduling barrier keeps every request
-        // ahead of the first use.
-        NodeGroup grp;
-        NodeGroupRaw raw;
-        if (g >= 2) group_request(a.sum, 1u, g, lane, raw);
-        const float total = a.sum[1];
-        const float u = a.uniforms ? a.uniforms[k] : rng_uniform(a.seed, a.calls, (uint64_t)k);
-        __builtin_amdgcn_sched_barrier(0);
-        if (g >= 2) {
-            group_finish(raw, grp);
-        } else {
-            group_load_tiny(a.sum, 1u, g, lane, grp);
-        }
-        float mass = stratum_mass(a, total, k, u);
-        float picked = total;
-        uint32_t node = (1u << g) + (g ? group_walk(grp, g, mass, picked) : 0u);
-        for (int i = 1; i < ngroups; ++i) {
-            g = group_levels(a.depth, ngroups, i);  // >= 5 once there are two groups
-            group_request(a.sum, node, g, lane, raw);
+        const int ngroups = group_count(depth);
+        int g = ngroups ? group_levels(depth, ngroups, 0) : 0;
+        uint32_t node;
+        float picked, mass;
+        if (depth >= 2) {
+            // The first group hangs under the root: its address is known, so it is requested
+            // together with the total and the draw; the scheduling barrier keeps every
+            // request ahead of the first use.
+            f32x4 r0, r1, r2, r3;
+            group_request(sum, 1u, g, lane, r0, r1, r2, r3);
+            const float total = sum[1];
+            const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
             __builtin_amdgcn_sched_barrier(0);
-            group_finish(raw, grp);
-            node = (node << g) + group_walk(grp, g, mass, picked);
+            mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
+            node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, mass, picked);
+            for (int i = 1; i < ngroups; ++i) {
+                g = group_levels(depth, ngroups, i);  // >= 5 once there are two groups
+                group_request(sum, node, g, lane, r0, r1, r2, r3);
+                __builtin_amdgcn_sched_barrier(0);
+                node = (node << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, mass, picked);
+            }
+        } else {
+            // one or two leaves
+            const float total = sum[1];
+            mass = stratum_mass(a, total, k);
+            picked = total;
+            node = (1u << g) + (g ? group_walk(group_load_tiny(sum, 1u, g, lane), g, mass, picked) : 0u);
         }
         if (lane == 0) {
             s_idx = (int64_t)node - a.leaves;
@@ -417,7 +425,7 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(IoTable t, SampleArgs a
 // the levels below; then the workgroup gathers its 256 rows with coalesced
 // writes. Same outputs, bit for bit, as k_per_sample_wide.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kWG) void k_per_sample_lds(IoTable t, SampleArgs a, int lds_levels) {
+__global__ __launch_bounds__(kWG) void k_per_sample_lds(SampleArgs a, IoTable t, int lds_levels) {
     extern __shared__ float s_top[];  // [2 << lds_levels] floats, then kWG int64 slots
     const uint32_t ntop = 2u << lds_levels;
     int64_t* s_slot = reinterpret_cast<int64_t*>(s_top + (ntop < 4 ? 4 : ntop));
