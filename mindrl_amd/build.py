@@ -17,6 +17,7 @@ HIPCC_FLAGS = [
     "-fhip-fp32-correctly-rounded-divide-sqrt",
     # no packed-fp32 instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall",
 ]
 

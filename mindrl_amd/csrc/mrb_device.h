@@ -149,6 +149,11 @@ __device__ __forceinline__ f32x16 group_load_tiny(const float* __restrict__ sum,
     return v;
 }
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), CTRL, 0xF, 0xF, true));
+}
+
 __device__ __forceinline__ float lane_value(float x, uint32_t src_lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)src_lane));
 }
@@ -175,10 +180,13 @@ __device__ __forceinline__ uint32_t group_walk(f32x16 v, int g, float& mass, flo
     const float q2a = q4.x + q4.y;
     const float q2b = q4.z + q4.w;
     const float c0 = q2a + q2b;
-    const float c1 = c0 + __shfl_xor(c0, 1);
-    const float c2 = c1 + __shfl_xor(c1, 2);
-    const float c3 = c2 + __shfl_xor(c2, 4);
-    const float c4 = c3 + __shfl_xor(c3, 8);
+    // Sums of aligned groups of 2, 4, 8, 16 and 32 lanes. Within a row of 16 lanes the
+    // partner value comes through DPP (no LDS crossbar): once the four lanes of a quad
+    // agree, any lane of the neighbouring quad / half-row / row-half is a valid partner.
+    const float c1 = c0 + dpp_move<0xB1>(c0);   // quad_perm [1,0,3,2]: lane ^ 1
+    const float c2 = c1 + dpp_move<0x4E>(c1);   // quad_perm [2,3,0,1]: lane ^ 2
+    const float c3 = c2 + dpp_move<0x141>(c2);  // row_half_mirror: lane i <-> 7 - i
+    const float c4 = c3 + dpp_move<0x140>(c3);  // row_mirror: lane i <-> 15 - i
     const float c5 = c4 + __shfl_xor(c4, 16);
     uint32_t p = 0;
     if (g > 9) walk_step<9>(c5, p, mass);
