@@ -158,49 +158,79 @@ __device__ __forceinline__ float lane_value(float x, uint32_t src_lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)src_lane));
 }
 
-// One step of the walk: `left` is the sum of the `1 << SL` bottom nodes starting at p.
-template <int SL>
-__device__ __forceinline__ void walk_step(float cand, uint32_t& p, float& mass) {
-    const float left = lane_value(cand, p >> 4);
-    const bool right = !(mass <= left);
-    mass = right ? mass - left : mass;
-    p = (uint32_t)__builtin_amdgcn_readfirstlane((int)(right ? p + (1u << SL) : p));
-}
-
-// Walks the g levels held in `v`, starting at the group's root with `mass`.
-// Returns the offset of the node reached among the group's 2^g bottom nodes;
-// `mass` is left as the remainder, `picked` receives that node's value.
-// The position is kept wave-uniform (scalar), so element selection inside a
-// lane is a register-indexed move, not a memory access; the level tests are
-// scalar branches over straight-line steps.
-__device__ __forceinline__ uint32_t group_walk(f32x16 v, int g, float& mass, float& picked) {
+// Walks the g levels held in `v` (this lane's 16 consecutive bottom nodes), starting
+// at the group's root with `mass`. Returns the offset of the node reached among the
+// group's 2^g bottom nodes; `mass` is left as the remainder, `picked` receives that
+// node's value.
+//
+// The walk is a chain of dependent compare/subtract steps. Instead of one thread
+// taking them while 63 wait on cross-lane reads, every lane follows the one path that
+// ends inside itself: at each of the (up to six) levels above the lane it knows from
+// its own lane number which way that path turns, applies the same compare and
+// subtraction the sequential walk would apply there, and remembers whether the
+// sequential walk would really have turned that way. Exactly one lane stays
+// consistent at every level; that lane's arithmetic is, operation for operation, the
+// sequential walk's. The four levels inside a lane are then taken with selects.
+__device__ __forceinline__ uint32_t group_walk(f32x16 v, int g, int lane, float& mass, float& picked) {
     const f32x8 q8 = __builtin_shufflevector(v, v, 0, 2, 4, 6, 8, 10, 12, 14) +
                      __builtin_shufflevector(v, v, 1, 3, 5, 7, 9, 11, 13, 15);
     const f32x4 q4 = __builtin_shufflevector(q8, q8, 0, 2, 4, 6) + __builtin_shufflevector(q8, q8, 1, 3, 5, 7);
     const float q2a = q4.x + q4.y;
     const float q2b = q4.z + q4.w;
-    const float c0 = q2a + q2b;
-    // Sums of aligned groups of 2, 4, 8, 16 and 32 lanes. Within a row of 16 lanes the
-    // partner value comes through DPP (no LDS crossbar): once the four lanes of a quad
-    // agree, any lane of the neighbouring quad / half-row / row-half is a valid partner.
-    const float c1 = c0 + dpp_move<0xB1>(c0);   // quad_perm [1,0,3,2]: lane ^ 1
-    const float c2 = c1 + dpp_move<0x4E>(c1);   // quad_perm [2,3,0,1]: lane ^ 2
-    const float c3 = c2 + dpp_move<0x141>(c2);  // row_half_mirror: lane i <-> 7 - i
-    const float c4 = c3 + dpp_move<0x140>(c3);  // row_mirror: lane i <-> 15 - i
-    const float c5 = c4 + __shfl_xor(c4, 16);
-    uint32_t p = 0;
-    if (g > 9) walk_step<9>(c5, p, mass);
-    if (g > 8) walk_step<8>(c4, p, mass);
-    if (g > 7) walk_step<7>(c3, p, mass);
-    if (g > 6) walk_step<6>(c2, p, mass);
-    if (g > 5) walk_step<5>(c1, p, mass);
-    if (g > 4) walk_step<4>(c0, p, mass);
-    if (g > 3) walk_step<3>(q2a, p, mass);
-    if (g > 2) walk_step<2>(q4[(p & 15u) >> 2], p, mass);
-    if (g > 1) walk_step<1>(q8[(p & 15u) >> 1], p, mass);
-    if (g > 0) walk_step<0>(v[p & 15u], p, mass);
-    picked = lane_value(v[p & 15u], p >> 4);
-    return p;
+    // S[s]: sum of the aligned group of 2^s lanes holding this lane; P[s]: the sibling
+    // group's sum. Within a row of 16 lanes the sibling's value comes through DPP: once
+    // the lanes of a group agree, any lane of the sibling group is a valid source.
+    float S[6], P[6];
+    S[0] = q2a + q2b;
+    P[0] = dpp_move<0xB1>(S[0]);  // quad_perm [1,0,3,2]: lane ^ 1
+    S[1] = S[0] + P[0];
+    P[1] = dpp_move<0x4E>(S[1]);  // quad_perm [2,3,0,1]: lane ^ 2
+    S[2] = S[1] + P[1];
+    P[2] = dpp_move<0x141>(S[2]);  // row_half_mirror: lane i <-> 7 - i
+    S[3] = S[2] + P[2];
+    P[3] = dpp_move<0x140>(S[3]);  // row_mirror: lane i <-> 15 - i
+    S[4] = S[3] + P[3];
+    P[4] = __shfl_xor(S[4], 16);
+    S[5] = S[4] + P[4];
+    P[5] = __shfl_xor(S[5], 32);
+    float m = mass;
+    bool ok = true;
+#pragma unroll
+    for (int s = 5; s >= 0; --s) {
+        const bool exists = s + 4 < g;  // wave-uniform
+        const bool bit = (lane >> s) & 1;
+        const float left = bit ? P[s] : S[s];  // the left child is the half whose lane bit is 0
+        const bool right = exists && !(m <= left);
+        ok = ok && (right == bit);
+        m = right ? m - left : m;
+    }
+    // inside the lane: 16 -> 8 -> 4 -> 2 -> 1 nodes
+    uint32_t in = 0;
+    bool r = 3 < g && !(m <= q2a);
+    m = r ? m - q2a : m;
+    in = r ? 8u : 0u;
+    const float h4a = r ? q4.z : q4.x;
+    const f32x4 h8 = r ? q8.hi : q8.lo;
+    const f32x8 hv = r ? v.hi : v.lo;
+    r = 2 < g && !(m <= h4a);
+    m = r ? m - h4a : m;
+    in += r ? 4u : 0u;
+    const float g8a = r ? h8.z : h8.x;
+    const f32x4 gv = r ? hv.hi : hv.lo;
+    r = 1 < g && !(m <= g8a);
+    m = r ? m - g8a : m;
+    in += r ? 2u : 0u;
+    const float fa = r ? gv.z : gv.x;
+    const float fb = r ? gv.w : gv.y;
+    r = 0 < g && !(m <= fa);
+    m = r ? m - fa : m;
+    in += r ? 1u : 0u;
+    const float mine = r ? fb : fa;
+    const unsigned long long winners = __ballot(ok);
+    const uint32_t w = (uint32_t)__builtin_ctzll(winners | (1ull << 63));
+    mass = lane_value(m, w);
+    picked = lane_value(mine, w);
+    return 16u * w + (uint32_t)__builtin_amdgcn_readlane((int)in, (int)w);
 }
 
 // Number of round trips and the levels taken by each for a tree of `depth` levels.

@@ -285,19 +285,19 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
             const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
             __builtin_amdgcn_sched_barrier(0);
             mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
-            node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, mass, picked);
+            node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
             for (int i = 1; i < ngroups; ++i) {
                 g = group_levels(depth, ngroups, i);  // >= 5 once there are two groups
                 group_request(sum, node, g, lane, r0, r1, r2, r3);
                 __builtin_amdgcn_sched_barrier(0);
-                node = (node << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, mass, picked);
+                node = (node << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
             }
         } else {
             // one or two leaves
             const float total = sum[1];
             mass = stratum_mass(a, total, k);
             picked = total;
-            node = (1u << g) + (g ? group_walk(group_load_tiny(sum, 1u, g, lane), g, mass, picked) : 0u);
+            node = (1u << g) + (g ? group_walk(group_load_tiny(sum, 1u, g, lane), g, lane, mass, picked) : 0u);
         }
         if (lane == 0) {
             s_idx = (int64_t)node - a.leaves;
