@@ -203,6 +203,10 @@ def main():
     dev_ms = ev0.elapsed_time(ev1)
     flags = buf.check()
 
+    # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this very command, scaled by what the
+    # same counters read for the ring-append copy kernel (profiles/k_per_sample_wide_config3_*.md); only valid for
+    # the default workload and library defaults.
+    traffic = 33.85e6 if (a.workload == "c3" and not a.capacity and not a.row_split and not a.sample_path) else None
     row_bytes = sum(buf._layout.bytes)
     algo_bytes = batch * (2 * row_bytes + 12)  # rows read + rows written + index (8) + weight (4)
     kern_s = dev_ms * 1e-3 / K
@@ -224,7 +228,7 @@ def main():
                    "alpha": 0.6, "beta": "0.4->1.0", "launch": "hip graph replay" if a.graph else "eager C-ABI calls",
                    "prefill_s": round(fill_s, 2), "device_flags": flags},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "k_per_sample_wide", "algorithmic_bytes_per_launch": algo_bytes,
                      "avg_launch_us": kern_s * 1e6},
     }

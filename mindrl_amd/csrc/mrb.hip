@@ -538,7 +538,9 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, 
     if (path == 1) {
         int split = (int)g_opt.row_split;
         if (split <= 0) {
-            split = (int)((max_units + 2 * kWG - 1) / (2 * kWG));  // about two granules per thread
+            // one pass of kInFlight granules per thread covers the widest field (measured best on
+            // 28 KB rows: 2 workgroups per row; more workgroups only repeat the tree walk)
+            split = (int)((max_units + kInFlight * kWG - 1) / (kInFlight * kWG));
             if (split < 1) split = 1;
             if (split > 16) split = 16;
         }

@@ -80,3 +80,32 @@ def test_field_layout():
         FieldLayout([(1,)] * 17, [np.float32] * 17)
     with pytest.raises(TypeError):
         as_torch_dtype("complex64")
+
+
+def test_kernels_use_no_scratch_memory(tmp_path):
+    """Register arrays that the compiler cannot keep in registers end up in scratch
+    (or LDS) and slow the sample kernel by 2x; the device assembly's metadata must show
+    private_segment_fixed_size 0 for every kernel and the expected LDS sizes."""
+    import subprocess
+    from mindrl_amd import build
+    out = tmp_path / "mrb.s"
+    flags = [f for f in build.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    res = subprocess.run(["/opt/rocm/bin/hipcc"] + flags + ["--cuda-device-only", "-S", "-o", str(out),
+                          os.path.join(build.CSRC, "mrb.hip")], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                         text=True)
+    assert res.returncode == 0, res.stdout
+    text = out.read_text()
+    kernels = {}
+    for block in text.split("  - .agpr_count:")[1:]:
+        name = re.search(r"\.name:\s+(\S+)", block).group(1)
+        kernels[name] = (int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", block).group(1)),
+                         int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
+                         int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
+    assert len(kernels) == 9, sorted(kernels)
+    for name, (scratch, lds, vgprs) in kernels.items():
+        assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
+        assert vgprs <= 128, (name, vgprs)
+        if "k_per_sample_wide" in name:
+            assert lds <= 1024, (name, lds)
+        if "k_tree_top" in name:
+            assert lds == 65536, (name, lds)
