@@ -43,7 +43,7 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=2000)
     p.add_argument("--warmup", type=int, default=200)
-    p.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    p.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2"])
     p.add_argument("--capacity", type=int, default=0, help="override the workload's capacity (for quick trials)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--graph", action="store_true", help="replay the timed steps as one captured HIP graph")
@@ -124,6 +124,89 @@ def cpu_baseline(workload, shapes, np_dtypes, batch, seed):
     }
 
 
+def bench_uniform(a):
+    """Config 2: SAC MuJoCo-shaped UniformReplayBuffer, capacity 1,000,000, 165 B rows; insert in chunks of
+    1000, then sample batch 256 with seeded uniform integer indices drawn on the host."""
+    import torch
+
+    from mindrl_amd import _lib
+    from mindrl_amd.core import UniformReplayBuffer
+    from mindrl_amd.core._rows import pointers
+
+    capacity, batch = (a.capacity or 1_000_000), 256
+    shapes, np_dtypes = [(17,), (6,), (1,), (17,), (1,)], ["float32", "float32", "float32", "float32", "bool"]
+    buf = UniformReplayBuffer(batch, capacity, shapes, [getattr(torch, d) for d in np_dtypes], seed=1002)
+    gen = torch.Generator(device="cuda").manual_seed(1002)
+    chunk = 1000
+    src = [torch.randn((chunk,) + s, device="cuda", generator=gen) if d != "bool"
+           else torch.rand((chunk,) + s, device="cuda", generator=gen) < 0.01 for s, d in zip(shapes, np_dtypes)]
+    L = _lib.lib()
+    sp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sptr = pointers(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(capacity // chunk):
+        _lib.check(L.mrb_urb_append(buf._h, sptr, chunk, sp))
+    torch.cuda.synchronize()
+    ins_s = time.perf_counter() - t0
+    K, W = a.steps, a.warmup
+    rng = np.random.default_rng(1002)
+    idx = torch.from_numpy(rng.integers(0, capacity, (K + W, batch))).cuda()
+    out = buf._layout.empty(batch, buf._dev)
+    optr = pointers(out)
+    ibase = idx.data_ptr()
+    for i in range(W):
+        _lib.check(L.mrb_urb_gather(buf._h, ibase + i * batch * 8, batch, optr, sp))
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for i in range(W, W + K):
+        L.mrb_urb_gather(buf._h, ibase + i * batch * 8, batch, optr, sp)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    buf.check()
+    row_bytes = sum(buf._layout.bytes)
+    algo = batch * (2 * row_bytes + 8)
+    kern_s = ev0.elapsed_time(ev1) * 1e-3 / K
+    res = {
+        "metric": "sampled transitions/sec (sample+gather), uniform buffer at cap 1M", "value": K * batch / wall,
+        "unit": "transitions/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": wall * 1e3 / K,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "config 2: SAC-shaped UniformReplayBuffer, capacity %d, 165 B rows, batch 256, "
+                               "host-drawn indices" % capacity, "row_bytes": row_bytes},
+        "roofline": {"bound": "hbm", "achieved": algo / kern_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "k_rows_gather",
+                     "algorithmic_bytes_per_launch": algo, "avg_launch_us": kern_s * 1e6},
+        "extras": {"inserts_per_s": capacity / ins_s, "insert_chunk": chunk},
+        "cpu_baseline": None,
+    }
+    if not a.no_cpu_baseline:
+        from oracle import orc
+        cap_c = min(capacity, 1 << 20)
+        o = orc.OracleUniform(cap_c, shapes, np_dtypes, seed=1002)
+        rows = [np.asarray(t.cpu().numpy()) for t in src]
+        for _ in range(cap_c // chunk):
+            o.append(rows, chunk)
+        Lo = orc.lib()
+        dst = o._dst(batch)
+        dptr = orc._ptr_array(dst)
+        hidx = rng.integers(0, o.count, (256, batch))
+        calls, t_end = 0, time.perf_counter() + 5.0
+        t0 = time.perf_counter()
+        while time.perf_counter() < t_end:
+            Lo.orc_urb_gather(o.h, hidx[calls % 256].ctypes.data, batch, dptr)
+            calls += 1
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": calls * batch / dt, "unit": "transitions/s", "cores": 1, "kind": "port",
+                               "sample": "%d gather calls of batch %d in %.1f s, capacity %d, 1 thread" % (
+                                   calls, batch, dt, cap_c)}
+    buf.destroy()
+    print(json.dumps(res))
+    return 0
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -138,6 +221,8 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
     torch.cuda.set_device(0)
+    if a.workload == "c2":
+        return bench_uniform(a)
     capacity, batch, shapes, np_dtypes, upd_n, ins_n, desc = WORKLOADS[a.workload]
     _lib.set_option("row_split", a.row_split)
     _lib.set_option("sample_path", a.sample_path)

@@ -452,16 +452,47 @@ __global__ __launch_bounds__(kWG) void k_per_sample_lds(SampleArgs a, IoTable t,
                 node = 2 * node + 1;
             }
         }
-        for (; d < a.depth; ++d) {
-            const float left = a.sum[2 * node];
-            if (mass <= left) {
-                node = 2 * node;
+        // Below the staged levels every dependent load brings three levels at once: the 8
+        // great-grandchildren of `node` are 32 contiguous, aligned bytes; the two levels
+        // between are rebuilt with the additions the tree was built with.
+        float picked = a.depth <= lds_levels ? s_top[node] : 0.0f;
+        for (; d + 3 <= a.depth; d += 3) {
+            const float4* src = reinterpret_cast<const float4*>(a.sum + ((uint64_t)node << 3));
+            const float4 lo = src[0], hi = src[1];
+            const float a0 = lo.x + lo.y, a1 = lo.z + lo.w, a2 = hi.x + hi.y;
+            const float b0 = a0 + a1;
+            uint32_t p = 0;
+            if (!(mass <= b0)) {
+                mass -= b0;
+                p = 4;
+            }
+            const float left1 = p ? a2 : a0;
+            if (!(mass <= left1)) {
+                mass -= left1;
+                p += 2;
+            }
+            const float n0 = p == 0 ? lo.x : p == 2 ? lo.z : p == 4 ? hi.x : hi.z;
+            const float n1 = p == 0 ? lo.y : p == 2 ? lo.w : p == 4 ? hi.y : hi.w;
+            if (!(mass <= n0)) {
+                mass -= n0;
+                p += 1;
+                picked = n1;
             } else {
-                mass -= left;
+                picked = n0;
+            }
+            node = (node << 3) + p;
+        }
+        for (; d < a.depth; ++d) {
+            const float2 pair = *reinterpret_cast<const float2*>(a.sum + 2 * (uint64_t)node);
+            if (mass <= pair.x) {
+                node = 2 * node;
+                picked = pair.x;
+            } else {
+                mass -= pair.x;
                 node = 2 * node + 1;
+                picked = pair.y;
             }
         }
-        const float picked = a.depth <= lds_levels ? s_top[node] : a.sum[node];
         const int64_t idx = (int64_t)node - a.leaves;
         a.out_idx[k] = idx;
         a.out_w[k] = is_weight(picked, total, a.mn[1], (float)a.size, a.beta);
