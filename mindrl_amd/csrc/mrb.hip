@@ -150,8 +150,11 @@ struct Per {
     unsigned long long* stamp = nullptr;
     float* maxp = nullptr;
     uint32_t* err = nullptr;
-    uint32_t* dirty[4] = {};
+    uint32_t* done = nullptr;
+    uint32_t* dirty[kMaxRounds] = {};
     int nrounds = 0;
+    int lo[kMaxRounds] = {};
+    int g[kMaxRounds] = {};
     int top_depth = 0;
     uint64_t epoch = 0;
     uint64_t seed = 0, calls = 0;
@@ -161,6 +164,7 @@ struct Per {
         if (stamp) (void)hipFree(stamp);
         if (maxp) (void)hipFree(maxp);
         if (err) (void)hipFree(err);
+        if (done) (void)hipFree(done);
         for (auto* d : dirty)
             if (d) (void)hipFree(d);
     }
@@ -201,18 +205,18 @@ int read_and_clear_flags(uint32_t* d_err, uint32_t* flags, hipStream_t s) {
     return MRB_OK;
 }
 
-// Rebuilds every internal node above the leaves marked dirty in this epoch.
-int tree_rebuild(Per& b, hipStream_t s) {
-    const uint32_t epoch32 = (uint32_t)b.epoch;
-    for (int r = 0; r < b.nrounds; ++r) {
-        const int lo = b.depth - kRoundLevels * r;
-        const uint32_t nblocks = (1u << lo) / kBlockNodes;
-        hipLaunchKernelGGL(k_tree_round, dim3((nblocks + 3) / 4), dim3(kWG), 0, s, b.sum, b.mn, lo, b.dirty[r], epoch32);
-        LAUNCH_CHECK("k_tree_round");
+// Rebuilds the tree above the leaves that `a` writes: one launch per round, the last of which
+// also rebuilds the top; a tree of <= 12 levels is one single-workgroup launch.
+int tree_rebuild(Per& b, const UpdateArgs& a, hipStream_t s) {
+    if (b.nrounds == 0) {
+        hipLaunchKernelGGL(k_tree_update, dim3(1), dim3(kWG), 0, s, a, -1);
+        LAUNCH_CHECK("k_tree_update");
+        return MRB_OK;
     }
-    if (b.top_depth > 0) {
-        hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, b.sum, b.mn, b.top_depth);
-        LAUNCH_CHECK("k_tree_top");
+    for (int r = 0; r < b.nrounds; ++r) {
+        const uint32_t tiles = (1u << b.lo[r]) / kBlockNodes;
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r);
+        LAUNCH_CHECK("k_tree_update");
     }
     return MRB_OK;
 }
@@ -224,10 +228,8 @@ int next_epoch(Per& b, hipStream_t s) {
     b.epoch += 1;
     if ((uint32_t)b.epoch == 0) {
         HIP_TRY(hipMemsetAsync(b.stamp, 0, sizeof(unsigned long long) * (size_t)b.leaves, s));
-        for (int r = 0; r < b.nrounds; ++r) {
-            const size_t nblocks = ((size_t)1 << (b.depth - kRoundLevels * r)) / kBlockNodes;
-            HIP_TRY(hipMemsetAsync(b.dirty[r], 0, sizeof(uint32_t) * nblocks, s));
-        }
+        for (int r = 0; r < b.nrounds; ++r)
+            HIP_TRY(hipMemsetAsync(b.dirty[r], 0, sizeof(uint32_t) * ((size_t)1 << (b.lo[r] - b.g[r])), s));
         b.epoch += 1;
     }
     return MRB_OK;
@@ -237,6 +239,7 @@ UpdateArgs update_args(Per& b) {
     UpdateArgs a{};
     a.capacity = b.rows.capacity;
     a.leaves = b.leaves;
+    a.depth = b.depth;
     a.alpha = b.alpha;
     a.epoch = (uint32_t)b.epoch;
     a.stamp = b.stamp;
@@ -244,8 +247,14 @@ UpdateArgs update_args(Per& b) {
     a.mn = b.mn;
     a.maxp = b.maxp;
     a.err = b.err;
-    for (int r = 0; r < 4; ++r) a.dirty[r] = b.dirty[r];
+    a.done = b.done;
     a.nrounds = b.nrounds;
+    for (int r = 0; r < kMaxRounds; ++r) {
+        a.dirty[r] = b.dirty[r];
+        a.lo[r] = b.lo[r];
+        a.g[r] = b.g[r];
+    }
+    a.top_depth = b.top_depth;
     return a;
 }
 
@@ -418,8 +427,20 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     }
     b->alpha = alpha;
     b->seed = seed;
-    b->nrounds = b->depth > kTopMaxDepth ? (b->depth - kTopMaxDepth + kRoundLevels - 1) / kRoundLevels : 0;
-    b->top_depth = b->depth - kRoundLevels * b->nrounds;
+    // Rebuild plan: the top (<= 12 levels) belongs to the last workgroup of the last round; the levels
+    // below it are split as evenly as possible into rounds of 2..8 levels.
+    b->top_depth = b->depth < kTopMaxDepth ? b->depth : kTopMaxDepth;
+    int rest = b->depth - b->top_depth;
+    if (rest == 1) {  // a round needs at least two levels (a lane's four nodes must share a block)
+        rest = 2;
+        b->top_depth -= 1;
+    }
+    b->nrounds = (rest + kRoundLevels - 1) / kRoundLevels;
+    for (int r = 0, lo = b->depth; r < b->nrounds; ++r) {
+        b->lo[r] = lo;
+        b->g[r] = rest / b->nrounds + (r < rest % b->nrounds ? 1 : 0);
+        lo -= b->g[r];
+    }
     const size_t nodes = 2 * (size_t)b->leaves;
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->sum), nodes * sizeof(float)));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->mn), nodes * sizeof(float)));
@@ -429,8 +450,10 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     HIP_TRY(hipMemset(b->sum, 0, nodes * sizeof(float)));
     HIP_TRY(hipMemset(b->stamp, 0, (size_t)b->leaves * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(b->err, 0, 16));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->done), 16));
+    HIP_TRY(hipMemset(b->done, 0, 16));
     for (int r = 0; r < b->nrounds; ++r) {
-        const size_t nblocks = ((size_t)1 << (b->depth - kRoundLevels * r)) / kBlockNodes;
+        const size_t nblocks = (size_t)1 << (b->lo[r] - b->g[r]);
         HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->dirty[r]), nblocks * sizeof(uint32_t)));
         HIP_TRY(hipMemset(b->dirty[r], 0, nblocks * sizeof(uint32_t)));
     }
@@ -459,24 +482,17 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     rc = next_epoch(*b, s);
     if (rc) return rc;
     UpdateArgs a = update_args(*b);
-    a.first_slot = first;
-    a.n = n;
     if (opt_priorities) {
         // push-then-update: the running max sees every priority of the call, surviving or not
         a.priorities = opt_priorities;
-        a.stamp = nullptr;
         a.n = nrows;
-        a.first_slot = b->pushes % cap;
         hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)nrows)), dim3(kWG), 0, s, a);
         LAUNCH_CHECK("k_update_stamp");
         a.priorities = opt_priorities + skip;
-        a.n = n;
-        a.first_slot = first;
-        a.stamp = b->stamp;
     }
-    hipLaunchKernelGGL(k_update_leaves, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
-    LAUNCH_CHECK("k_update_leaves");
-    rc = tree_rebuild(*b, s);
+    a.first_slot = first;
+    a.n = n;
+    rc = tree_rebuild(*b, a, s);
     if (rc) return rc;
     b->pushes += nrows;
     b->size = b->size + nrows < cap ? b->size + nrows : cap;
@@ -497,9 +513,7 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     a.n = n;
     hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
     LAUNCH_CHECK("k_update_stamp");
-    hipLaunchKernelGGL(k_update_leaves, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
-    LAUNCH_CHECK("k_update_leaves");
-    return tree_rebuild(*b, s);
+    return tree_rebuild(*b, a, s);
 }
 
 int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, int64_t* out_indices,

@@ -11,9 +11,9 @@
 namespace mrb {
 
 constexpr int kWG = 256;          // threads per workgroup of the row and sample kernels
-constexpr int kRoundLevels = 8;   // tree levels rebuilt by one pass of k_tree_round
-constexpr int kBlockNodes = 256;  // nodes per wave in k_tree_round (float4 per lane)
-constexpr int kTopMaxDepth = 12;  // deepest level k_tree_top starts from (4096 nodes)
+constexpr int kRoundLevels = 8;   // most tree levels rebuilt by one round of k_tree_update
+constexpr int kBlockNodes = 256;  // nodes per wave tile in k_tree_update (float4 per lane)
+constexpr int kTopMaxDepth = 12;  // deepest level the last workgroup's top rebuild starts from (4096 nodes)
 
 // Per-call table of the fields of a row, passed to kernels by value.
 // `store` is the buffer's [capacity, row_bytes] matrix, `io` the caller's
@@ -517,63 +517,75 @@ __global__ __launch_bounds__(kWG) void k_per_sample_lds(SampleArgs a, IoTable t,
 }
 
 // ---------------------------------------------------------------------------
-// update_priorities, pass 1 (PriorityReplayBufferUpdate,
-// mindspore_rl/core/priority_replay_buffer.py:71-73,108-120): every valid
-// entry j raises stamp[index_j] to (epoch << 32 | j) with an integer max, so
-// after the pass the stamp names the LAST entry of this call that targets the
-// leaf (last write wins). The running max priority takes an integer max of the
-// float bits (order-preserving for non-negative floats). No float is summed
-// atomically anywhere.
-//   indices == NULL: entry j targets slot (first_slot + j) mod capacity
-//   stamp   == NULL: only the running max is updated
+// Tree updates (PriorityReplayBufferUpdate and the tree half of
+// PriorityReplayBufferPush, mindspore_rl/core/priority_replay_buffer.py:67-73,
+// 78-90,108-120).
+//
+// The reference writes one leaf at a time and walks to the root after each.
+// Here a call is two or three launches:
+//   k_update_stamp   every valid entry j raises stamp[index_j] to
+//                    (epoch << 32 | j) with an INTEGER max, so the stamp names
+//                    the last entry of the call that targets the leaf (last
+//                    write wins), marks the leaf's block dirty, and folds
+//                    p_j^alpha into the running max (integer max of the float
+//                    bits, order-preserving for non-negative floats).
+//   k_tree_update    level-synchronous rebuild, one launch per round of <= 8
+//                    levels. A wave owns a tile of 256 consecutive nodes; the
+//                    lowest round first replaces the leaves named by the
+//                    stamps (or, for a push, the leaves of the pushed slot
+//                    range). Only dirty blocks load or store. The workgroup
+//                    that finishes the last round last also rebuilds the top
+//                    (<= 12 levels), so no separate launch is needed for it.
+// Every parent is written as the single rounded sum / min of its two final
+// children, which is what a leaf-to-root walk after the last write leaves
+// behind; recomputing a clean node reproduces its bits. No float is ever
+// accumulated atomically.
 // ---------------------------------------------------------------------------
+constexpr int kMaxRounds = 3;
+
 struct UpdateArgs {
-    const int64_t* indices;
-    const float* priorities;  // NULL: every entry takes the running max priority as it is
+    // entries
+    const int64_t* indices;   // NULL: entry j targets slot (first_slot + j) mod capacity
+    const float* priorities;  // NULL: the targeted leaves take the running max priority as it is
     int64_t n;
-    int64_t capacity;
     int64_t first_slot;
+    // buffer
+    int64_t capacity;
     int64_t leaves;
+    int depth;
     float alpha;
     uint32_t epoch;
     unsigned long long* stamp;  // [leaves]
     float* sum;
     float* mn;
-    float* maxp;    // running max priority (device scalar)
+    float* maxp;  // running max priority (device scalar)
     uint32_t* err;
-    uint32_t* dirty[4];  // per rebuild round: one word per 256-node block
+    uint32_t* done;  // workgroups that have finished the current launch (reset by the last one)
+    // rebuild plan: round r starts at depth lo[r] and rebuilds g[r] levels; the top starts at top_depth
     int nrounds;
+    int lo[kMaxRounds];
+    int g[kMaxRounds];
+    int top_depth;
+    uint32_t* dirty[kMaxRounds];  // per round: one epoch word per block of 1 << g[r] nodes at depth lo[r]
 };
 
-__device__ __forceinline__ bool update_entry(const UpdateArgs& a, int64_t j, int64_t& idx, float& q, bool report) {
-    if (a.indices) {
-        idx = a.indices[j];
-        if (idx < 0 || idx >= a.capacity) {
-            if (report) atomicOr(a.err, MRB_DERR_INDEX);
-            return false;
-        }
-    } else {
-        idx = a.first_slot + j;
-        if (idx >= a.capacity) idx -= a.capacity;
-    }
-    const float p = a.priorities[j];
-    if (!(p >= 0.0f) || p > 3.0e38f) {
-        if (report) atomicOr(a.err, MRB_DERR_PRIORITY);
-        return false;
-    }
-    q = powf_det(p, a.alpha);
-    return true;
-}
+__device__ __forceinline__ bool valid_priority(float p) { return p >= 0.0f && p <= 3.0e38f; }
 
 __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
     const int64_t j = (int64_t)blockIdx.x * kWG + threadIdx.x;
     float q = 0.0f;
     if (j < a.n) {
-        int64_t idx;
-        float qq;
-        if (update_entry(a, j, idx, qq, true)) {
-            q = qq;
-            if (a.stamp) atomicMax(&a.stamp[idx], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
+        const float p = a.priorities[j];
+        int64_t idx = a.indices ? a.indices[j] : 0;
+        const bool idx_ok = !a.indices || (idx >= 0 && idx < a.capacity);
+        if (!idx_ok) atomicOr(a.err, MRB_DERR_INDEX);
+        if (!valid_priority(p)) atomicOr(a.err, MRB_DERR_PRIORITY);
+        if (idx_ok && valid_priority(p)) {
+            q = powf_det(p, a.alpha);
+            if (a.indices) {
+                atomicMax(&a.stamp[idx], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
+                if (a.nrounds) a.dirty[0][idx >> a.g[0]] = a.epoch;
+            }
         }
     }
     // wave max, then one integer atomic per wave
@@ -581,107 +593,171 @@ __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
     if ((threadIdx.x & 63) == 0 && q > 0.0f) atomicMax(reinterpret_cast<unsigned int*>(a.maxp), __float_as_uint(q));
 }
 
-__device__ __forceinline__ void mark_dirty(const UpdateArgs& a, int64_t idx) {
-    for (int r = 0; r < a.nrounds; ++r) a.dirty[r][idx >> (kRoundLevels * (r + 1))] = a.epoch;
-}
-
-// Pass 2: the winning entry of each leaf writes it (sum and min trees) and
-// marks the 256-node blocks above it dirty for the rebuild rounds.
-//   indices given:            winner = entry named by the stamp
-//   indices NULL, priorities: slots are distinct, every entry writes
-//   indices NULL, no priorities: every slot takes the running max priority
-__global__ __launch_bounds__(kWG) void k_update_leaves(UpdateArgs a) {
-    const int64_t j = (int64_t)blockIdx.x * kWG + threadIdx.x;
-    if (j >= a.n) return;
-    int64_t idx;
-    float q;
-    if (a.priorities && a.indices) {
-        if (!update_entry(a, j, idx, q, false)) return;
-        if (a.stamp[idx] != (((unsigned long long)a.epoch << 32) | (unsigned long long)j)) return;
-    } else if (a.priorities) {
-        // freshly pushed slot: an invalid priority leaves it at the running max, as a plain push would
-        if (!update_entry(a, j, idx, q, false)) q = *a.maxp;
+// New value of leaf `leaf`, if this call writes it.
+//   indices given:  the entry named by the stamp
+//   range + priorities: entry (leaf - first_slot) mod capacity; an invalid priority leaves the
+//                   fresh slot at the running max, as a plain push would
+//   range only:     the running max priority
+__device__ __forceinline__ bool leaf_value(const UpdateArgs& a, int64_t leaf, float& q) {
+    if (a.indices) {
+        const unsigned long long st = a.stamp[leaf];
+        if ((uint32_t)(st >> 32) != a.epoch) return false;
+        q = powf_det(a.priorities[(uint32_t)st], a.alpha);
+        return true;
+    }
+    if (leaf >= a.capacity) return false;
+    int64_t j = leaf - a.first_slot;
+    if (j < 0) j += a.capacity;
+    if (j >= a.n) return false;
+    if (a.priorities) {
+        const float p = a.priorities[j];
+        q = valid_priority(p) ? powf_det(p, a.alpha) : *a.maxp;
     } else {
-        idx = a.first_slot + j;
-        if (idx >= a.capacity) idx -= a.capacity;
         q = *a.maxp;
     }
-    a.sum[a.leaves + idx] = q;
-    a.mn[a.leaves + idx] = q;
-    mark_dirty(a, idx);
+    return true;
 }
 
-// ---------------------------------------------------------------------------
-// Rebuild round: one wave per block of 256 consecutive nodes at depth
-// `lo_depth`. A block whose dirty word carries this call's epoch recomputes
-// the 8 levels above it from those 256 nodes (float4 per lane, then wave
-// shuffles), each parent as the single rounded sum / min of its two children
-// — the same operation, on the same operands, as a leaf-to-root walk performs.
-// Recomputing a clean node reproduces its bits, so only values that a
-// sequential update would have changed change.
-// ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kWG) void k_tree_round(float* __restrict__ sum, float* __restrict__ mn, int lo_depth,
-                                                    const uint32_t* __restrict__ dirty, uint32_t epoch) {
-    const uint32_t block = blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
-    const uint32_t nblocks = (1u << lo_depth) / kBlockNodes;
-    if (block >= nblocks) return;
-    if (dirty[block] != epoch) return;
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t first = (1u << lo_depth) + block * kBlockNodes;  // heap index of the block's first node
-#pragma unroll
-    for (int which = 0; which < 2; ++which) {
-        float* tree = which ? mn : sum;
-        const float4 v = *reinterpret_cast<const float4*>(tree + first + 4 * lane);
-        float a0, a1, c;
-        if (which) {
-            a0 = fminf(v.x, v.y);
-            a1 = fminf(v.z, v.w);
-            c = fminf(a0, a1);
-        } else {
-            a0 = v.x + v.y;
-            a1 = v.z + v.w;
-            c = a0 + a1;
+// Does the pushed slot range [first_slot, first_slot + n) mod capacity meet leaves [lo, hi)?
+__device__ __forceinline__ bool range_meets(const UpdateArgs& a, int64_t lo, int64_t hi) {
+    const int64_t end = a.first_slot + a.n;
+    if (lo < (end < a.capacity ? end : a.capacity) && hi > a.first_slot) return true;
+    return end > a.capacity && lo < end - a.capacity;
+}
+
+// One wave rebuilds `g` levels above a tile of up to 256 consecutive nodes at depth `lo`.
+//   tile       index of the tile within the level
+//   sparse     skip clean blocks (rounds; g >= 2 there, so a lane's four nodes share a block):
+//              a block is dirty if its word in dirty_in carries this call's epoch or, at the
+//              leaf level of a push (dirty_in NULL), if it meets the pushed slot range
+//   dirty_out  next round's words, marked for every block rebuilt here (may be NULL)
+// Lanes of clean blocks neither load nor store; the shuffles of a dirty block only mix
+// lanes of that block.
+__device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, uint32_t tile, bool sparse,
+                                           const uint32_t* __restrict__ dirty_in, uint32_t* __restrict__ dirty_out,
+                                           int g_next, uint32_t lane) {
+    const uint32_t level_nodes = 1u << lo;
+    const bool leaf_level = lo == a.depth;
+    if (level_nodes < 4) {
+        // one or two nodes: scalar, lane 0
+        if (lane == 0) {
+            float s0 = a.sum[level_nodes], m0 = a.mn[level_nodes], q;
+            if (leaf_level && leaf_value(a, 0, q)) {
+                s0 = m0 = q;
+                a.sum[level_nodes] = q;
+                a.mn[level_nodes] = q;
+            }
+            if (level_nodes == 2) {
+                float s1 = a.sum[3], m1 = a.mn[3];
+                if (leaf_level && leaf_value(a, 1, q)) {
+                    s1 = m1 = q;
+                    a.sum[3] = q;
+                    a.mn[3] = q;
+                }
+                if (g >= 1) {
+                    a.sum[1] = s0 + s1;
+                    a.mn[1] = fminf(m0, m1);
+                }
+            }
         }
-        // level lo_depth-1: 128 nodes, two per lane; level lo_depth-2: 64 nodes, one per lane
-        *reinterpret_cast<float2*>(tree + (first >> 1) + 2 * lane) = make_float2(a0, a1);
-        tree[(first >> 2) + lane] = c;
-        // levels lo_depth-3 .. lo_depth-8: 32, 16, 8, 4, 2, 1 nodes
+        return;
+    }
+    const uint32_t tile_nodes = level_nodes < (uint32_t)kBlockNodes ? level_nodes : (uint32_t)kBlockNodes;
+    const uint32_t off = tile * kBlockNodes + 4 * lane;  // this lane's first node within the level
+    const uint32_t first = level_nodes + tile * kBlockNodes;  // heap index of the tile's first node
+    bool active = 4 * lane < tile_nodes;
+    if (active && sparse) {
+        if (dirty_in) {
+            active = dirty_in[off >> g] == a.epoch;
+        } else if (leaf_level && !a.indices) {
+            const int64_t b0 = (int64_t)(off >> g) << g;
+            active = range_meets(a, b0, b0 + (1ll << g));
+        }
+    }
+    float4 vs = make_float4(0.f, 0.f, 0.f, 0.f), vm = vs;
+    if (active) {
+        vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * lane);
+        vm = *reinterpret_cast<const float4*>(a.mn + first + 4 * lane);
+        if (leaf_level) {
+            float q;
+            bool wrote = false;
+            if (leaf_value(a, off + 0, q)) { vs.x = vm.x = q; wrote = true; }
+            if (leaf_value(a, off + 1, q)) { vs.y = vm.y = q; wrote = true; }
+            if (leaf_value(a, off + 2, q)) { vs.z = vm.z = q; wrote = true; }
+            if (leaf_value(a, off + 3, q)) { vs.w = vm.w = q; wrote = true; }
+            if (wrote) {
+                *reinterpret_cast<float4*>(a.sum + first + 4 * lane) = vs;
+                *reinterpret_cast<float4*>(a.mn + first + 4 * lane) = vm;
+            }
+        }
+        if (dirty_out && ((off & ((1u << g) - 1)) == 0)) dirty_out[(off >> g) >> g_next] = a.epoch;
+    }
+    // level lo-1: two nodes per lane; level lo-2: one node per lane
+    const float s0 = vs.x + vs.y, s1 = vs.z + vs.w;
+    const float m0 = fminf(vm.x, vm.y), m1 = fminf(vm.z, vm.w);
+    float cs = s0 + s1, cm = fminf(m0, m1);
+    if (active && g >= 1) {
+        *reinterpret_cast<float2*>(a.sum + (first >> 1) + 2 * lane) = make_float2(s0, s1);
+        *reinterpret_cast<float2*>(a.mn + (first >> 1) + 2 * lane) = make_float2(m0, m1);
+    }
+    if (active && g >= 2) {
+        a.sum[(first >> 2) + lane] = cs;
+        a.mn[(first >> 2) + lane] = cm;
+    }
+    // levels lo-3 .. lo-8: 32, 16, 8, 4, 2, 1 nodes per full tile
 #pragma unroll
-        for (int s = 0; s < 6; ++s) {
-            const float o = __shfl_xor(c, 1 << s);
-            c = which ? fminf(c, o) : c + o;
-            if ((lane & ((2u << s) - 1)) == 0) tree[(first >> (3 + s)) + (lane >> (s + 1))] = c;
+    for (int s = 0; s < 6; ++s) {
+        cs = cs + __shfl_xor(cs, 1 << s);
+        cm = fminf(cm, __shfl_xor(cm, 1 << s));
+        if (active && g >= 3 + s && (lane & ((2u << s) - 1)) == 0) {
+            a.sum[(first >> (3 + s)) + (lane >> (s + 1))] = cs;
+            a.mn[(first >> (3 + s)) + (lane >> (s + 1))] = cm;
         }
     }
 }
 
-// ---------------------------------------------------------------------------
-// Top of the tree: one workgroup loads the 2^top_depth (<= 4096) nodes at
-// depth `top_depth` into LDS, rebuilds every level above them and writes
-// nodes [1, 2^top_depth) back.
-// ---------------------------------------------------------------------------
-constexpr int kTopWG = 1024;
-__global__ __launch_bounds__(kTopWG) void k_tree_top(float* __restrict__ sum, float* __restrict__ mn, int top_depth) {
-    __shared__ float s_sum[2 << kTopMaxDepth];
-    __shared__ float s_min[2 << kTopMaxDepth];
-    const uint32_t n = 1u << top_depth;
-    for (uint32_t i = n + threadIdx.x; i < 2 * n; i += kTopWG) {
-        s_sum[i] = sum[i];
-        s_min[i] = mn[i];
+// Rebuilds everything above depth `top` (<= 12) with one workgroup of 256 threads:
+// first up to 8 levels over the 1..16 tiles of that depth, then the rest in one tile.
+__device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g1 = top < kRoundLevels ? top : kRoundLevels;
+    const uint32_t tiles = (1u << top) <= (uint32_t)kBlockNodes ? 1u : (1u << top) / kBlockNodes;
+    for (uint32_t t = wave; t < tiles; t += kWG / 64) tile_round(a, top, g1, t, false, nullptr, nullptr, 0, lane);
+    if (top > g1) {
+        __threadfence();  // the tiles' parents, written by other waves, are read below
+        __syncthreads();
+        if (wave == 0) tile_round(a, top - g1, top - g1, 0, false, nullptr, nullptr, 0, lane);
+    }
+}
+
+// round >= 0: one wave per tile of round `round`; round < 0: a tree of <= 12 levels, one workgroup.
+__global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round) {
+    if (round < 0) {
+        top_rebuild(a, a.depth);
+        return;
+    }
+    const uint32_t lane = threadIdx.x & 63;
+    const int lo = a.lo[round], g = a.g[round];
+    const uint32_t tile = blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
+    const bool last_round = round + 1 == a.nrounds;
+    if (tile < (1u << lo) / kBlockNodes)
+        tile_round(a, lo, g, tile, true, (round == 0 && !a.indices) ? nullptr : a.dirty[round],
+                   last_round ? nullptr : a.dirty[round + 1], last_round ? 0 : a.g[round + 1], lane);
+    if (!last_round) return;
+    // The workgroup that finishes last continues with the top of the tree. Its fence makes the
+    // other workgroups' stores (each fenced before the ticket was taken) visible to its loads.
+    __shared__ bool s_last;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t ticket = atomicAdd(a.done, 1u);
+        s_last = ticket == gridDim.x - 1;
+        if (s_last) *a.done = 0;
     }
     __syncthreads();
-    for (int d = top_depth - 1; d >= 0; --d) {
-        const uint32_t lo = 1u << d;
-        for (uint32_t i = lo + threadIdx.x; i < 2 * lo; i += kTopWG) {
-            s_sum[i] = s_sum[2 * i] + s_sum[2 * i + 1];
-            s_min[i] = fminf(s_min[2 * i], s_min[2 * i + 1]);
-        }
-        __syncthreads();
-    }
-    for (uint32_t i = 1 + threadIdx.x; i < n; i += kTopWG) {
-        sum[i] = s_sum[i];
-        mn[i] = s_min[i];
-    }
+    if (!s_last) return;
+    __threadfence();
+    top_rebuild(a, a.top_depth);
 }
 
 // Fills a float array with one value (tree initialisation: sums 0, mins FLT_MAX).
