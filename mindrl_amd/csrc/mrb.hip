@@ -150,7 +150,6 @@ struct Per {
     unsigned long long* stamp = nullptr;
     float* maxp = nullptr;
     uint32_t* err = nullptr;
-    uint32_t* done = nullptr;
     uint32_t* dirty[kMaxRounds] = {};
     int nrounds = 0;
     int lo[kMaxRounds] = {};
@@ -164,7 +163,6 @@ struct Per {
         if (stamp) (void)hipFree(stamp);
         if (maxp) (void)hipFree(maxp);
         if (err) (void)hipFree(err);
-        if (done) (void)hipFree(done);
         for (auto* d : dirty)
             if (d) (void)hipFree(d);
     }
@@ -205,19 +203,15 @@ int read_and_clear_flags(uint32_t* d_err, uint32_t* flags, hipStream_t s) {
     return MRB_OK;
 }
 
-// Rebuilds the tree above the leaves that `a` writes: one launch per round, the last of which
-// also rebuilds the top; a tree of <= 12 levels is one single-workgroup launch.
+// Rebuilds the tree above the leaves that `a` writes: one launch per round, then the top.
 int tree_rebuild(Per& b, const UpdateArgs& a, hipStream_t s) {
-    if (b.nrounds == 0) {
-        hipLaunchKernelGGL(k_tree_update, dim3(1), dim3(kWG), 0, s, a, -1);
-        LAUNCH_CHECK("k_tree_update");
-        return MRB_OK;
-    }
     for (int r = 0; r < b.nrounds; ++r) {
         const uint32_t tiles = (1u << b.lo[r]) / kBlockNodes;
         hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r);
         LAUNCH_CHECK("k_tree_update");
     }
+    hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a);
+    LAUNCH_CHECK("k_tree_top");
     return MRB_OK;
 }
 
@@ -247,7 +241,6 @@ UpdateArgs update_args(Per& b) {
     a.mn = b.mn;
     a.maxp = b.maxp;
     a.err = b.err;
-    a.done = b.done;
     a.nrounds = b.nrounds;
     for (int r = 0; r < kMaxRounds; ++r) {
         a.dirty[r] = b.dirty[r];
@@ -450,8 +443,6 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     HIP_TRY(hipMemset(b->sum, 0, nodes * sizeof(float)));
     HIP_TRY(hipMemset(b->stamp, 0, (size_t)b->leaves * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(b->err, 0, 16));
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->done), 16));
-    HIP_TRY(hipMemset(b->done, 0, 16));
     for (int r = 0; r < b->nrounds; ++r) {
         const size_t nblocks = (size_t)1 << (b->lo[r] - b->g[r]);
         HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->dirty[r]), nblocks * sizeof(uint32_t)));

@@ -533,9 +533,8 @@ __global__ __launch_bounds__(kWG) void k_per_sample_lds(SampleArgs a, IoTable t,
 //                    levels. A wave owns a tile of 256 consecutive nodes; the
 //                    lowest round first replaces the leaves named by the
 //                    stamps (or, for a push, the leaves of the pushed slot
-//                    range). Only dirty blocks load or store. The workgroup
-//                    that finishes the last round last also rebuilds the top
-//                    (<= 12 levels), so no separate launch is needed for it.
+//                    range). Only dirty blocks load or store.
+//   k_tree_top       one workgroup rebuilds the top (<= 12 levels).
 // Every parent is written as the single rounded sum / min of its two final
 // children, which is what a leaf-to-root walk after the last write leaves
 // behind; recomputing a clean node reproduces its bits. No float is ever
@@ -560,7 +559,6 @@ struct UpdateArgs {
     float* mn;
     float* maxp;  // running max priority (device scalar)
     uint32_t* err;
-    uint32_t* done;  // workgroups that have finished the current launch (reset by the last one)
     // rebuild plan: round r starts at depth lo[r] and rebuilds g[r] levels; the top starts at top_depth
     int nrounds;
     int lo[kMaxRounds];
@@ -716,26 +714,22 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
     }
 }
 
-// Rebuilds everything above depth `top` (<= 12) with one workgroup of 256 threads:
-// first up to 8 levels over the 1..16 tiles of that depth, then the rest in one tile.
+// Rebuilds everything above depth `top` (<= 12) with one workgroup: first up to 8 levels
+// over the 1..16 tiles of that depth (one wave each), then the rest in one tile.
 __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top) {
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int g1 = top < kRoundLevels ? top : kRoundLevels;
     const uint32_t tiles = (1u << top) <= (uint32_t)kBlockNodes ? 1u : (1u << top) / kBlockNodes;
-    for (uint32_t t = wave; t < tiles; t += kWG / 64) tile_round(a, top, g1, t, false, nullptr, nullptr, 0, lane);
+    for (uint32_t t = wave; t < tiles; t += nwaves) tile_round(a, top, g1, t, false, nullptr, nullptr, 0, lane);
     if (top > g1) {
-        __threadfence();  // the tiles' parents, written by other waves, are read below
+        __threadfence_block();  // the tiles' parents, written by other waves of this workgroup, are read below
         __syncthreads();
         if (wave == 0) tile_round(a, top - g1, top - g1, 0, false, nullptr, nullptr, 0, lane);
     }
 }
 
-// round >= 0: one wave per tile of round `round`; round < 0: a tree of <= 12 levels, one workgroup.
+// One wave per tile of round `round` (>= 0).
 __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round) {
-    if (round < 0) {
-        top_rebuild(a, a.depth);
-        return;
-    }
     const uint32_t lane = threadIdx.x & 63;
     const int lo = a.lo[round], g = a.g[round];
     const uint32_t tile = blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
@@ -743,22 +737,14 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round) {
     if (tile < (1u << lo) / kBlockNodes)
         tile_round(a, lo, g, tile, true, (round == 0 && !a.indices) ? nullptr : a.dirty[round],
                    last_round ? nullptr : a.dirty[round + 1], last_round ? 0 : a.g[round + 1], lane);
-    if (!last_round) return;
-    // The workgroup that finishes last continues with the top of the tree. Its fence makes the
-    // other workgroups' stores (each fenced before the ticket was taken) visible to its loads.
-    __shared__ bool s_last;
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const uint32_t ticket = atomicAdd(a.done, 1u);
-        s_last = ticket == gridDim.x - 1;
-        if (s_last) *a.done = 0;
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    top_rebuild(a, a.top_depth);
 }
+
+// The top of the tree (everything above a.top_depth; the whole tree, leaves included, when it has
+// no rounds), one workgroup. A separate launch rather than a continuation of the last round by
+// its last workgroup: publishing the rounds' stores to that workgroup needs an agent-scope
+// fence per workgroup, which on this multi-die part costs far more than a launch.
+constexpr int kTopWG = 1024;
+__global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a) { top_rebuild(a, a.top_depth); }
 
 // Fills a float array with one value (tree initialisation: sums 0, mins FLT_MAX).
 __global__ __launch_bounds__(kWG) void k_fill_f32(float* p, float v, uint64_t n) {
