@@ -296,6 +296,9 @@ def main():
     algo_bytes = batch * (2 * row_bytes + 12)  # rows read + rows written + index (8) + weight (4)
     kern_s = dev_ms * 1e-3 / K
     achieved = algo_bytes / kern_s / 1e9
+    # the library's own choice (mrb_per_sample): the LDS-top kernel for many narrow rows, else the wide-row kernel
+    lds_path = a.sample_path == 2 or (a.sample_path == 0 and batch >= 8192 and max(buf._layout.bytes) <= 256)
+    kernel_name = "k_per_sample_lds" if lds_path else "k_per_sample_wide"
     out = {
         "metric": "sampled transitions/sec (sample+IS+gather) at cap 1M; HBM GB/s vs peak",
         "value": K * batch / wall,
@@ -314,7 +317,7 @@ def main():
                    "prefill_s": round(fill_s, 2), "device_flags": flags},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "k_per_sample_wide", "algorithmic_bytes_per_launch": algo_bytes,
+                     "kernel": kernel_name, "algorithmic_bytes_per_launch": algo_bytes,
                      "avg_launch_us": kern_s * 1e6},
     }
 

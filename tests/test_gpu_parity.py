@@ -323,21 +323,22 @@ def test_config5_tree_descent_stress(mrb, orc):
     g.destroy()
 
 
-def test_config3_atari_shape_properties(mrb, orc):
-    """Config 3's row shape (u8[84,84,4] + next_idx i64 + action i32 + reward f32 + done
-    bool = 28 241 stored bytes) at capacity 2^17 (3.7 GB) instead of 10^6: the tree logic
-    does not depend on row content, so indices/weights/trees are compared with an oracle
-    holding only the four small fields, and the image field is checked against torch's own
-    index_select of the storage."""
+@pytest.mark.parametrize("cap", [1 << 17, 1_000_000])
+def test_config3_atari_shape_properties(mrb, orc, cap):
+    """Config 3's rows (u8[84,84,4] + next_idx i64 + action i32 + reward f32 + done bool =
+    28 241 stored bytes), batch 512, at capacity 2^17 and at the full 10^6 (28.2 GB in HBM).
+    The tree logic does not depend on row content, so indices, weights, the small fields and
+    both trees are compared with an oracle that holds only the four small fields, and the
+    image field is checked against torch's own index_select of the storage."""
     shapes = [(84, 84, 4), (1,), (1,), (1,), (1,)]
     dtypes = [np.uint8, np.int64, np.int32, np.float32, np.bool_]
     rng = np.random.default_rng(1003)
-    cap, batch = 1 << 17, 512
+    batch = 512
     g = mrb.PER(0.6, cap, batch, shapes, torch_types(dtypes), seed0=1003)
     c = orc.OraclePER(0.6, cap, shapes[1:], dtypes[1:], seed=1003)
     gen = torch.Generator(device="cuda").manual_seed(1003)
-    chunk = 4096
-    for start in range(0, cap, chunk):
+    for start in range(0, cap, 4096):
+        chunk = min(4096, cap - start)
         small = [np.arange(start + 1, start + chunk + 1, dtype=np.int64)[:, None] % cap,
                  rng.integers(0, 18, (chunk, 1)).astype(np.int32),
                  rng.integers(-1, 2, (chunk, 1)).astype(np.float32), rng.random((chunk, 1)) < 0.01]
