@@ -43,7 +43,7 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=2000)
     p.add_argument("--warmup", type=int, default=200)
-    p.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2"])
+    p.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2", "res"])
     p.add_argument("--capacity", type=int, default=0, help="override the workload's capacity (for quick trials)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--graph", action="store_true", help="replay the timed steps as one captured HIP graph")
@@ -207,6 +207,87 @@ def bench_uniform(a):
     return 0
 
 
+def bench_reservoir(a):
+    """ReservoirReplayBuffer, capacity 1,000,000, rows f32[17] + i32[6] (92 B): push batches of 4096 well past
+    the capacity (so every batch draws replacement slots and elects winners), then sample 256 per call."""
+    import torch
+
+    from mindrl_amd import _lib
+    from mindrl_amd.core import ReservoirReplayBuffer
+    from mindrl_amd.core._rows import pointers
+
+    capacity, batch, chunk = (a.capacity or 1_000_000), 256, 4096
+    shapes, np_dtypes = [(17,), (6,)], ["float32", "int32"]
+    buf = ReservoirReplayBuffer(capacity, batch, shapes, [torch.float32, torch.int32], seed1=1006)
+    src = [torch.randn(chunk, 17, device="cuda"), torch.randint(0, 9, (chunk, 6), dtype=torch.int32, device="cuda")]
+    L = _lib.lib()
+    sp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sptr = pointers(src)
+    for _ in range(capacity // chunk + 1):
+        _lib.check(L.mrb_res_push(buf._h, sptr, chunk, sp))
+    torch.cuda.synchronize()
+    n_push = 500
+    t0 = time.perf_counter()
+    for _ in range(n_push):
+        L.mrb_res_push(buf._h, sptr, chunk, sp)
+    torch.cuda.synchronize()
+    push_s = time.perf_counter() - t0
+    K, W = a.steps, a.warmup
+    out = buf._layout.empty(batch, buf._dev)
+    optr = pointers(out)
+    for _ in range(W):
+        _lib.check(L.mrb_res_sample(buf._h, batch, None, optr, sp))
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(K):
+        L.mrb_res_sample(buf._h, batch, None, optr, sp)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    row_bytes = sum(buf._layout.bytes)
+    algo = batch * 2 * row_bytes
+    kern_s = ev0.elapsed_time(ev1) * 1e-3 / K
+    res = {
+        "metric": "sampled transitions/sec, reservoir buffer at cap 1M", "value": K * batch / wall,
+        "unit": "transitions/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": wall * 1e3 / K,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "ReservoirReplayBuffer, capacity %d, 92 B rows, push 4096 per call past capacity, "
+                               "sample 256 per call" % capacity, "row_bytes": row_bytes},
+        "roofline": {"bound": "hbm", "achieved": algo / kern_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "k_rows_gather",
+                     "algorithmic_bytes_per_launch": algo, "avg_launch_us": kern_s * 1e6},
+        "extras": {"pushes_per_s": n_push * chunk / push_s, "push_chunk": chunk},
+        "cpu_baseline": None,
+    }
+    if not a.no_cpu_baseline:
+        from oracle import orc
+        o = orc.OracleReservoir(capacity, shapes, np_dtypes, seed=1006)
+        rows = [t.cpu().numpy() for t in src]
+        for _ in range(capacity // chunk + 1):
+            o.push(rows, chunk)
+        t0 = time.perf_counter()
+        for _ in range(100):
+            o.push(rows, chunk)
+        cpu_push = 100 * chunk / (time.perf_counter() - t0)
+        Lo = orc.lib()
+        dst = o._dst(batch)
+        dptr = orc._ptr_array(dst)
+        calls, t_end = 0, time.perf_counter() + 4.0
+        t0 = time.perf_counter()
+        while time.perf_counter() < t_end:
+            Lo.orc_res_sample(o.h, batch, None, dptr)
+            calls += 1
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": calls * batch / dt, "unit": "transitions/s", "cores": 1, "kind": "port",
+                               "sample": "%d sample calls of batch %d in %.1f s (and %.3g pushed rows/s), capacity "
+                                         "%d, 1 thread" % (calls, batch, dt, cpu_push, capacity)}
+    buf.destroy()
+    print(json.dumps(res))
+    return 0
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -223,6 +304,8 @@ def main():
     torch.cuda.set_device(0)
     if a.workload == "c2":
         return bench_uniform(a)
+    if a.workload == "res":
+        return bench_reservoir(a)
     capacity, batch, shapes, np_dtypes, upd_n, ins_n, desc = WORKLOADS[a.workload]
     _lib.set_option("row_split", a.row_split)
     _lib.set_option("sample_path", a.sample_path)

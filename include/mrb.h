@@ -141,6 +141,26 @@ int mrb_per_field_ptr(int64_t h, int field, void **dev_ptr);
 /* Replaces PriorityReplayBufferDestroy (priority_replay_buffer.py:74-76,138). */
 int mrb_per_destroy(int64_t h);
 
+/* ---- reservoir replay buffer --------------------------------------------- */
+
+/* Replaces ReservoirReplayBufferCreate
+ * (mindspore_rl/core/reservoir_replay_buffer.py:61-63). */
+int mrb_res_create(int64_t capacity, int nfields, const int64_t *field_bytes, uint64_t seed, int64_t *out_handle);
+/* Replaces ReservoirReplayBufferPush (reservoir_replay_buffer.py:64,68-79), batched: equals nrows
+ * sequential pushes of Algorithm R. Row number t (counted from 0 over the buffer's life) goes to slot
+ * t while t < capacity; afterwards it draws r uniformly in [0, t] from the buffer's counter-based
+ * generator and replaces slot r if r < capacity (else it is dropped). Rows of one call that pick the
+ * same slot: the later row wins. */
+int mrb_res_push(int64_t h, const void *const *src_fields, int64_t nrows, void *stream);
+/* Replaces ReservoirReplayBufferSample (reservoir_replay_buffer.py:65,81-89): n slots drawn uniformly
+ * in [0, size) with replacement (n may exceed size), optionally written to out_indices, and gathered. */
+int mrb_res_sample(int64_t h, int64_t n, int64_t *out_indices, void *const *dst_fields, void *stream);
+/* Rows held and rows ever pushed. */
+int mrb_res_state(int64_t h, int64_t *size, int64_t *total);
+int mrb_res_field_ptr(int64_t h, int field, void **dev_ptr);
+/* Replaces ReservoirReplayBufferDestroy (reservoir_replay_buffer.py:66,91-100). */
+int mrb_res_destroy(int64_t h);
+
 #ifdef __cplusplus
 }
 #endif

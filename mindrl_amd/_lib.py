@@ -42,6 +42,12 @@ SIGNATURES = {
     "mrb_per_check": [_i64, C.POINTER(C.c_uint32), _vp],
     "mrb_per_field_ptr": [_i64, _int, _pvp],
     "mrb_per_destroy": [_i64],
+    "mrb_res_create": [_i64, _int, _pi64, _u64, _pi64],
+    "mrb_res_push": [_i64, _pvp, _i64, _vp],
+    "mrb_res_sample": [_i64, _i64, _vp, _pvp, _vp],
+    "mrb_res_state": [_i64, _pi64, _pi64],
+    "mrb_res_field_ptr": [_i64, _int, _pvp],
+    "mrb_res_destroy": [_i64],
 }
 
 _lib = None

@@ -1,5 +1,6 @@
 """Buffer classes with the constructor and method signatures of mindspore_rl.core."""
 from .priority_replay_buffer import PriorityReplayBuffer
+from .reservoir_replay_buffer import ReservoirReplayBuffer
 from .uniform_replay_buffer import UniformReplayBuffer
 
-__all__ = ["PriorityReplayBuffer", "UniformReplayBuffer"]
+__all__ = ["PriorityReplayBuffer", "ReservoirReplayBuffer", "UniformReplayBuffer"]

@@ -1,0 +1,89 @@
+"""ReservoirReplayBuffer with the interface of
+mindspore_rl/core/reservoir_replay_buffer.py:23-100, backed by libmrb.so."""
+import ctypes as C
+import os
+
+import torch
+
+from .. import _lib
+from ._rows import FieldLayout, device, pointers, stream_ptr, view_of
+
+
+class ReservoirReplayBuffer:
+    """Reservoir-sampling buffer (Vitter's Algorithm R) resident in HBM: keeps an
+    unbiased sample of everything ever pushed.
+
+    Same constructor and methods as the reference class
+    (mindspore_rl/core/reservoir_replay_buffer.py:61-100).
+
+    Args:
+        capacity (int): rows kept.
+        sample_size (int): rows returned by sample() (may exceed capacity: draws are with replacement).
+        shapes, dtypes: shape / element type of each tensor of a transition.
+        seed0, seed1 (int): generator seed; seed1 if non-zero, else seed0, else entropy.
+    """
+
+    def __init__(self, capacity, sample_size, shapes, dtypes, seed0=0, seed1=0):
+        self._dev = device()
+        self._layout = FieldLayout(shapes, dtypes)
+        self._capacity = int(capacity)
+        self._sample_size = int(sample_size)
+        seed = int(seed1) or int(seed0) or int.from_bytes(os.urandom(8), "little")
+        h = C.c_int64(0)
+        _lib.check(_lib.lib().mrb_res_create(self._capacity, len(self._layout), self._layout.c_bytes,
+                                             seed & (2**64 - 1), C.byref(h)))
+        self._h = h.value
+        self._handle = torch.tensor([self._h], dtype=torch.int64)
+        self._keep = None
+
+    def push(self, *transition):
+        """Pushes one transition (tensors of shape_i) or a batch ([n, *shape_i])
+        (reservoir_replay_buffer.py:68-79). Returns the handle tensor int64[1]."""
+        if len(transition) == 1 and isinstance(transition[0], (list, tuple)):
+            transition = tuple(transition[0])
+        n = self._layout.batch_of(transition)
+        src = self._layout.to_device(transition, self._dev)
+        _lib.check(_lib.lib().mrb_res_push(self._h, pointers(src), n, stream_ptr()))
+        self._keep = src
+        return self._handle
+
+    insert = push
+
+    def sample(self, with_indices=False):
+        """`sample_size` rows drawn uniformly with replacement (reservoir_replay_buffer.py:81-89)."""
+        n = self._sample_size
+        dst = self._layout.empty(n, self._dev)
+        idx = torch.empty(n, dtype=torch.int64, device=self._dev) if with_indices else None
+        _lib.check(_lib.lib().mrb_res_sample(self._h, n, idx.data_ptr() if with_indices else None, pointers(dst),
+                                             stream_ptr()))
+        return (idx, tuple(dst)) if with_indices else tuple(dst)
+
+    def destroy(self):
+        """Releases the native buffer (reservoir_replay_buffer.py:91-100)."""
+        if self._h:
+            h, self._h = self._h, 0
+            _lib.check(_lib.lib().mrb_res_destroy(h))
+        return self._handle
+
+    def size(self):
+        return self._state()[0]
+
+    def total(self):
+        return self._state()[1]
+
+    def _state(self):
+        s, t = C.c_int64(0), C.c_int64(0)
+        _lib.check(_lib.lib().mrb_res_state(self._h, C.byref(s), C.byref(t)))
+        return s.value, t.value
+
+    def storage(self):
+        """Views of the row storage, one [capacity, *shape_i] tensor per field."""
+        views = []
+        for i, (s, d) in enumerate(zip(self._layout.shapes, self._layout.dtypes)):
+            p = C.c_void_p()
+            _lib.check(_lib.lib().mrb_res_field_ptr(self._h, i, C.byref(p)))
+            views.append(view_of(p.value, (self._capacity,) + s, d, self, self._dev))
+        return tuple(views)
+
+    def __repr__(self):
+        return "ReservoirReplayBuffer<>"

@@ -168,10 +168,23 @@ struct Per {
     }
 };
 
+struct Res {
+    RowStore rows;
+    int64_t size = 0, total = 0;
+    uint64_t seed = 0, calls = 0, epoch = 0;
+    unsigned long long* stamp = nullptr;
+    uint32_t* err = nullptr;
+    ~Res() {
+        if (stamp) (void)hipFree(stamp);
+        if (err) (void)hipFree(err);
+    }
+};
+
 std::mutex g_mu;
 int64_t g_next = 1;
 std::unordered_map<int64_t, std::shared_ptr<Urb>> g_urb;
 std::unordered_map<int64_t, std::shared_ptr<Per>> g_per;
+std::unordered_map<int64_t, std::shared_ptr<Res>> g_res;
 
 std::shared_ptr<Urb> find_urb(int64_t h) {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -184,6 +197,14 @@ std::shared_ptr<Per> find_per(int64_t h) {
     return it == g_per.end() ? nullptr : it->second;
 }
 
+std::shared_ptr<Res> find_res(int64_t h) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_res.find(h);
+    return it == g_res.end() ? nullptr : it->second;
+}
+#define GET_RES(b, h)                                                              \
+    auto b = find_res(h);                                                          \
+    if (!b) return fail(MRB_EHANDLE, "unknown reservoir buffer handle %lld", (long long)(h))
 #define GET_URB(b, h)                                                              \
     auto b = find_urb(h);                                                          \
     if (!b) return fail(MRB_EHANDLE, "unknown uniform buffer handle %lld", (long long)(h))
@@ -610,6 +631,95 @@ int mrb_per_destroy(int64_t h) {
         if (it == g_per.end()) return fail(MRB_EHANDLE, "unknown priority buffer handle %lld", (long long)h);
         b = it->second;
         g_per.erase(it);
+    }
+    HIP_TRY(hipDeviceSynchronize());
+    return MRB_OK;
+}
+
+/* -------------------------------------------------------------- reservoir */
+
+int mrb_res_create(int64_t capacity, int nfields, const int64_t* field_bytes, uint64_t seed, int64_t* out_handle) {
+    if (!out_handle) return fail(MRB_EINVAL, "out_handle is NULL");
+    auto b = std::make_shared<Res>();
+    int rc = rows_alloc(b->rows, capacity, nfields, field_bytes);
+    if (rc) return rc;
+    b->seed = seed;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->stamp), (size_t)capacity * sizeof(unsigned long long)));
+    HIP_TRY(hipMemset(b->stamp, 0, (size_t)capacity * sizeof(unsigned long long)));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16));
+    HIP_TRY(hipMemset(b->err, 0, 16));
+    std::lock_guard<std::mutex> lk(g_mu);
+    *out_handle = g_next++;
+    g_res[*out_handle] = b;
+    return MRB_OK;
+}
+
+int mrb_res_push(int64_t h, const void* const* src_fields, int64_t nrows, void* stream) {
+    GET_RES(b, h);
+    if (nrows <= 0) return fail(MRB_EINVAL, "nrows %lld must be positive", (long long)nrows);
+    if (nrows > 0x7fffffffll) return fail(MRB_EINVAL, "nrows %lld exceeds 2^31 - 1 rows per call", (long long)nrows);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    IoTable t;
+    int rc = make_table(b->rows, src_fields, nrows, t);
+    if (rc) return rc;
+    const int64_t cap = b->rows.capacity;
+    // Rows of one call can only collide on a slot once replacement has begun.
+    const bool elect = nrows > 1 && b->total + nrows > cap;
+    if (elect) {
+        b->epoch += 1;
+        if ((uint32_t)b->epoch == 0) {
+            HIP_TRY(hipMemsetAsync(b->stamp, 0, (size_t)cap * sizeof(unsigned long long), s));
+            b->epoch += 1;
+        }
+        hipLaunchKernelGGL(k_res_elect, dim3(grid_exact((uint64_t)nrows)), dim3(kWG), 0, s, b->stamp, b->total, nrows,
+                           cap, b->seed, (uint32_t)b->epoch);
+        LAUNCH_CHECK("k_res_elect");
+    }
+    hipLaunchKernelGGL(k_res_put, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t,
+                       elect ? b->stamp : nullptr, b->total, cap, b->seed, (uint32_t)b->epoch);
+    LAUNCH_CHECK("k_res_put");
+    b->total += nrows;
+    b->size = b->total < cap ? b->total : cap;
+    return MRB_OK;
+}
+
+int mrb_res_sample(int64_t h, int64_t n, int64_t* out_indices, void* const* dst_fields, void* stream) {
+    GET_RES(b, h);
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (b->size <= 0) return fail(MRB_ESTATE, "sample from an empty buffer");
+    IoTable t;
+    int rc = make_table(b->rows, dst_fields, n, t);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0,
+                       static_cast<hipStream_t>(stream), t, b->rows.capacity, b->size,
+                       static_cast<const int64_t*>(nullptr), (int64_t)-1, b->seed, b->calls + 1, out_indices, b->err);
+    LAUNCH_CHECK("k_rows_gather");
+    b->calls += 1;
+    return MRB_OK;
+}
+
+int mrb_res_state(int64_t h, int64_t* size, int64_t* total) {
+    GET_RES(b, h);
+    if (size) *size = b->size;
+    if (total) *total = b->total;
+    return MRB_OK;
+}
+
+int mrb_res_field_ptr(int64_t h, int field, void** dev_ptr) {
+    GET_RES(b, h);
+    if (field < 0 || field >= b->rows.nfields || !dev_ptr) return fail(MRB_EINVAL, "bad field %d", field);
+    *dev_ptr = b->rows.data[field];
+    return MRB_OK;
+}
+
+int mrb_res_destroy(int64_t h) {
+    std::shared_ptr<Res> b;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        auto it = g_res.find(h);
+        if (it == g_res.end()) return fail(MRB_EHANDLE, "unknown reservoir buffer handle %lld", (long long)h);
+        b = it->second;
+        g_res.erase(it);
     }
     HIP_TRY(hipDeviceSynchronize());
     return MRB_OK;

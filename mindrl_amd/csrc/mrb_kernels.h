@@ -191,6 +191,49 @@ __global__ __launch_bounds__(kWG) void k_rows_gather(IoTable t, int64_t capacity
     }
 }
 
+// ---------------------------------------------------------------------------
+// Reservoir push (ReservoirReplayBufferPush,
+// mindspore_rl/core/reservoir_replay_buffer.py:64,68-79), Algorithm R for a
+// batch: row j of the call is row number t = total + j of the buffer's life.
+//   t < capacity : slot t
+//   otherwise    : r uniform in [0, t]; slot r if r < capacity, else dropped
+// k_res_elect makes the last row of the call that picks a slot its owner
+// (integer max of (epoch << 32 | j)); k_res_put copies the owners' rows.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int64_t reservoir_slot(int64_t t, int64_t capacity, uint64_t seed) {
+    if (t < capacity) return t;
+    const int64_t r = rng_below(seed, 0, (uint64_t)t, t + 1);
+    return r < capacity ? r : -1;
+}
+
+__global__ __launch_bounds__(kWG) void k_res_elect(unsigned long long* __restrict__ stamp, int64_t total,
+                                                   int64_t nrows, int64_t capacity, uint64_t seed, uint32_t epoch) {
+    const int64_t j = (int64_t)blockIdx.x * kWG + threadIdx.x;
+    if (j >= nrows) return;
+    const int64_t slot = reservoir_slot(total + j, capacity, seed);
+    if (slot >= 0) atomicMax(&stamp[slot], ((unsigned long long)epoch << 32) | (unsigned long long)j);
+}
+
+// stamp == NULL: a single row, no election needed.
+__global__ __launch_bounds__(kWG) void k_res_put(IoTable t, const unsigned long long* __restrict__ stamp,
+                                                 int64_t total, int64_t capacity, uint64_t seed, uint32_t epoch) {
+    const uint64_t work = t.prefix[t.nfields];
+    const uint64_t stride = (uint64_t)gridDim.x * kWG;
+    for (uint64_t w = (uint64_t)blockIdx.x * kWG + threadIdx.x; w < work; w += stride) {
+        const int f = field_of(t, w);
+        uint64_t row;
+        uint32_t unit;
+        split_work(w - t.prefix[f], t.units[f], row, unit);
+        const int64_t slot = reservoir_slot(total + (int64_t)row, capacity, seed);
+        if (slot < 0) continue;
+        if (stamp && stamp[slot] != (((unsigned long long)epoch << 32) | row)) continue;
+        const uint32_t vl = t.vec_log2[f];
+        const uint64_t off = (uint64_t)unit << vl;
+        copy_granule(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f] + off,
+                     as_global(t.io[f]) + row * t.row_bytes[f] + off, vl);
+    }
+}
+
 // Arguments common to both sample kernels. Passed first, with the fields that the
 // tree descent needs at the front: the leading kernel-argument dwords are preloaded
 // into scalar registers at wave launch, which saves a dependent fetch.

@@ -33,6 +33,10 @@
  *   orc_rng_*       the reference's generator (engine + distribution) is
  *                   unspecified by its sources: parity unpinned; draws are
  *                   normally supplied by the caller.
+ *   orc_res_*       reservoir policy (draw range, which stream): parity unpinned;
+ *                   pinned by the reservoir's defining property (every row kept
+ *                   with probability capacity / rows seen) and the reference
+ *                   test's row-consistency invariant.
  *   ring / gather / tree build / update: pinned by closed forms, brute force
  *                   and numpy library routines in tests/test_oracle_*.py.
  */
@@ -256,6 +260,68 @@ void orc_urb_reset(orc_urb *b) { b->count = 0; } /* uniform_replay_buffer.py:149
 int64_t orc_urb_count(const orc_urb *b) { return b->count; }
 int64_t orc_urb_head(const orc_urb *b) { return b->head; }
 const void *orc_urb_field(const orc_urb *b, int i) { return b->rows.data[i]; }
+
+/* ------------------------------------------------------------------------
+ * Reservoir buffer (mindspore_rl/core/reservoir_replay_buffer.py:61-100):
+ * Vitter's Algorithm R. The first `capacity` rows fill the slots in order; row
+ * number t (0-based) after that draws r uniformly in [0, t] and replaces slot r
+ * if r < capacity, so every row seen so far is retained with probability
+ * capacity / (t + 1). sample() draws slots uniformly in [0, size) with
+ * replacement (the reference's own test samples 256 rows from 100,
+ * tests/st/test_reservoir_replay_buffer.py:33-49).
+ * Parity unpinned: the reference's generator and draw order are not in its
+ * sources; draw t of the push stream is orc_rng_below(seed, 0, t, t + 1), call
+ * c of sample() uses stream counter c + 1.
+ * ---------------------------------------------------------------------- */
+typedef struct {
+    orc_rows rows;
+    int64_t size, total;
+    uint64_t seed, calls;
+} orc_res;
+
+orc_res *orc_res_create(int64_t capacity, int nfields, const int64_t *bytes, uint64_t seed) {
+    orc_res *b = (orc_res *)calloc(1, sizeof(orc_res));
+    if (!b) return NULL;
+    if (rows_init(&b->rows, capacity, nfields, bytes)) {
+        free(b);
+        return NULL;
+    }
+    b->seed = seed;
+    return b;
+}
+void orc_res_destroy(orc_res *b) {
+    if (!b) return;
+    rows_free(&b->rows);
+    free(b);
+}
+int orc_res_push(orc_res *b, const void *const *src, int64_t nrows) {
+    if (nrows <= 0) return 1;
+    for (int64_t j = 0; j < nrows; ++j) {
+        int64_t t = b->total;
+        if (t < b->rows.capacity) {
+            rows_put(&b->rows, t, src, j);
+            b->size += 1;
+        } else {
+            int64_t r = orc_rng_below(b->seed, 0, (uint64_t)t, t + 1);
+            if (r < b->rows.capacity) rows_put(&b->rows, r, src, j);
+        }
+        b->total += 1;
+    }
+    return 0;
+}
+int orc_res_sample(orc_res *b, int64_t n, int64_t *out_indices, void *const *dst) {
+    if (n <= 0 || b->size <= 0) return 1;
+    for (int64_t k = 0; k < n; ++k) {
+        int64_t idx = orc_rng_below(b->seed, b->calls + 1, (uint64_t)k, b->size);
+        if (out_indices) out_indices[k] = idx;
+        rows_get(&b->rows, idx, dst, k);
+    }
+    b->calls += 1;
+    return 0;
+}
+int64_t orc_res_size(const orc_res *b) { return b->size; }
+int64_t orc_res_total(const orc_res *b) { return b->total; }
+const void *orc_res_field(const orc_res *b, int i) { return b->rows.data[i]; }
 
 /* ------------------------------------------------------------------------
  * Prioritized buffer (priority_replay_buffer.py:60-138): FIFO rows + a sum

@@ -50,6 +50,13 @@ def lib():
         "orc_urb_count": (i64, [vp]),
         "orc_urb_head": (i64, [vp]),
         "orc_urb_field": (vp, [vp, C.c_int]),
+        "orc_res_create": (vp, [i64, C.c_int, vp, u64]),
+        "orc_res_destroy": (None, [vp]),
+        "orc_res_push": (C.c_int, [vp, pvp, i64]),
+        "orc_res_sample": (C.c_int, [vp, i64, vp, pvp]),
+        "orc_res_size": (i64, [vp]),
+        "orc_res_total": (i64, [vp]),
+        "orc_res_field": (vp, [vp, C.c_int]),
         "orc_per_create": (vp, [i64, f32, C.c_int, vp, u64]),
         "orc_per_destroy": (None, [vp]),
         "orc_per_update": (C.c_int, [vp, vp, vp, i64]),
@@ -172,6 +179,47 @@ class OracleUniform(_Rows):
     def field(self, i):
         n = self.capacity * self.bytes[i]
         raw = (C.c_ubyte * n).from_address(lib().orc_urb_field(self.h, i))
+        return np.frombuffer(raw, np.uint8).view(self.dtypes[i]).reshape((self.capacity,) + self.shapes[i]).copy()
+
+
+class OracleReservoir(_Rows):
+    """CPU twin of ReservoirReplayBuffer (mindspore_rl/core/reservoir_replay_buffer.py:23-100)."""
+
+    def __init__(self, capacity, shapes, dtypes, seed=0):
+        super().__init__(shapes, dtypes)
+        self.capacity = int(capacity)
+        self.h = lib().orc_res_create(self.capacity, len(self.bytes), self._fb, seed)
+        if not self.h:
+            raise ValueError("orc_res_create failed")
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_res_destroy(self.h)
+            self.h = None
+
+    def push(self, fields, nrows):
+        src = self._src(fields, nrows)
+        if lib().orc_res_push(self.h, _ptr_array(src), nrows):
+            raise ValueError("orc_res_push failed")
+
+    def sample(self, n):
+        idx = np.empty(n, np.int64)
+        dst = self._dst(n)
+        if lib().orc_res_sample(self.h, n, idx.ctypes.data, _ptr_array(dst)):
+            raise ValueError("orc_res_sample failed")
+        return idx, dst
+
+    @property
+    def size(self):
+        return lib().orc_res_size(self.h)
+
+    @property
+    def total(self):
+        return lib().orc_res_total(self.h)
+
+    def field(self, i):
+        n = self.capacity * self.bytes[i]
+        raw = (C.c_ubyte * n).from_address(lib().orc_res_field(self.h, i))
         return np.frombuffer(raw, np.uint8).view(self.dtypes[i]).reshape((self.capacity,) + self.shapes[i]).copy()
 
 

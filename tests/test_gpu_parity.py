@@ -17,14 +17,14 @@ def mrb():
     if not torch.cuda.is_available():
         pytest.fail("no HIP device: the GPU parity tests cannot run (there is no CPU fallback)")
     from mindrl_amd import _lib
-    from mindrl_amd.core import PriorityReplayBuffer, UniformReplayBuffer
+    from mindrl_amd.core import PriorityReplayBuffer, ReservoirReplayBuffer, UniformReplayBuffer
     _lib.lib()
 
     class NS:
         pass
 
     ns = NS()
-    ns.lib, ns.PER, ns.URB = _lib, PriorityReplayBuffer, UniformReplayBuffer
+    ns.lib, ns.PER, ns.URB, ns.RES = _lib, PriorityReplayBuffer, UniformReplayBuffer, ReservoirReplayBuffer
     yield ns
     _lib.set_option("sample_path", 0)
     _lib.set_option("row_split", 0)
@@ -97,6 +97,46 @@ def test_uniform_successive_samples_differ_and_errors(mrb):
         g._state()  # destroyed handle
     with pytest.raises(ValueError):
         mrb.URB(1, 0, [(1,)], [torch.int32])
+
+
+# ---------------------------------------------------------------- reservoir
+@pytest.mark.parametrize("cap", [1, 10, 100, 5000])
+def test_reservoir_random_pushes_bit_exact(mrb, orc, cap):
+    """Batched and single pushes well past the capacity; storage compared slot by slot, then samples."""
+    shapes, dtypes = [(17,), (6,), (1,)], [np.float32, np.int32, np.bool_]
+    rng = np.random.default_rng(cap)
+    g = mrb.RES(cap, 64, shapes, torch_types(dtypes), seed0=0, seed1=42)
+    c = orc.OracleReservoir(cap, shapes, dtypes, seed=42)
+    for step in range(30):
+        n = 1 if step % 4 == 0 else int(rng.integers(1, 3 * cap + 5))
+        rows = random_rows(rng, n, shapes, dtypes)
+        g.push(*to_dev(rows)) if n > 1 else g.push(*[torch.from_numpy(r[0]).cuda() for r in rows])
+        c.push(rows, n)
+        assert (g.size(), g.total()) == (c.size, c.total)
+        for f, view in enumerate(g.storage()):
+            assert np.array_equal(t2n(view).view(np.uint8), c.field(f).view(np.uint8)), (step, f)
+        gi, gf = g.sample(with_indices=True)
+        ci, cf = c.sample(64)
+        assert np.array_equal(t2n(gi), ci)
+        for a, b in zip(gf, cf):
+            assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+    g.destroy()
+
+
+def test_reservoir_reference_scenario(mrb):
+    """tests/st/test_reservoir_replay_buffer.py:33-54 on the HIP buffer."""
+    prb = mrb.RES(100, 256, ((17,), (6,)), (torch.float32, torch.int32), seed0=0, seed1=42)
+    for i in range(100):
+        prb.push(torch.ones(17) * i, (torch.ones(6) * i).to(torch.int32))
+    states, actions = prb.sample()
+    states, actions = t2n(states), t2n(actions)
+    assert states.shape == (256, 17) and actions.shape == (256, 6)
+    assert np.allclose(states, states[:, 0:1]) and np.allclose(actions, actions[:, 0:1])
+    assert np.allclose(states[:, 0], actions[:, 0])
+    h = prb.destroy()
+    assert h.dtype == torch.int64 and tuple(h.shape) == (1,)
+    with pytest.raises(ValueError):
+        mrb.RES(4, 2, [(1,)], [torch.int32], seed0=1).sample()  # empty
 
 
 # ---------------------------------------------------------------------- PER

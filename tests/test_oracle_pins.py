@@ -378,3 +378,52 @@ def test_errors(orc):
         per.update([0], [-1.0])
     with pytest.raises(ValueError):
         per.update([0], [np.nan])
+
+
+# ---------------------------------------------------------------- reservoir
+def test_reservoir_keeps_every_row_with_equal_probability(orc):
+    """Defining property of reservoir sampling: after N rows, each is held with probability capacity / N."""
+    cap, n, trials = 8, 40, 6000
+    kept = np.zeros(n)
+    for t in range(trials):
+        b = orc.OracleReservoir(cap, [(1,)], [np.int32], seed=5000 + t)
+        if t % 2:
+            b.push([np.arange(n, dtype=np.int32)[:, None]], n)  # one batch
+        else:
+            for i in range(n):  # row by row: same policy
+                b.push([np.array([[i]], np.int32)], 1)
+        held = b.field(0)[:, 0]
+        assert len(set(held)) == cap and b.size == cap and b.total == n
+        kept[held] += 1
+    p = kept / trials
+    sigma = np.sqrt(0.2 * 0.8 / trials)
+    assert np.all(np.abs(p - cap / n) < 5 * sigma), p
+
+
+def test_reservoir_fill_phase_and_batch_equals_sequential(orc):
+    a = orc.OracleReservoir(10, [(2,), (1,)], [np.float32, np.int32], seed=9)
+    b = orc.OracleReservoir(10, [(2,), (1,)], [np.float32, np.int32], seed=9)
+    ids = np.arange(37)
+    rows = [np.stack([ids, -ids], 1).astype(np.float32), ids.astype(np.int32)[:, None]]
+    a.push([r[:6] for r in rows], 6)
+    assert a.size == 6 and list(a.field(1)[:6, 0]) == [0, 1, 2, 3, 4, 5]  # slots fill in order
+    a.push([r[6:] for r in rows], 31)
+    for i in range(37):
+        b.push([r[i:i + 1] for r in rows], 1)
+    assert np.array_equal(a.field(0), b.field(0)) and np.array_equal(a.field(1), b.field(1))
+    assert a.total == b.total == 37 and a.size == 10
+
+
+def test_reservoir_reference_scenario(orc):
+    """tests/st/test_reservoir_replay_buffer.py:33-54: capacity 100, sample 256 rows after 100 pushes
+    whose values equal their row number; every sampled row is internally consistent."""
+    buf = orc.OracleReservoir(100, [(17,), (6,)], [np.float32, np.int32], seed=42)
+    for i in range(100):
+        buf.push([np.ones((1, 17), np.float32) * i, np.ones((1, 6), np.int32) * i], 1)
+    idx, (states, actions) = buf.sample(256)
+    assert np.allclose(states, states[:, 0:1]) and np.allclose(actions, actions[:, 0:1])
+    assert np.allclose(states[:, 0], actions[:, 0]) and np.array_equal(states[:, 0], idx)
+    idx2, _ = buf.sample(256)
+    assert not np.array_equal(idx, idx2) and idx.min() >= 0 and idx.max() < 100
+    with pytest.raises(ValueError):
+        orc.OracleReservoir(4, [(1,)], [np.int32]).sample(2)  # empty
