@@ -75,6 +75,11 @@ int mrb_urb_create(int64_t capacity, int nfields, const int64_t *field_bytes, in
  * nrows rows; src_fields[i] is a contiguous [nrows, field_bytes[i]] matrix.
  * nrows > capacity keeps the last `capacity` rows. */
 int mrb_urb_append(int64_t h, const void *const *src_fields, int64_t nrows, void *stream);
+/* Buffer-to-buffer append in one launch: the n rows of `src` at logical positions first_logical ..
+ * first_logical + n - 1 (0 = oldest, negative counts back from the newest) are appended to `h` with
+ * mrb_urb_append's semantics. Replaces the get_item + insert loop of NStepBuffer.get_data
+ * (mindspore_rl/utils/n_step_buffer.py:85-92). Both buffers need the same fields. */
+int mrb_urb_append_from(int64_t h, int64_t src, int64_t first_logical, int64_t n, void *stream);
 /* Replaces P.BufferGetItem (uniform_replay_buffer.py:83,128): row at LOGICAL
  * position (0 = oldest, negative counts back from the newest) copied to
  * dst_fields[i] ([field_bytes[i]] each). */

@@ -24,6 +24,7 @@ SIGNATURES = {
     "mrb_set_option": [C.c_char_p, _i64],
     "mrb_urb_create": [_i64, _int, _pi64, _pi64],
     "mrb_urb_append": [_i64, _pvp, _i64, _vp],
+    "mrb_urb_append_from": [_i64, _i64, _i64, _i64, _vp],
     "mrb_urb_get_item": [_i64, _i64, _pvp, _vp],
     "mrb_urb_gather": [_i64, _vp, _i64, _pvp, _vp],
     "mrb_urb_sample": [_i64, _i64, _vp, _pvp, _vp],

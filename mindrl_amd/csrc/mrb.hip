@@ -124,7 +124,8 @@ int rows_put(const RowStore& r, const void* const* src, int64_t skip, int64_t n,
     }
     int rc = make_table(r, shifted, n, t);
     if (rc) return rc;
-    hipLaunchKernelGGL(k_rows_put, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, r.capacity, first_slot);
+    hipLaunchKernelGGL(k_rows_put, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, r.capacity, first_slot,
+                       (int64_t)0, (int64_t)0);
     LAUNCH_CHECK("k_rows_put");
     return MRB_OK;
 }
@@ -138,6 +139,24 @@ struct Urb {
         if (err) (void)hipFree(err);
     }
 };
+
+// count / head after appending n rows (write position chosen once per call: `count` while the
+// buffer has never wrapped, else `head`).
+void urb_advance(Urb& b, int64_t n) {
+    const int64_t cap = b.rows.capacity;
+    if (b.count < cap && b.head == 0) {
+        const int64_t room = cap - b.count;
+        if (n <= room) {
+            b.count += n;
+        } else {
+            b.count = cap;
+            b.head = (n - room) % cap;
+        }
+    } else {
+        b.head = (b.head + n) % cap;
+        b.count = b.count + n < cap ? b.count + n : cap;
+    }
+}
 
 struct Per {
     RowStore rows;
@@ -325,18 +344,41 @@ int mrb_urb_append(int64_t h, const void* const* src_fields, int64_t nrows, void
     const int64_t first = (w + skip) % cap;
     int rc = rows_put(b->rows, src_fields, skip, nrows - skip, first, static_cast<hipStream_t>(stream));
     if (rc) return rc;
-    if (growing) {
-        const int64_t room = cap - b->count;
-        if (nrows <= room) {
-            b->count += nrows;
-        } else {
-            b->count = cap;
-            b->head = (nrows - room) % cap;
-        }
-    } else {
-        b->head = (b->head + nrows) % cap;
-        b->count = b->count + nrows < cap ? b->count + nrows : cap;
-    }
+    urb_advance(*b, nrows);
+    return MRB_OK;
+}
+
+/* Appends to `h` the `n` rows of uniform buffer `src` at logical positions first .. first + n - 1
+ * (0 = oldest), in one launch. */
+int mrb_urb_append_from(int64_t h, int64_t src, int64_t first_logical, int64_t n, void* stream) {
+    GET_URB(b, h);
+    auto from = find_urb(src);
+    if (!from) return fail(MRB_EHANDLE, "unknown uniform buffer handle %lld", (long long)src);
+    if (from.get() == b.get()) return fail(MRB_EINVAL, "source and destination are the same buffer");
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (first_logical < 0) first_logical += from->count;
+    if (first_logical < 0 || first_logical + n > from->count)
+        return fail(MRB_EINVAL, "rows [%lld, %lld) outside the %lld stored rows", (long long)first_logical,
+                    (long long)(first_logical + n), (long long)from->count);
+    if (from->rows.nfields != b->rows.nfields) return fail(MRB_EINVAL, "buffers differ in their fields");
+    for (int i = 0; i < b->rows.nfields; ++i)
+        if (from->rows.bytes[i] != b->rows.bytes[i]) return fail(MRB_EINVAL, "buffers differ in field %d", i);
+    const int64_t cap = b->rows.capacity;
+    // source slot of the first row: logical -> physical as in get_item
+    const int64_t t0 = from->count - from->head;
+    const int64_t src_first = first_logical < t0 ? first_logical + from->head : first_logical - t0;
+    const bool growing = b->count < cap && b->head == 0;
+    const int64_t w = growing ? b->count : b->head;
+    const int64_t skip = n > cap ? n - cap : 0;
+    IoTable t;
+    const void* io[MRB_MAX_FIELDS];
+    for (int i = 0; i < b->rows.nfields; ++i) io[i] = from->rows.data[i];
+    int rc = make_table(b->rows, io, n - skip, t);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_rows_put, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, static_cast<hipStream_t>(stream),
+                       t, cap, (w + skip) % cap, from->rows.capacity, (src_first + skip) % from->rows.capacity);
+    LAUNCH_CHECK("k_rows_put");
+    urb_advance(*b, n);
     return MRB_OK;
 }
 

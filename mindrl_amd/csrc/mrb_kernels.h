@@ -143,7 +143,10 @@ __device__ __forceinline__ void split_work(uint64_t local, uint32_t units, uint6
 // PriorityReplayBufferPush (mindspore_rl/core/priority_replay_buffer.py:67-69).
 // The host guarantees nrows <= capacity, so no two rows share a slot.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kWG) void k_rows_put(IoTable t, int64_t capacity, int64_t first_slot) {
+// src_capacity > 0: the source is itself a ring of that many rows and row r is read from its
+// slot (src_first + r) mod src_capacity (buffer-to-buffer copy); 0: the source is contiguous.
+__global__ __launch_bounds__(kWG) void k_rows_put(IoTable t, int64_t capacity, int64_t first_slot,
+                                                  int64_t src_capacity, int64_t src_first) {
     const uint64_t total = t.prefix[t.nfields];
     const uint64_t stride = (uint64_t)gridDim.x * kWG;
     for (uint64_t w = (uint64_t)blockIdx.x * kWG + threadIdx.x; w < total; w += stride) {
@@ -153,9 +156,16 @@ __global__ __launch_bounds__(kWG) void k_rows_put(IoTable t, int64_t capacity, i
         split_work(w - t.prefix[f], t.units[f], row, unit);
         int64_t slot = first_slot + (int64_t)row;
         if (slot >= capacity) slot -= capacity;
+        uint64_t src_row = row;
+        if (src_capacity > 0) {
+            int64_t q = src_first + (int64_t)row;
+            if (q >= src_capacity) q -= src_capacity;
+            src_row = (uint64_t)q;
+        }
         const uint32_t vl = t.vec_log2[f];
         const uint64_t off = (uint64_t)unit << vl;
-        copy_granule(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f] + off, as_global(t.io[f]) + row * t.row_bytes[f] + off, vl);
+        copy_granule(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f] + off,
+                     as_global(t.io[f]) + src_row * t.row_bytes[f] + off, vl);
     }
 }
 

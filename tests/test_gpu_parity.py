@@ -99,6 +99,69 @@ def test_uniform_successive_samples_differ_and_errors(mrb):
         mrb.URB(1, 0, [(1,)], [torch.int32])
 
 
+# -------------------------------------------------------------- n-step buffer
+class OracleNStep:
+    """The reference's NStepBuffer, line for line, over two oracle ring buffers
+    (mindspore_rl/utils/n_step_buffer.py:51-103)."""
+
+    def __init__(self, orc, shapes, dtypes, td_step, buffer_size):
+        self.buffer = orc.OracleUniform(buffer_size, shapes, dtypes)
+        self.td_data = orc.OracleUniform(td_step, shapes, dtypes)
+        self.td = td_step
+
+    def push(self, rows):
+        self.buffer.append(rows, 1)
+
+    def get_data(self):
+        check = self.buffer.count > self.td
+        m = 0
+        while m < self.td and check:
+            keep = self.buffer.get_item(self.buffer.count - self.td + m)
+            self.td_data.append([k[None] for k in keep], 1)
+            m += 1
+        return check
+
+    def clear(self):
+        self.buffer.reset()
+        self.td_data.reset()
+
+
+@pytest.mark.parametrize("td,size", [(1, 5), (3, 10), (5, 6), (4, 64)])
+def test_n_step_buffer_matches_reference_loop(mrb, orc, td, size):
+    from mindrl_amd.utils import NStepBuffer
+    shapes, dtypes = [(4,), (1,)], [np.float32, np.int32]
+    rng = np.random.default_rng(td * 100 + size)
+    g = NStepBuffer(shapes, torch_types(dtypes), td, buffer_size=size)
+    c = OracleNStep(orc, shapes, dtypes, td, size)
+    for step in range(6 * size):
+        rows = random_rows(rng, 1, shapes, dtypes)
+        assert g.push([torch.from_numpy(r[0]).cuda() for r in rows]) is True
+        c.push(rows)
+        if step % 3 == 0:
+            check, data = g.get_data()
+            assert bool(check[0]) == c.get_data() and tuple(check.shape) == (1,)
+            for f, view in enumerate(data):
+                assert np.array_equal(t2n(view).view(np.uint8), c.td_data.field(f).view(np.uint8)), (step, f)
+            assert int(g.td_data.count) == c.td_data.count and int(g.td_data.head) == c.td_data.head
+        assert int(g.size()) == c.buffer.count
+        if step == 4 * size:
+            g.clear()
+            c.clear()
+    g.destroy()
+
+
+def test_create_replay_buffer_builds_working_buffers(mrb):
+    from mindrl_amd.core import create_replay_buffer
+    cfg = {"number": 2, "type": mrb.URB, "capacity": 50, "sample_size": 4,
+           "data_shape": [(4,), (1,)], "data_type": ["float32", "int32"]}
+    bufs = create_replay_buffer(cfg)
+    assert len(bufs) == 2
+    bufs[0].insert([torch.ones(8, 4).cuda(), torch.arange(8, dtype=torch.int32).reshape(8, 1).cuda()])
+    assert int(bufs[0].count) == 8 and int(bufs[1].count) == 0 and tuple(bufs[0].sample()[0].shape) == (4, 4)
+    for b in bufs:
+        b.destroy()
+
+
 # ---------------------------------------------------------------- reservoir
 @pytest.mark.parametrize("cap", [1, 10, 100, 5000])
 def test_reservoir_random_pushes_bit_exact(mrb, orc, cap):

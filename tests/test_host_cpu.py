@@ -24,7 +24,7 @@ def declared_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = declared_symbols()
-    assert len(names) == 30
+    assert len(names) == 31
     L = _lib.lib()
     for n in names:
         assert hasattr(L, n), "libmrb.so does not export %s" % n
@@ -109,3 +109,24 @@ def test_kernels_use_no_scratch_memory(tmp_path):
             assert lds <= 1024, (name, lds)
         if "k_tree_update" in name:
             assert lds <= 64, (name, lds)
+
+
+def test_create_replay_buffer_follows_the_reference_config_entry():
+    """mindspore_rl/core/msrl.py:270-300: type / number / params-or-(sample_size, capacity) + data_shape / data_type."""
+    from mindrl_amd.core import create_replay_buffer
+
+    class Fake:
+        def __init__(self, sample_size, capacity, shapes, types):
+            self.args = (sample_size, capacity, shapes, types)
+
+    cfg = {"number": 1, "type": Fake, "capacity": 100000, "sample_size": 64,
+           "data_shape": [(4,), (1,)], "data_type": ["float32", "int32"]}
+    one = create_replay_buffer(cfg)
+    assert one.args == (64, 100000, ((4,), (1,)), ("float32", "int32"))
+    many = create_replay_buffer(dict(cfg, number=3))
+    assert len(many) == 3 and all(isinstance(m, Fake) for m in many)
+    with_params = create_replay_buffer({"type": Fake, "params": {"sample_size": 2, "capacity": 5},
+                                        "data_shape": [(1,)], "data_type": ["float32"]})
+    assert with_params.args == (2, 5, ((1,),), ("float32",))
+    default_size = create_replay_buffer({"type": Fake, "capacity": 7, "data_shape": [(1,)], "data_type": ["int32"]})
+    assert default_size.args[0] == 1
