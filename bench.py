@@ -43,7 +43,7 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=2000)
     p.add_argument("--warmup", type=int, default=200)
-    p.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2", "res"])
+    p.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2", "res", "dr"])
     p.add_argument("--capacity", type=int, default=0, help="override the workload's capacity (for quick trials)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--graph", action="store_true", help="replay the timed steps as one captured HIP graph")
@@ -288,6 +288,65 @@ def bench_reservoir(a):
     return 0
 
 
+def bench_discounted_return(a):
+    """DiscountedReturn on [Timestep 1000, Batch 16384] float32 rewards with 1 % episode ends."""
+    import torch
+
+    from mindrl_amd import _lib
+
+    t, b, inner, gamma = 1000, (a.capacity or 16384), 1, 0.99
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    r = torch.randn(t, b, inner, device="cuda", generator=gen)
+    d = torch.rand(t, b, device="cuda", generator=gen) < 0.01
+    v = torch.randn(b, inner, device="cuda", generator=gen)
+    out = torch.empty_like(r)
+    L = _lib.lib()
+    sp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    K, W = min(a.steps, 200), min(a.warmup, 20)
+
+    def step():
+        rc = L.mrb_discounted_return(r.data_ptr(), d.data_ptr(), v.data_ptr(), out.data_ptr(), t, b, inner, gamma, sp)
+        if rc:
+            _lib.check(rc)
+
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(K):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    algo = t * b * inner * 8 + t * b
+    kern_s = ev0.elapsed_time(ev1) * 1e-3 / K
+    res = {
+        "metric": "discounted-return elements/sec", "value": K * t * b * inner / wall, "unit": "elements/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": wall * 1e3 / K, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "DiscountedReturn, reward [1000, %d, 1] f32, gamma 0.99, 1 %% dones" % b},
+        "roofline": {"bound": "hbm", "achieved": algo / kern_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "k_discounted_return",
+                     "algorithmic_bytes_per_launch": algo, "avg_launch_us": kern_s * 1e6},
+        "cpu_baseline": None,
+    }
+    if not a.no_cpu_baseline:
+        from oracle import orc
+        rn, dn, vn = r.cpu().numpy(), d.cpu().numpy(), v.cpu().numpy()
+        calls, t_end = 0, time.perf_counter() + 5.0
+        t0 = time.perf_counter()
+        while time.perf_counter() < t_end:
+            orc.discounted_return(rn, dn, vn, gamma)
+            calls += 1
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": calls * t * b * inner / dt, "unit": "elements/s", "cores": 1, "kind": "port",
+                               "sample": "%d calls on the same [1000, %d, 1] input in %.1f s, 1 thread" % (calls, b, dt)}
+    print(json.dumps(res))
+    return 0
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -306,6 +365,8 @@ def main():
         return bench_uniform(a)
     if a.workload == "res":
         return bench_reservoir(a)
+    if a.workload == "dr":
+        return bench_discounted_return(a)
     capacity, batch, shapes, np_dtypes, upd_n, ins_n, desc = WORKLOADS[a.workload]
     _lib.set_option("row_split", a.row_split)
     _lib.set_option("sample_path", a.sample_path)

@@ -166,6 +166,16 @@ int mrb_res_field_ptr(int64_t h, int field, void **dev_ptr);
 /* Replaces ReservoirReplayBufferDestroy (reservoir_replay_buffer.py:66,91-100). */
 int mrb_res_destroy(int64_t h);
 
+/* ---- discounted return --------------------------------------------------- */
+
+/* Replaces the fused DiscountedReturn primitive and the loop it stands for
+ * (mindspore_rl/utils/discounted_return.py:71,84-92): backwards over time,
+ *   last = reward[t] + (1 - done[t]) * gamma * last;  out[t] = last.
+ * reward and out are [timesteps, batch, inner] float32, done is [timesteps, batch] (one byte per
+ * flag), last_value is [batch, inner] float32; all device pointers. */
+int mrb_discounted_return(const float *reward, const uint8_t *done, const float *last_value, float *out,
+                          int64_t timesteps, int64_t batch, int64_t inner, float gamma, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

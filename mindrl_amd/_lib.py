@@ -49,6 +49,7 @@ SIGNATURES = {
     "mrb_res_state": [_i64, _pi64, _pi64],
     "mrb_res_field_ptr": [_i64, _int, _pvp],
     "mrb_res_destroy": [_i64],
+    "mrb_discounted_return": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp],
 }
 
 _lib = None

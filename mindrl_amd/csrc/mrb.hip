@@ -767,4 +767,22 @@ int mrb_res_destroy(int64_t h) {
     return MRB_OK;
 }
 
+/* ------------------------------------------------------- discounted return */
+
+int mrb_discounted_return(const float* reward, const uint8_t* done, const float* last_value, float* out,
+                          int64_t timesteps, int64_t batch, int64_t inner, float gamma, void* stream) {
+    if (!reward || !done || !last_value || !out) return fail(MRB_EINVAL, "a data pointer is NULL");
+    if (timesteps <= 0 || batch <= 0 || inner <= 0)
+        return fail(MRB_EINVAL, "timesteps %lld, batch %lld, inner %lld must be positive", (long long)timesteps,
+                    (long long)batch, (long long)inner);
+    if (!(gamma >= 0.0f && gamma <= 1.0f))
+        return fail(MRB_EINVAL, "The discounted factor should be a number in range [0, 1], but got %g.", (double)gamma);
+    const int64_t cols = batch * inner;
+    if (cols > (1ll << 40) / timesteps) return fail(MRB_EINVAL, "problem too large");
+    hipLaunchKernelGGL(k_discounted_return, dim3(grid_exact((uint64_t)cols)), dim3(kWG), 0,
+                       static_cast<hipStream_t>(stream), reward, done, last_value, out, timesteps, batch, inner, gamma);
+    LAUNCH_CHECK("k_discounted_return");
+    return MRB_OK;
+}
+
 }  // extern "C"

@@ -799,6 +799,47 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round) {
 constexpr int kTopWG = 1024;
 __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a) { top_rebuild(a, a.top_depth); }
 
+// ---------------------------------------------------------------------------
+// Discounted return (mindspore_rl/utils/discounted_return.py:84-92): one thread per
+// (batch, inner) column walks the time axis backwards; neighbouring threads hold
+// neighbouring columns, so every step's loads and stores are coalesced. The loads do
+// not depend on the recurrence, so they are issued UNROLL steps ahead of their use.
+//   last = reward[t] + ((1 - done[t]) * gamma) * last, each operation rounded once.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kWG) void k_discounted_return(const float* __restrict__ reward,
+                                                           const uint8_t* __restrict__ done,
+                                                           const float* __restrict__ last_value,
+                                                           float* __restrict__ out, int64_t timesteps, int64_t batch,
+                                                           int64_t inner, float gamma) {
+    constexpr int UNROLL = 8;
+    const int64_t cols = batch * inner;
+    const int64_t c = (int64_t)blockIdx.x * kWG + threadIdx.x;
+    if (c >= cols) return;
+    const int64_t b = c / inner;
+    float last = last_value[c];
+    int64_t t = timesteps - 1;
+    for (; t >= UNROLL - 1; t -= UNROLL) {
+        float r[UNROLL];
+        uint8_t d[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            r[u] = __builtin_nontemporal_load(reward + (t - u) * cols + c);
+            d[u] = done[(t - u) * batch + b];
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const float scaled = (1.0f - (d[u] ? 1.0f : 0.0f)) * gamma;
+            last = r[u] + scaled * last;
+            __builtin_nontemporal_store(last, out + (t - u) * cols + c);
+        }
+    }
+    for (; t >= 0; --t) {
+        const float scaled = (1.0f - (done[t * batch + b] ? 1.0f : 0.0f)) * gamma;
+        last = reward[t * cols + c] + scaled * last;
+        out[t * cols + c] = last;
+    }
+}
+
 // Fills a float array with one value (tree initialisation: sums 0, mins FLT_MAX).
 __global__ __launch_bounds__(kWG) void k_fill_f32(float* p, float v, uint64_t n) {
     const uint64_t stride = (uint64_t)gridDim.x * kWG;

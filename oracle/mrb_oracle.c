@@ -262,6 +262,29 @@ int64_t orc_urb_head(const orc_urb *b) { return b->head; }
 const void *orc_urb_field(const orc_urb *b, int i) { return b->rows.data[i]; }
 
 /* ------------------------------------------------------------------------
+ * Discounted return (mindspore_rl/utils/discounted_return.py:84-92, the
+ * reference's own non-fused loop): walking the time axis backwards,
+ *   last = reward[t] + (1 - done[t]) * gamma * last;  out[t] = last
+ * with reward [T, B, inner], done [T, B], last_state_value [B, inner], all
+ * float32, each operation rounded once, left to right as written there.
+ * Pinned by the reference's known-answer vectors
+ * (tests/st/test_discounted_return.py:39-53).
+ * ---------------------------------------------------------------------- */
+void orc_discounted_return(const float *reward, const unsigned char *done, const float *last_value, float *out,
+                           int64_t timesteps, int64_t batch, int64_t inner, float gamma) {
+    for (int64_t b = 0; b < batch; ++b)
+        for (int64_t i = 0; i < inner; ++i) {
+            float last = last_value[b * inner + i];
+            for (int64_t t = timesteps - 1; t >= 0; --t) {
+                float keep = 1.0f - (done[t * batch + b] ? 1.0f : 0.0f);
+                float scaled = keep * gamma;
+                last = reward[(t * batch + b) * inner + i] + scaled * last;
+                out[(t * batch + b) * inner + i] = last;
+            }
+        }
+}
+
+/* ------------------------------------------------------------------------
  * Reservoir buffer (mindspore_rl/core/reservoir_replay_buffer.py:61-100):
  * Vitter's Algorithm R. The first `capacity` rows fill the slots in order; row
  * number t (0-based) after that draws r uniformly in [0, t] and replaces slot r

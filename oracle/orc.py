@@ -50,6 +50,7 @@ def lib():
         "orc_urb_count": (i64, [vp]),
         "orc_urb_head": (i64, [vp]),
         "orc_urb_field": (vp, [vp, C.c_int]),
+        "orc_discounted_return": (None, [vp, vp, vp, vp, i64, i64, i64, f32]),
         "orc_res_create": (vp, [i64, C.c_int, vp, u64]),
         "orc_res_destroy": (None, [vp]),
         "orc_res_push": (C.c_int, [vp, pvp, i64]),
@@ -91,6 +92,22 @@ def powf_array(x, a):
 def rng_uniform(seed, counter, n):
     L = lib()
     return np.array([L.orc_rng_uniform(seed, counter, k) for k in range(n)], np.float32)
+
+
+def discounted_return(reward, done, last_state_value, gamma):
+    """CPU twin of DiscountedReturn (mindspore_rl/utils/discounted_return.py:84-92).
+    reward [T, B, ...] float32, done [T, B] bool, last_state_value [B, ...] float32."""
+    r = np.ascontiguousarray(reward, np.float32)
+    d = np.ascontiguousarray(done, np.bool_)
+    v = np.ascontiguousarray(last_state_value, np.float32)
+    t = r.shape[0]
+    batch = d.shape[1] if d.ndim > 1 else 1
+    inner = r.size // (t * batch) if t * batch else 1
+    assert d.size == t * batch and v.size == batch * inner
+    out = np.empty_like(r)
+    lib().orc_discounted_return(r.ctypes.data, d.ctypes.data, v.ctypes.data, out.ctypes.data, t, batch, inner,
+                                float(np.float32(gamma)))
+    return out
 
 
 def _field_bytes(shapes, dtypes):

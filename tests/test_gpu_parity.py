@@ -99,6 +99,35 @@ def test_uniform_successive_samples_differ_and_errors(mrb):
         mrb.URB(1, 0, [(1,)], [torch.int32])
 
 
+# --------------------------------------------------------- discounted return
+def test_discounted_return_reference_vectors(mrb):
+    """tests/st/test_discounted_return.py:39-53 on the HIP kernel."""
+    from mindrl_amd.utils import DiscountedReturn
+    net = DiscountedReturn(gamma=0.99)
+    ret = net(torch.tensor([[1.], [1.], [1.], [1.]]), torch.tensor([[False], [False], [True], [False]]),
+              torch.tensor([2.]))
+    assert np.allclose(t2n(ret), np.array([[2.9701], [1.99], [1.], [2.98]], dtype=np.float32))
+    ret = net(torch.tensor([1., 1., 1., 1.]), torch.tensor([False, True, False, True]), torch.tensor(2.))
+    assert np.allclose(t2n(ret), np.array([1.99, 1, 1.99, 1.], dtype=np.float32))
+    with pytest.raises(ValueError, match="range"):
+        DiscountedReturn(gamma=1.5)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 1, 1), (37, 3, 1), (100, 64, 5), (1000, 256, 1), (9, 1000, 17)])
+def test_discounted_return_bit_exact(mrb, orc, shape):
+    from mindrl_amd.utils import DiscountedReturn
+    t, b, inner = shape
+    rng = np.random.default_rng(t * 7 + b)
+    r = rng.normal(size=(t, b, inner)).astype(np.float32)
+    d = rng.random((t, b)) < 0.05
+    v = rng.normal(size=(b, inner)).astype(np.float32)
+    for gamma in (0.0, 0.9, 0.99, 1.0):
+        got = t2n(DiscountedReturn(gamma)(torch.from_numpy(r).cuda(), torch.from_numpy(d).cuda(),
+                                          torch.from_numpy(v).cuda()))
+        want = orc.discounted_return(r, d, v, gamma)
+        assert got.shape == r.shape and np.array_equal(got.view(np.int32), want.view(np.int32)), gamma
+
+
 # -------------------------------------------------------------- n-step buffer
 class OracleNStep:
     """The reference's NStepBuffer, line for line, over two oracle ring buffers

@@ -24,7 +24,7 @@ def declared_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = declared_symbols()
-    assert len(names) == 31
+    assert len(names) == 32
     L = _lib.lib()
     for n in names:
         assert hasattr(L, n), "libmrb.so does not export %s" % n
@@ -101,7 +101,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
         kernels[name] = (int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
-    assert len(kernels) == 10, sorted(kernels)
+    assert len(kernels) == 11, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)

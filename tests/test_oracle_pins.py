@@ -427,3 +427,41 @@ def test_reservoir_reference_scenario(orc):
     assert not np.array_equal(idx, idx2) and idx.min() >= 0 and idx.max() < 100
     with pytest.raises(ValueError):
         orc.OracleReservoir(4, [(1,)], [np.int32]).sample(2)  # empty
+
+
+# --------------------------------------------------------- discounted return
+def test_discounted_return_reference_known_answers(orc):
+    """The reference's own vectors (tests/st/test_discounted_return.py:39-53)."""
+    ret = orc.discounted_return(np.ones((4, 1), np.float32), [[False], [False], [True], [False]], [2.0], 0.99)
+    assert np.allclose(ret, np.array([[2.9701], [1.99], [1.0], [2.98]], np.float32))
+    ret = orc.discounted_return(np.ones(4, np.float32), np.array([False, True, False, True])[:, None], [2.0], 0.99)
+    assert np.allclose(ret, np.array([1.99, 1.0, 1.99, 1.0], np.float32))
+
+
+def test_discounted_return_closed_forms(orc):
+    rng = np.random.default_rng(4)
+    t, b, inner = 50, 7, 3
+    r = rng.normal(size=(t, b, inner)).astype(np.float32)
+    v = rng.normal(size=(b, inner)).astype(np.float32)
+    none = np.zeros((t, b), bool)
+    # gamma 0: the return is the reward; gamma 1 without episode ends: reversed running sum plus the bootstrap
+    assert np.array_equal(orc.discounted_return(r, none, v, 0.0), r)
+    want = np.cumsum(r[::-1].astype(np.float64), 0)[::-1] + v
+    np.testing.assert_allclose(orc.discounted_return(r, none, v, 1.0), want, rtol=1e-5, atol=1e-5)
+    # general: float64 evaluation of the definition, episode ends cutting the bootstrap
+    d = rng.random((t, b)) < 0.1
+    g = 0.97
+    want = np.zeros((t, b, inner))
+    last = v.astype(np.float64)
+    for step in range(t - 1, -1, -1):
+        last = r[step] + (1 - d[step])[:, None] * g * last
+        want[step] = last
+    np.testing.assert_allclose(orc.discounted_return(r, d, v, g), want, rtol=1e-5, atol=1e-5)
+    # a done at step s makes everything at or before s independent of what follows
+    d2 = none.copy()
+    d2[20] = True
+    a1 = orc.discounted_return(r, d2, v, g)
+    r2 = r.copy()
+    r2[21:] += 5.0
+    a2 = orc.discounted_return(r2, d2, v * 3, g)
+    assert np.array_equal(a1[:21], a2[:21]) and not np.array_equal(a1[21:], a2[21:])
