@@ -811,7 +811,7 @@ __global__ __launch_bounds__(kWG) void k_discounted_return(const float* __restri
                                                            const float* __restrict__ last_value,
                                                            float* __restrict__ out, int64_t timesteps, int64_t batch,
                                                            int64_t inner, float gamma) {
-    constexpr int UNROLL = 8;
+    constexpr int UNROLL = 32;
     const int64_t cols = batch * inner;
     const int64_t c = (int64_t)blockIdx.x * kWG + threadIdx.x;
     if (c >= cols) return;
