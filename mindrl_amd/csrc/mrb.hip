@@ -168,6 +168,8 @@ struct Per {
     float* mn = nullptr;
     unsigned long long* stamp = nullptr;
     float* maxp = nullptr;
+    float* powered = nullptr;  // scratch of the last update_priorities call, grown on demand
+    int64_t powered_cap = 0;
     uint32_t* err = nullptr;
     uint32_t* dirty[kMaxRounds] = {};
     int nrounds = 0;
@@ -181,6 +183,7 @@ struct Per {
         if (mn) (void)hipFree(mn);
         if (stamp) (void)hipFree(stamp);
         if (maxp) (void)hipFree(maxp);
+        if (powered) (void)hipFree(powered);
         if (err) (void)hipFree(err);
         for (auto* d : dirty)
             if (d) (void)hipFree(d);
@@ -559,9 +562,19 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     if (n > 0xffffffffll) return fail(MRB_EINVAL, "n %lld exceeds 2^32 - 1 entries per call", (long long)n);
     if (!indices || !priorities) return fail(MRB_EINVAL, "indices or priorities is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (n > b->powered_cap) {
+        // hipFree waits for the device, so no kernel still reads the old scratch
+        if (b->powered) HIP_TRY(hipFree(b->powered));
+        b->powered = nullptr;
+        b->powered_cap = 0;
+        const int64_t want = n > 4096 ? n : 4096;
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->powered), (size_t)want * sizeof(float)));
+        b->powered_cap = want;
+    }
     int rc = next_epoch(*b, s);
     if (rc) return rc;
     UpdateArgs a = update_args(*b);
+    a.powered = b->powered;
     a.indices = indices;
     a.priorities = priorities;
     a.n = n;

@@ -610,6 +610,7 @@ struct UpdateArgs {
     unsigned long long* stamp;  // [leaves]
     float* sum;
     float* mn;
+    float* powered;  // [n] priorities^alpha of this call's entries (update_priorities only)
     float* maxp;  // running max priority (device scalar)
     uint32_t* err;
     // rebuild plan: round r starts at depth lo[r] and rebuilds g[r] levels; the top starts at top_depth
@@ -634,6 +635,7 @@ __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
         if (idx_ok && valid_priority(p)) {
             q = powf_det(p, a.alpha);
             if (a.indices) {
+                a.powered[j] = q;
                 atomicMax(&a.stamp[idx], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
                 if (a.nrounds) a.dirty[0][idx >> a.g[0]] = a.epoch;
             }
@@ -653,7 +655,7 @@ __device__ __forceinline__ bool leaf_value(const UpdateArgs& a, int64_t leaf, fl
     if (a.indices) {
         const unsigned long long st = a.stamp[leaf];
         if ((uint32_t)(st >> 32) != a.epoch) return false;
-        q = powf_det(a.priorities[(uint32_t)st], a.alpha);
+        q = a.powered[(uint32_t)st];  // p^alpha of the winning entry, computed by k_update_stamp with full waves
         return true;
     }
     if (leaf >= a.capacity) return false;
