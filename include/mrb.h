@@ -166,6 +166,25 @@ int mrb_res_field_ptr(int64_t h, int field, void **dev_ptr);
 /* Replaces ReservoirReplayBufferDestroy (reservoir_replay_buffer.py:66,91-100). */
 int mrb_res_destroy(int64_t h);
 
+/* ---- checkpoint hooks ----------------------------------------------------- */
+
+/* Host-side bookkeeping of a buffer as int64[4], for saving a buffer and loading it into a fresh one
+ * of the same construction (the reference never persists its buffers; the row data itself is reached
+ * through the *_field_ptr views):
+ *   uniform   {count, head, seed, calls}      prioritized {size, pushes, seed, calls}
+ *   reservoir {size, total, seed, calls}
+ * set_counters validates the values against the capacity. */
+int mrb_urb_get_counters(int64_t h, int64_t *out4);
+int mrb_urb_set_counters(int64_t h, const int64_t *in4);
+int mrb_per_get_counters(int64_t h, int64_t *out4);
+int mrb_per_set_counters(int64_t h, const int64_t *in4);
+int mrb_res_get_counters(int64_t h, int64_t *out4);
+int mrb_res_set_counters(int64_t h, const int64_t *in4);
+/* Sets the leaves of slots [0, n) of both trees to `leaves` (device f32[n], values as stored, i.e.
+ * already raised to alpha), every other leaf to empty (sum 0, min FLT_MAX), rebuilds all internal
+ * nodes and sets the running max priority. */
+int mrb_per_load_leaves(int64_t h, const float *leaves, int64_t n, float max_priority, void *stream);
+
 /* ---- discounted return --------------------------------------------------- */
 
 /* Replaces the fused DiscountedReturn primitive and the loop it stands for

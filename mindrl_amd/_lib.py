@@ -49,6 +49,13 @@ SIGNATURES = {
     "mrb_res_state": [_i64, _pi64, _pi64],
     "mrb_res_field_ptr": [_i64, _int, _pvp],
     "mrb_res_destroy": [_i64],
+    "mrb_urb_get_counters": [_i64, _pi64],
+    "mrb_urb_set_counters": [_i64, _pi64],
+    "mrb_per_get_counters": [_i64, _pi64],
+    "mrb_per_set_counters": [_i64, _pi64],
+    "mrb_res_get_counters": [_i64, _pi64],
+    "mrb_res_set_counters": [_i64, _pi64],
+    "mrb_per_load_leaves": [_i64, _vp, _i64, _f32, _vp],
     "mrb_discounted_return": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp],
 }
 

@@ -109,3 +109,29 @@ class FieldLayout:
 
 def pointers(tensors):
     return _lib.ptr_array([t.data_ptr() for t in tensors])
+
+
+def get_counters(fn, handle):
+    arr = (C.c_int64 * 4)()
+    _lib.check(fn(handle, arr))
+    return [int(v) for v in arr]
+
+
+def set_counters(fn, handle, values):
+    arr = (C.c_int64 * 4)(*[int(v) - (1 << 64) if int(v) >= (1 << 63) else int(v) for v in values])
+    _lib.check(fn(handle, arr))
+
+
+def save_fields(views, nrows):
+    """Host copies of the first `nrows` rows of each field's storage."""
+    return [v[:nrows].cpu() for v in views]
+
+
+def load_fields(views, saved, layout):
+    if len(saved) != len(views):
+        raise ValueError("state holds %d fields, buffer has %d" % (len(saved), len(views)))
+    for v, t, shape, dtype in zip(views, saved, layout.shapes, layout.dtypes):
+        t = torch.as_tensor(t)
+        if tuple(t.shape[1:]) != shape or t.dtype != dtype or t.shape[0] > v.shape[0]:
+            raise ValueError("saved field %s %s does not fit storage %s %s" % (tuple(t.shape), t.dtype, tuple(v.shape), dtype))
+        v[: t.shape[0]].copy_(t)

@@ -7,7 +7,8 @@ import numpy as np
 import torch
 
 from .. import _lib
-from ._rows import FieldLayout, device, pointers, stream_ptr, view_of
+from ._rows import (FieldLayout, device, get_counters, load_fields, pointers, save_fields, set_counters, stream_ptr,
+                    view_of)
 
 
 class PriorityReplayBuffer:
@@ -153,6 +154,33 @@ class PriorityReplayBuffer:
             _lib.check(_lib.lib().mrb_per_field_ptr(self._h, i, C.byref(p)))
             views.append(view_of(p.value, (self._capacity,) + s, d, self, self._dev))
         return tuple(views)
+
+    def state_dict(self):
+        """Everything needed to rebuild this buffer: rows, the leaves of the sum tree (internal nodes
+        are rebuilt on load, which reproduces them bit for bit), size, pushes, running max priority and
+        the generator's position. (The reference never persists its buffers; this is this library's
+        own format.)"""
+        size, pushes, seed, calls = get_counters(_lib.lib().mrb_per_get_counters, self._h)
+        sum_heap, _ = self.export_tree()
+        leaves = sum_heap.size // 2
+        return {"kind": "priority", "capacity": self._capacity, "alpha": self._alpha, "size": size, "pushes": pushes,
+                "seed": seed & ((1 << 64) - 1), "calls": calls, "max_priority": float(self.max_priority),
+                "leaves": torch.from_numpy(sum_heap[leaves:leaves + size].copy()),
+                "fields": save_fields(self.storage(), size)}
+
+    def load_state_dict(self, state):
+        """Restores a state_dict() taken from a buffer of the same capacity, alpha, shapes and types."""
+        if state.get("kind") != "priority" or state["capacity"] != self._capacity:
+            raise ValueError("state does not belong to a PriorityReplayBuffer of capacity %d" % self._capacity)
+        load_fields(self.storage(), state["fields"], self._layout)
+        leaves = torch.as_tensor(state["leaves"]).to(device=self._dev, dtype=torch.float32).contiguous()
+        if leaves.numel() != state["size"]:
+            raise ValueError("state holds %d leaves for %d rows" % (leaves.numel(), state["size"]))
+        set_counters(_lib.lib().mrb_per_set_counters, self._h,
+                     [state["size"], state["pushes"], state["seed"], state["calls"]])
+        _lib.check(_lib.lib().mrb_per_load_leaves(self._h, leaves.data_ptr() if leaves.numel() else None,
+                                                  leaves.numel(), float(state["max_priority"]), stream_ptr()))
+        torch.cuda.current_stream().synchronize()
 
     def check(self):
         """Synchronises; raises if a kernel recorded a data error since the last check."""

@@ -6,7 +6,8 @@ import os
 import torch
 
 from .. import _lib
-from ._rows import FieldLayout, device, pointers, stream_ptr, view_of
+from ._rows import (FieldLayout, device, get_counters, load_fields, pointers, save_fields, set_counters, stream_ptr,
+                    view_of)
 
 
 class ReservoirReplayBuffer:
@@ -75,6 +76,22 @@ class ReservoirReplayBuffer:
         s, t = C.c_int64(0), C.c_int64(0)
         _lib.check(_lib.lib().mrb_res_state(self._h, C.byref(s), C.byref(t)))
         return s.value, t.value
+
+    def state_dict(self):
+        """Rows, size, rows ever pushed and the generator's position (this library's own format; the
+        reference never persists its buffers)."""
+        torch.cuda.current_stream().synchronize()
+        size, total, seed, calls = get_counters(_lib.lib().mrb_res_get_counters, self._h)
+        return {"kind": "reservoir", "capacity": self._capacity, "size": size, "total": total,
+                "seed": seed & ((1 << 64) - 1), "calls": calls, "fields": save_fields(self.storage(), size)}
+
+    def load_state_dict(self, state):
+        """Restores a state_dict() taken from a buffer of the same capacity, shapes and types."""
+        if state.get("kind") != "reservoir" or state["capacity"] != self._capacity:
+            raise ValueError("state does not belong to a ReservoirReplayBuffer of capacity %d" % self._capacity)
+        load_fields(self.storage(), state["fields"], self._layout)
+        set_counters(_lib.lib().mrb_res_set_counters, self._h,
+                     [state["size"], state["total"], state["seed"], state["calls"]])
 
     def storage(self):
         """Views of the row storage, one [capacity, *shape_i] tensor per field."""

@@ -6,7 +6,8 @@ import numpy as np
 import torch
 
 from .. import _lib
-from ._rows import FieldLayout, device, pointers, stream_ptr, view_of
+from ._rows import (FieldLayout, device, get_counters, load_fields, pointers, save_fields, set_counters, stream_ptr,
+                    view_of)
 
 
 class UniformReplayBuffer:
@@ -120,6 +121,23 @@ class UniformReplayBuffer:
         _lib.check(_lib.lib().mrb_urb_check(self._h, C.byref(flags), stream_ptr()))
         if flags.value:
             raise IndexError("UniformReplayBuffer: index outside [0, count) (flags=%d)" % flags.value)
+
+    def state_dict(self):
+        """Everything needed to rebuild this buffer: rows, count, head and the generator's position.
+        (The reference never persists its buffers; this is this library's own format.)"""
+        torch.cuda.current_stream().synchronize()
+        count, head, seed, calls = get_counters(_lib.lib().mrb_urb_get_counters, self._h)
+        nrows = self._capacity if (head != 0 or count == self._capacity) else count
+        return {"kind": "uniform", "capacity": self._capacity, "count": count, "head": head,
+                "seed": seed & ((1 << 64) - 1), "calls": calls, "fields": save_fields(self.buffer, nrows)}
+
+    def load_state_dict(self, state):
+        """Restores a state_dict() taken from a buffer of the same capacity, shapes and types."""
+        if state.get("kind") != "uniform" or state["capacity"] != self._capacity:
+            raise ValueError("state does not belong to a UniformReplayBuffer of capacity %d" % self._capacity)
+        load_fields(self.buffer, state["fields"], self._layout)
+        set_counters(_lib.lib().mrb_urb_set_counters, self._h,
+                     [state["count"], state["head"], state["seed"], state["calls"]])
 
     def _state(self):
         c, h = C.c_int32(0), C.c_int32(0)

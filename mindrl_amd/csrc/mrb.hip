@@ -780,6 +780,88 @@ int mrb_res_destroy(int64_t h) {
     return MRB_OK;
 }
 
+/* -------------------------------------------------------- checkpoint hooks */
+
+int mrb_urb_get_counters(int64_t h, int64_t* out4) {
+    GET_URB(b, h);
+    if (!out4) return fail(MRB_EINVAL, "out4 is NULL");
+    out4[0] = b->count, out4[1] = b->head, out4[2] = (int64_t)b->seed, out4[3] = (int64_t)b->calls;
+    return MRB_OK;
+}
+
+int mrb_urb_set_counters(int64_t h, const int64_t* in4) {
+    GET_URB(b, h);
+    if (!in4) return fail(MRB_EINVAL, "in4 is NULL");
+    const int64_t cap = b->rows.capacity;
+    if (in4[0] < 0 || in4[0] > cap || in4[1] < 0 || in4[1] >= cap)
+        return fail(MRB_EINVAL, "count %lld / head %lld do not fit capacity %lld", (long long)in4[0], (long long)in4[1],
+                    (long long)cap);
+    b->count = in4[0], b->head = in4[1], b->seed = (uint64_t)in4[2], b->calls = (uint64_t)in4[3];
+    return MRB_OK;
+}
+
+int mrb_per_get_counters(int64_t h, int64_t* out4) {
+    GET_PER(b, h);
+    if (!out4) return fail(MRB_EINVAL, "out4 is NULL");
+    out4[0] = b->size, out4[1] = b->pushes, out4[2] = (int64_t)b->seed, out4[3] = (int64_t)b->calls;
+    return MRB_OK;
+}
+
+int mrb_per_set_counters(int64_t h, const int64_t* in4) {
+    GET_PER(b, h);
+    if (!in4) return fail(MRB_EINVAL, "in4 is NULL");
+    const int64_t cap = b->rows.capacity;
+    const int64_t want = in4[1] < cap ? in4[1] : cap;
+    if (in4[1] < 0 || in4[0] != want)
+        return fail(MRB_EINVAL, "size %lld does not follow from %lld pushes into capacity %lld", (long long)in4[0],
+                    (long long)in4[1], (long long)cap);
+    b->size = in4[0], b->pushes = in4[1], b->seed = (uint64_t)in4[2], b->calls = (uint64_t)in4[3];
+    return MRB_OK;
+}
+
+int mrb_res_get_counters(int64_t h, int64_t* out4) {
+    GET_RES(b, h);
+    if (!out4) return fail(MRB_EINVAL, "out4 is NULL");
+    out4[0] = b->size, out4[1] = b->total, out4[2] = (int64_t)b->seed, out4[3] = (int64_t)b->calls;
+    return MRB_OK;
+}
+
+int mrb_res_set_counters(int64_t h, const int64_t* in4) {
+    GET_RES(b, h);
+    if (!in4) return fail(MRB_EINVAL, "in4 is NULL");
+    const int64_t cap = b->rows.capacity;
+    const int64_t want = in4[1] < cap ? in4[1] : cap;
+    if (in4[1] < 0 || in4[0] != want)
+        return fail(MRB_EINVAL, "size %lld does not follow from %lld rows pushed into capacity %lld", (long long)in4[0],
+                    (long long)in4[1], (long long)cap);
+    b->size = in4[0], b->total = in4[1], b->seed = (uint64_t)in4[2], b->calls = (uint64_t)in4[3];
+    return MRB_OK;
+}
+
+int mrb_per_load_leaves(int64_t h, const float* leaves, int64_t n, float max_priority, void* stream) {
+    GET_PER(b, h);
+    if (n < 0 || n > b->rows.capacity) return fail(MRB_EINVAL, "n %lld outside [0, capacity]", (long long)n);
+    if (n > 0 && !leaves) return fail(MRB_EINVAL, "leaves is NULL");
+    if (!(max_priority >= 0.0f) || max_priority > 3.0e38f) return fail(MRB_EINVAL, "max_priority %g is not a priority", (double)max_priority);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t nodes = 2 * (size_t)b->leaves;
+    HIP_TRY(hipMemsetAsync(b->sum, 0, nodes * sizeof(float), s));
+    hipLaunchKernelGGL(k_fill_f32, dim3(grid_for(nodes)), dim3(kWG), 0, s, b->mn, FLT_MAX, (uint64_t)nodes);
+    LAUNCH_CHECK("k_fill_f32");
+    HIP_TRY(hipMemcpyAsync(b->maxp, &max_priority, sizeof(float), hipMemcpyHostToDevice, s));
+    HIP_TRY(hipStreamSynchronize(s));  // max_priority lives on this stack frame
+    if (n == 0) return MRB_OK;
+    int rc = next_epoch(*b, s);
+    if (rc) return rc;
+    // a push of slots [0, n) whose priorities are taken as they are: x^1 == x exactly
+    UpdateArgs a = update_args(*b);
+    a.alpha = 1.0f;
+    a.priorities = leaves;
+    a.first_slot = 0;
+    a.n = n;
+    return tree_rebuild(*b, a, s);
+}
+
 /* ------------------------------------------------------- discounted return */
 
 int mrb_discounted_return(const float* reward, const uint8_t* done, const float* last_value, float* out,

@@ -99,6 +99,72 @@ def test_uniform_successive_samples_differ_and_errors(mrb):
         mrb.URB(1, 0, [(1,)], [torch.int32])
 
 
+# ------------------------------------------------------------------ checkpoint
+def test_state_dict_round_trip_continues_identically(mrb, tmp_path):
+    """A buffer restored from state_dict() (through torch.save / torch.load(weights_only=True)) into a
+    fresh buffer behaves exactly like the original from then on: same storage, same trees, same draws."""
+    rng = np.random.default_rng(77)
+    shapes, dtypes = [(5,), (1,)], [np.float32, np.int32]
+
+    def reload(state):
+        torch.save(state, tmp_path / "buf.pt")
+        return torch.load(tmp_path / "buf.pt", weights_only=True)
+
+    # prioritized: wrapped ring, updated priorities, generator advanced
+    a = mrb.PER(0.6, 300, 16, shapes, torch_types(dtypes), seed0=5)
+    a.insert(*to_dev(random_rows(rng, 450, shapes, dtypes)))
+    a.update_priorities(torch.from_numpy(rng.integers(0, 300, 200)).cuda(),
+                        torch.from_numpy(rng.pareto(1.5, 200).astype(np.float32) + 1e-6).cuda())
+    a.sample(0.4)
+    b = mrb.PER(0.6, 300, 16, shapes, torch_types(dtypes), seed0=999)
+    b.load_state_dict(reload(a.state_dict()))
+    for step in range(5):
+        sa, sb = a.export_tree(), b.export_tree()
+        assert np.array_equal(bits(sa[0][1:]), bits(sb[0][1:])) and np.array_equal(bits(sa[1][1:]), bits(sb[1][1:]))
+        assert a.max_priority == b.max_priority and a._state()[:2] == b._state()[:2]
+        oa, ob = a.sample(0.7), b.sample(0.7)
+        for x, y in zip(oa, ob):
+            assert torch.equal(x, y)
+        rows = to_dev(random_rows(rng, 7, shapes, dtypes))
+        a.insert(*rows), b.insert(*rows)
+        a.update_priorities(oa[0], oa[1] + 0.5), b.update_priorities(ob[0], ob[1] + 0.5)
+    a.destroy(), b.destroy()
+    # an empty prioritized buffer round-trips too
+    e = mrb.PER(0.6, 10, 2, shapes, torch_types(dtypes), seed0=1)
+    f = mrb.PER(0.6, 10, 2, shapes, torch_types(dtypes), seed0=2)
+    f.load_state_dict(reload(e.state_dict()))
+    assert f.size() == 0
+    e.destroy(), f.destroy()
+
+    # uniform: wrapped ring
+    u = mrb.URB(8, 50, shapes, torch_types(dtypes), seed=3)
+    u.insert(to_dev(random_rows(rng, 70, shapes, dtypes)))
+    u.sample()
+    w = mrb.URB(8, 50, shapes, torch_types(dtypes), seed=4)
+    w.load_state_dict(reload(u.state_dict()))
+    assert (int(u.count), int(u.head)) == (int(w.count), int(w.head)) == (50, 20)
+    for x, y in zip(u.sample(), w.sample()):
+        assert torch.equal(x, y)
+    for x, y in zip(u.get_item(0), w.get_item(0)):
+        assert torch.equal(x, y)
+    with pytest.raises(ValueError):
+        mrb.URB(8, 51, shapes, torch_types(dtypes)).load_state_dict(u.state_dict())
+    u.destroy(), w.destroy()
+
+    # reservoir: past capacity
+    r = mrb.RES(20, 8, shapes, torch_types(dtypes), seed1=6)
+    r.push(*to_dev(random_rows(rng, 90, shapes, dtypes)))
+    q = mrb.RES(20, 8, shapes, torch_types(dtypes), seed1=7)
+    q.load_state_dict(reload(r.state_dict()))
+    more = to_dev(random_rows(rng, 40, shapes, dtypes))
+    r.push(*more), q.push(*more)
+    for x, y in zip(r.storage(), q.storage()):
+        assert torch.equal(x, y)
+    for x, y in zip(r.sample(), q.sample()):
+        assert torch.equal(x, y)
+    r.destroy(), q.destroy()
+
+
 # --------------------------------------------------------- discounted return
 def test_discounted_return_reference_vectors(mrb):
     """tests/st/test_discounted_return.py:39-53 on the HIP kernel."""
