@@ -168,6 +168,11 @@ struct Per {
     float* mn = nullptr;
     unsigned long long* stamp = nullptr;
     float* maxp = nullptr;
+    // sparse plan for very large trees (see k_tree_sparse): lowest s_g0 levels per entry, then s_rounds tile rounds
+    int s_g0 = 0, s_rounds = 0, s_top = 0;
+    int s_lo[kMaxRounds] = {}, s_g[kMaxRounds] = {};
+    uint32_t* s_dirty[kMaxRounds] = {};
+    unsigned long long* owner = nullptr;
     float* powered = nullptr;  // scratch of the last update_priorities call, grown on demand
     int64_t powered_cap = 0;
     uint32_t* err = nullptr;
@@ -184,6 +189,9 @@ struct Per {
         if (stamp) (void)hipFree(stamp);
         if (maxp) (void)hipFree(maxp);
         if (powered) (void)hipFree(powered);
+        if (owner) (void)hipFree(owner);
+        for (auto* d : s_dirty)
+            if (d) (void)hipFree(d);
         if (err) (void)hipFree(err);
         for (auto* d : dirty)
             if (d) (void)hipFree(d);
@@ -267,6 +275,9 @@ int next_epoch(Per& b, hipStream_t s) {
         HIP_TRY(hipMemsetAsync(b.stamp, 0, sizeof(unsigned long long) * (size_t)b.leaves, s));
         for (int r = 0; r < b.nrounds; ++r)
             HIP_TRY(hipMemsetAsync(b.dirty[r], 0, sizeof(uint32_t) * ((size_t)1 << (b.lo[r] - b.g[r])), s));
+        for (int r = 0; r < b.s_rounds; ++r)
+            HIP_TRY(hipMemsetAsync(b.s_dirty[r], 0, sizeof(uint32_t) * ((size_t)1 << (b.s_lo[r] - b.s_g[r])), s));
+        if (b.owner) HIP_TRY(hipMemsetAsync(b.owner, 0, sizeof(unsigned long long) * ((size_t)b.leaves >> b.s_g0), s));
         b.epoch += 1;
     }
     return MRB_OK;
@@ -514,6 +525,25 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
         HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->dirty[r]), nblocks * sizeof(uint32_t)));
         HIP_TRY(hipMemset(b->dirty[r], 0, nblocks * sizeof(uint32_t)));
     }
+    if (b->depth >= 22) {
+        // sparse plan: with >= 16384 leaf tiles a call with few entries is better driven by its entries
+        b->s_g0 = b->depth - 20 < 4 ? 4 : (b->depth - 20 > 6 ? 6 : b->depth - 20);
+        const int d2 = b->depth - b->s_g0;
+        b->s_top = kTopMaxDepth;
+        const int rest2 = d2 - b->s_top;  // >= 4
+        b->s_rounds = (rest2 + kRoundLevels - 1) / kRoundLevels;
+        for (int r = 0, lo = d2; r < b->s_rounds; ++r) {
+            b->s_lo[r] = lo;
+            b->s_g[r] = rest2 / b->s_rounds + (r < rest2 % b->s_rounds ? 1 : 0);
+            lo -= b->s_g[r];
+            const size_t nblocks = (size_t)1 << (b->s_lo[r] - b->s_g[r]);
+            HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->s_dirty[r]), nblocks * sizeof(uint32_t)));
+            HIP_TRY(hipMemset(b->s_dirty[r], 0, nblocks * sizeof(uint32_t)));
+        }
+        const size_t nown = (size_t)b->leaves >> b->s_g0;
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->owner), nown * sizeof(unsigned long long)));
+        HIP_TRY(hipMemset(b->owner, 0, nown * sizeof(unsigned long long)));
+    }
     hipLaunchKernelGGL(k_fill_f32, dim3(grid_for(nodes)), dim3(kWG), 0, nullptr, b->mn, FLT_MAX, (uint64_t)nodes);
     LAUNCH_CHECK("k_fill_f32");
     const float one = 1.0f;
@@ -578,9 +608,32 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     a.indices = indices;
     a.priorities = priorities;
     a.n = n;
+    // Few entries on a very large tree: rebuild the lowest levels per entry, not per tile.
+    const bool sparse = b->s_g0 > 0 && n <= (b->leaves >> 8);
+    if (sparse) {
+        a.sparse_g0 = b->s_g0;
+        a.owner = b->owner;
+        a.nrounds = b->s_rounds;
+        a.top_depth = b->s_top;
+        for (int r = 0; r < kMaxRounds; ++r) {
+            a.dirty[r] = b->s_dirty[r];
+            a.lo[r] = b->s_lo[r];
+            a.g[r] = b->s_g[r];
+        }
+    }
     hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
     LAUNCH_CHECK("k_update_stamp");
-    return tree_rebuild(*b, a, s);
+    if (!sparse) return tree_rebuild(*b, a, s);
+    hipLaunchKernelGGL(k_tree_sparse, dim3(grid_exact((uint64_t)n << (b->s_g0 - 2))), dim3(kWG), 0, s, a);
+    LAUNCH_CHECK("k_tree_sparse");
+    for (int r = 0; r < b->s_rounds; ++r) {
+        const uint32_t tiles = (1u << b->s_lo[r]) / kBlockNodes;
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r);
+        LAUNCH_CHECK("k_tree_update");
+    }
+    hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a);
+    LAUNCH_CHECK("k_tree_top");
+    return MRB_OK;
 }
 
 int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, int64_t* out_indices,

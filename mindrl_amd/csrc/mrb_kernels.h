@@ -619,6 +619,10 @@ struct UpdateArgs {
     int g[kMaxRounds];
     int top_depth;
     uint32_t* dirty[kMaxRounds];  // per round: one epoch word per block of 1 << g[r] nodes at depth lo[r]
+    // sparse updates of very large trees: the lowest sparse_g0 levels are rebuilt per entry
+    // (k_tree_sparse) instead of per tile; owner[block] elects one entry per block of leaves
+    int sparse_g0;               // 0 = not used
+    unsigned long long* owner;   // [leaves >> sparse_g0]
 };
 
 __device__ __forceinline__ bool valid_priority(float p) { return p >= 0.0f && p <= 3.0e38f; }
@@ -637,7 +641,10 @@ __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
             if (a.indices) {
                 a.powered[j] = q;
                 atomicMax(&a.stamp[idx], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
-                if (a.nrounds) a.dirty[0][idx >> a.g[0]] = a.epoch;
+                if (a.sparse_g0)
+                    atomicMax(&a.owner[idx >> a.sparse_g0], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
+                else if (a.nrounds)
+                    a.dirty[0][idx >> a.g[0]] = a.epoch;
             }
         }
     }
@@ -765,6 +772,68 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
         if (active && g >= 3 + s && (lane & ((2u << s) - 1)) == 0) {
             a.sum[(first >> (3 + s)) + (lane >> (s + 1))] = cs;
             a.mn[(first >> (3 + s)) + (lane >> (s + 1))] = cm;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Sparse lowest round for very large trees (e.g. 2^24 leaves, 65,536 entries): scanning
+// every 256-leaf tile costs more in wave launches than the update itself, so here the
+// ENTRIES drive the work. A group of L = 2^(g0-2) lanes (g0 = 4..6) takes one entry; if
+// that entry owns its block of 2^g0 leaves (integer-max election in k_update_stamp), the
+// group loads the block, replaces the leaves the stamps name, rebuilds the g0 levels
+// above with the same pairwise operations as tile_round and marks the next round's block.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kWG) void k_tree_sparse(UpdateArgs a) {
+    const int g0 = a.sparse_g0;
+    const uint32_t group = 1u << (g0 - 2);
+    const uint64_t tid = (uint64_t)blockIdx.x * kWG + threadIdx.x;
+    const int64_t j = (int64_t)(tid >> (g0 - 2));
+    const uint32_t sub = (uint32_t)tid & (group - 1);
+    bool active = j < a.n;
+    int64_t idx = 0;
+    if (active) {
+        idx = a.indices[j];
+        active = idx >= 0 && idx < a.capacity && valid_priority(a.priorities[j]) &&
+                 a.owner[idx >> g0] == (((unsigned long long)a.epoch << 32) | (unsigned long long)j);
+    }
+    const uint64_t block = (uint64_t)idx >> g0;
+    const uint64_t first = (uint64_t)a.leaves + (block << g0);  // heap index of the block's first leaf
+    float4 vs = make_float4(0.f, 0.f, 0.f, 0.f), vm = vs;
+    if (active) {
+        vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * sub);
+        vm = *reinterpret_cast<const float4*>(a.mn + first + 4 * sub);
+        const int64_t leaf0 = (int64_t)((block << g0) + 4 * sub);
+        float q;
+        bool wrote = false;
+        if (leaf_value(a, leaf0 + 0, q)) { vs.x = vm.x = q; wrote = true; }
+        if (leaf_value(a, leaf0 + 1, q)) { vs.y = vm.y = q; wrote = true; }
+        if (leaf_value(a, leaf0 + 2, q)) { vs.z = vm.z = q; wrote = true; }
+        if (leaf_value(a, leaf0 + 3, q)) { vs.w = vm.w = q; wrote = true; }
+        if (wrote) {
+            *reinterpret_cast<float4*>(a.sum + first + 4 * sub) = vs;
+            *reinterpret_cast<float4*>(a.mn + first + 4 * sub) = vm;
+        }
+        if (sub == 0 && a.nrounds) a.dirty[0][block >> a.g[0]] = a.epoch;
+    }
+    const float s0 = vs.x + vs.y, s1 = vs.z + vs.w;
+    const float m0 = fminf(vm.x, vm.y), m1 = fminf(vm.z, vm.w);
+    float cs = s0 + s1, cm = fminf(m0, m1);
+    if (active) {
+        *reinterpret_cast<float2*>(a.sum + (first >> 1) + 2 * sub) = make_float2(s0, s1);
+        *reinterpret_cast<float2*>(a.mn + (first >> 1) + 2 * sub) = make_float2(m0, m1);
+        a.sum[(first >> 2) + sub] = cs;
+        a.mn[(first >> 2) + sub] = cm;
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        if (s < g0 - 2) {  // wave-uniform
+            cs = cs + __shfl_xor(cs, 1 << s);
+            cm = fminf(cm, __shfl_xor(cm, 1 << s));
+            if (active && (sub & ((2u << s) - 1)) == 0) {
+                a.sum[(first >> (3 + s)) + (sub >> (s + 1))] = cs;
+                a.mn[(first >> (3 + s)) + (sub >> (s + 1))] = cm;
+            }
         }
     }
 }

@@ -521,6 +521,38 @@ def test_config5_tree_descent_stress(mrb, orc):
     g.destroy()
 
 
+@pytest.mark.parametrize("cap", [3_000_000, 20_000_000])
+def test_sparse_updates_on_very_large_trees(mrb, orc, cap):
+    """Trees of 22 and 25 levels: updates with few entries take the entry-driven lowest round
+    (groups of 4 and 8 lanes per entry); sizes 1, 1000 (10 % duplicates, some invalid) and 60,000."""
+    shapes, dtypes = [(1,)], [np.uint8]
+    rng = np.random.default_rng(cap % 1000)
+    g, c = make_pair(mrb, orc, 0.6, cap, 256, seed=3, shapes=shapes, dtypes=dtypes)
+    rows = [np.zeros((cap, 1), np.uint8)]
+    pr = rng.lognormal(0, 1, cap).astype(np.float32)
+    g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda())
+    c.push(rows, cap)
+    c.update(np.arange(cap), pr)
+    for n in (1, 1000, 60000, 7):
+        idx = rng.integers(0, cap, n)
+        if n >= 1000:
+            idx[rng.integers(0, n, n // 10)] = idx[rng.integers(0, n, n // 10)]
+        up = rng.pareto(1.5, n).astype(np.float32) + np.float32(1e-6)
+        g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(up).cuda())
+        c.update(idx, up)
+        u = rng.random(256).astype(np.float32)
+        assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(256, 0.5, u), "n %d" % n)
+    assert_tree_equal(g, c, "cap %d" % cap)
+    assert np.float32(g.max_priority) == np.float32(c.max_priority)
+    # invalid entries are skipped and flagged, valid ones in the same call still land
+    g.update_priorities(torch.tensor([5, cap + 3, -1, 9]).cuda(), torch.tensor([2.0, 1.0, 1.0, float("nan")]).cuda())
+    c.update([5], [2.0])
+    with pytest.raises(IndexError):
+        g.check()
+    assert_tree_equal(g, c, "cap %d after invalid entries" % cap)
+    g.destroy()
+
+
 @pytest.mark.parametrize("cap", [1 << 17, 1_000_000])
 def test_config3_atari_shape_properties(mrb, orc, cap):
     """Config 3's rows (u8[84,84,4] + next_idx i64 + action i32 + reward f32 + done bool =
