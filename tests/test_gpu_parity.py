@@ -425,6 +425,47 @@ def test_per_error_paths(mrb):
         mrb.PER(0.6, -5, 4, [(1,)], [torch.int32])
 
 
+@pytest.mark.parametrize("path", [1, 2])
+def test_sixteen_fields_of_odd_sizes(mrb, orc, path):
+    """The maximum of 16 fields, row sizes 1..4100 bytes covering every copy granule (1, 2, 4, 8,
+    16 bytes) and rows that need several passes per workgroup; all three buffer kinds."""
+    sizes = [1, 2, 3, 4, 6, 8, 12, 16, 20, 24, 48, 100, 1000, 4096, 4100, 7]
+    shapes, dtypes = [(n,) for n in sizes], [np.uint8] * len(sizes)
+    shapes[7], dtypes[7] = (4,), np.float32   # 16 bytes
+    shapes[9], dtypes[9] = (3,), np.int64     # 24 bytes
+    rng = np.random.default_rng(16)
+    mrb.lib.set_option("sample_path", path)
+    cap, batch = 300, 40
+    g, c = make_pair(mrb, orc, 0.7, cap, batch, seed=2, shapes=shapes, dtypes=dtypes)
+    u = mrb.URB(batch, cap, shapes, torch_types(dtypes), seed=8)
+    cu = orc.OracleUniform(cap, shapes, dtypes, seed=8)
+    r = mrb.RES(cap, batch, shapes, torch_types(dtypes), seed1=8)
+    cr = orc.OracleReservoir(cap, shapes, dtypes, seed=8)
+    for step in range(6):
+        n = int(rng.integers(1, 250))
+        rows = random_rows(rng, n, shapes, dtypes)
+        dev = to_dev(rows)
+        g.insert(*dev), c.push(rows, n)
+        u.insert(dev), cu.append(rows, n)
+        r.push(*dev), cr.push(rows, n)
+        draws = rng.random(batch).astype(np.float32)
+        assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(draws).cuda()), c.sample(batch, 0.5, draws),
+                            "step %d" % step)
+        ui, uf = u.sample_with_indices()
+        ci, cf = cu.sample(batch)
+        assert np.array_equal(t2n(ui), ci)
+        ri, rf = r.sample(with_indices=True)
+        ki, kf = cr.sample(batch)
+        assert np.array_equal(t2n(ri), ki)
+        for f in range(len(sizes)):
+            assert np.array_equal(t2n(uf[f]).view(np.uint8), cf[f].view(np.uint8)), (step, f)
+            assert np.array_equal(t2n(rf[f]).view(np.uint8), kf[f].view(np.uint8)), (step, f)
+            assert np.array_equal(t2n(u.buffer[f]).view(np.uint8), cu.field(f).view(np.uint8)), (step, f)
+    mrb.lib.set_option("sample_path", 0)
+    for b in (g, u, r):
+        b.destroy()
+
+
 # ------------------------------------------------- BASELINE.json configurations
 def test_config1_dqn_per_cartpole_full_loop(mrb, orc):
     """Config 1: capacity 10 000, alpha .6, beta .4, eps 1e-6; fill, then 1000 x
