@@ -433,7 +433,7 @@ def main():
     flags = buf.check()
 
     # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this very command, scaled by what the
-    # same counters read for the ring-append copy kernel (profiles/k_per_sample_wide_config3_*.md); only valid for
+    # same counters read for the ring-append copy kernel; only valid for
     # the default workload and library defaults.
     traffic = 33.85e6 if (a.workload == "c3" and not a.capacity and not a.row_split and not a.sample_path) else None
     row_bytes = sum(buf._layout.bytes)

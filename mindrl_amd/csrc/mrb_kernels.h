@@ -244,9 +244,8 @@ __global__ __launch_bounds__(kWG) void k_res_put(IoTable t, const unsigned long 
     }
 }
 
-// Arguments common to both sample kernels. Passed first, with the fields that the
-// tree descent needs at the front: the leading kernel-argument dwords are preloaded
-// into scalar registers at wave launch, which saves a dependent fetch.
+// Arguments common to both sample kernels (the wide-row kernel additionally takes the
+// fields its tree descent needs first as plain leading parameters).
 struct SampleArgs {
     const float* sum;       // sum tree, heap order
     const float* uniforms;  // f32[batch] or NULL -> generator
@@ -294,10 +293,10 @@ constexpr int kInFlight = 4;  // granules a thread holds between its loads and i
 
 // ---------------------------------------------------------------------------
 // PER sample, wide rows: `split` workgroups per sampled row. Wave 0 of every
-// workgroup walks the sum tree for its stratum with group_load/group_walk (one
-// dependent load per 10 levels; the first group sits under the root, so its
-// load is issued together with the total and the uniform draw) and publishes
-// the slot through LDS. The workgroup's share of the row — granules of all
+// workgroup walks the sum tree for its stratum with group_request / group_walk
+// (one dependent load per 10 levels; the first group sits under the root, so it
+// is requested together with the total and the uniform draw) and publishes the
+// slot through LDS. The workgroup's share of the row — granules of all
 // fields, numbered consecutively — is then copied with every load issued
 // before the first store, so a row costs one memory round trip, not one per
 // field. The row's first workgroup computes the importance weight while its

@@ -466,7 +466,7 @@ def test_sixteen_fields_of_odd_sizes(mrb, orc, path):
         b.destroy()
 
 
-# ------------------------------------------------- BASELINE.json configurations
+# ----------------------------------------------- the five benchmark configurations
 def test_config1_dqn_per_cartpole_full_loop(mrb, orc):
     """Config 1: capacity 10 000, alpha .6, beta .4, eps 1e-6; fill, then 1000 x
     {sample 64, update with |N(0,1)|+eps, insert 1}. Every step compared."""
