@@ -72,9 +72,12 @@ class FieldLayout:
             raise ValueError("expected %d tensors per element, got %d" % (len(self), len(fields)))
         n = None
         for f, numel in zip(fields, self.numel):
-            total = int(np.prod(tuple(f.shape), dtype=np.int64)) if len(f.shape) else 1
+            if isinstance(f, torch.Tensor):
+                total = f.numel()
+            else:
+                total = int(np.prod(tuple(np.shape(f)), dtype=np.int64)) if len(np.shape(f)) else 1
             if total % numel:
-                raise ValueError("tensor of shape %s does not hold whole elements of %d values" % (tuple(f.shape), numel))
+                raise ValueError("tensor of shape %s does not hold whole elements of %d values" % (tuple(np.shape(f)), numel))
             rows = total // numel
             if n is None:
                 n = rows
@@ -86,9 +89,11 @@ class FieldLayout:
         """Contiguous device tensors of the declared dtypes (copies host data if needed)."""
         out = []
         for f, d in zip(fields, self.dtypes):
+            if isinstance(f, torch.Tensor) and f.is_cuda and f.dtype == d and f.is_contiguous() and f.device == dev:
+                out.append(f)  # the common case: nothing to convert
+                continue
             t = f if isinstance(f, torch.Tensor) else torch.as_tensor(np.asarray(f))
-            t = t.to(device=dev, dtype=d, non_blocking=False).contiguous()
-            out.append(t)
+            out.append(t.to(device=dev, dtype=d, non_blocking=False).contiguous())
         return out
 
     def empty(self, n, dev):
