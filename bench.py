@@ -496,6 +496,34 @@ def main():
             L.mrb_per_push(h, sptr, ins_n, None, sp)
         torch.cuda.synchronize()
         extras["loop_steps_per_s"] = n_it / (time.perf_counter() - t0)
+        # Reference points for the sample kernel on the same storage and output buffers: what a copy of the same
+        # number of bytes costs per launch, with and without the random row addresses, and without any tree work.
+        big = max(range(len(fields)), key=lambda i: fields[i].numel() * fields[i].element_size())
+        store = buf.storage()[big]
+        dst = fields[big]
+        n_it = 500
+
+        def per_launch(fn):
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n_it):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / n_it
+
+        step(W)
+        torch.cuda.synchronize()
+        sampled = idx.clone()  # a real set of sampled slots
+        extras["ceiling_contiguous_copy_us"] = per_launch(lambda: dst.copy_(store[:batch]))
+        extras["ceiling_index_select_us"] = per_launch(lambda: torch.index_select(store, 0, sampled, out=dst))
+        extras["ceiling_bytes"] = 2 * dst.numel() * dst.element_size()
+        # the library's own gather at given slots (no tree work): the optional next_obs dereference of config 3
+        L.mrb_per_gather(h, sampled.data_ptr(), batch, fptr, sp)
+        extras["gather_at_given_slots_us"] = per_launch(lambda: L.mrb_per_gather(h, sampled.data_ptr(), batch, fptr, sp))
         out["extras"] = extras
 
     if not a.no_cpu_baseline:

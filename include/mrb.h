@@ -134,6 +134,12 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float *uniforms, 
  * duplicates), every ancestor of a touched leaf recomputed from its final
  * children; max priority = max(old, all priorities[j]^alpha). */
 int mrb_per_update(int64_t h, const int64_t *indices, const float *priorities, int64_t n, void *stream);
+/* Rows at the given physical slots (device int64[n], each in [0, size)), gathered like mrb_urb_gather:
+ * dst_fields[i][k] = storage_i[indices[k]]. No counterpart among the reference's primitives; it serves
+ * transitions that store a slot number instead of a copy of the next observation (a frame-shared
+ * next_obs index): the caller samples, then gathers field rows at the sampled next_idx values.
+ * Out-of-range slots are clamped and reported by mrb_per_check (MRB_DERR_INDEX). */
+int mrb_per_gather(int64_t h, const int64_t *indices, int64_t n, void *const *dst_fields, void *stream);
 /* Parity hook: copies both trees in canonical heap order (root at 1, leaf i at
  * leaves + i, element 0 unused) to HOST arrays of 2 * leaves floats each.
  * Either pointer may be NULL. Synchronises `stream`. */

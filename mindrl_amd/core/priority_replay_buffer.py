@@ -100,6 +100,17 @@ class PriorityReplayBuffer:
         self._keep = (idx, pr)
         return self._handle
 
+    def gather(self, indices, out=None):
+        """Rows at the given slots (int64, each in [0, size)): one [n, *shape_i] tensor per field.
+        For transitions that store the slot of their successor instead of a copy of it, e.g.
+        `next_rows = buf.gather(sampled_next_idx)`."""
+        idx = torch.as_tensor(indices).to(device=self._dev, dtype=torch.int64).contiguous().reshape(-1)
+        n = idx.numel()
+        dst = self._layout.check_out(out, n, self._dev) if out is not None else self._layout.empty(n, self._dev)
+        _lib.check(_lib.lib().mrb_per_gather(self._h, idx.data_ptr(), n, pointers(dst), stream_ptr()))
+        self._keep = idx
+        return tuple(dst)
+
     def full(self):
         """Always False, as in the reference (priority_replay_buffer.py:122-124)."""
         return torch.tensor(False)

@@ -696,6 +696,21 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, 
     return MRB_OK;
 }
 
+int mrb_per_gather(int64_t h, const int64_t* indices, int64_t n, void* const* dst_fields, void* stream) {
+    GET_PER(b, h);
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (!indices) return fail(MRB_EINVAL, "indices is NULL");
+    if (b->size <= 0) return fail(MRB_ESTATE, "gather from an empty buffer");
+    IoTable t;
+    int rc = make_table(b->rows, dst_fields, n, t);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0,
+                       static_cast<hipStream_t>(stream), t, b->rows.capacity, b->size, indices, (int64_t)-1,
+                       (uint64_t)0, (uint64_t)0, static_cast<int64_t*>(nullptr), b->err);
+    LAUNCH_CHECK("k_rows_gather");
+    return MRB_OK;
+}
+
 int mrb_per_export_tree(int64_t h, float* sum_heap, float* min_heap, int64_t* leaves, void* stream) {
     GET_PER(b, h);
     hipStream_t s = static_cast<hipStream_t>(stream);

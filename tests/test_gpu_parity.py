@@ -627,6 +627,10 @@ def test_config3_atari_shape_properties(mrb, orc, cap):
         ci, cw, cf = c.sample(batch, beta, u)
         assert_sample_equal((out[0], out[1]) + tuple(out[3:]), (ci, cw, cf), "step %d" % step)
         assert torch.equal(out[2], store[0].index_select(0, out[0]))
+        # dereference of the frame-shared next_obs index: rows gathered at the sampled next_idx values
+        nxt = g.gather(out[3].reshape(-1))
+        assert torch.equal(nxt[0], store[0].index_select(0, out[3].reshape(-1)))
+        assert np.array_equal(t2n(nxt[1]), c.field(0)[cf[0].reshape(-1)])
         td = (np.abs(rng.normal(size=batch)) + 1e-6).astype(np.float32)
         g.update_priorities(out[0], torch.from_numpy(td).cuda())
         c.update(ci, td)
