@@ -130,6 +130,64 @@ int rows_put(const RowStore& r, const void* const* src, int64_t skip, int64_t n,
     return MRB_OK;
 }
 
+// Workgroups per row for the wide-row kernel: one pass of kInFlight granules per thread covers the
+// widest field (measured best on 28 KB rows: 2 workgroups per row).
+int wide_split(const RowStore& r) {
+    if (g_opt.row_split > 0) return (int)g_opt.row_split;
+    uint32_t max_units = 0;
+    for (int i = 0; i < r.nfields; ++i)
+        if (r.units[i] > max_units) max_units = r.units[i];
+    int split = (int)((max_units + kInFlight * kWG - 1) / (kInFlight * kWG));
+    return split < 1 ? 1 : (split > 16 ? 16 : split);
+}
+
+int64_t widest_field(const RowStore& r) {
+    int64_t m = 0;
+    for (int i = 0; i < r.nfields; ++i)
+        if (r.bytes[i] > m) m = r.bytes[i];
+    return m;
+}
+
+int launch_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, hipStream_t s) {
+    SplitPlan plan{};
+    plan.split = wide_split(r);
+    for (int i = 0; i < r.nfields; ++i) plan.per[i] = (r.units[i] + plan.split - 1) / plan.split;
+    hipLaunchKernelGGL(k_per_sample_wide, dim3((uint32_t)(a.batch * plan.split)), dim3(kWG), 0, s, a.sum, a.uniforms,
+                       a.depth, plan.split, a.batch, a.seed, a.calls, a, t, plan);
+    LAUNCH_CHECK("k_per_sample_wide");
+    return MRB_OK;
+}
+
+// Gather of n rows whose slots are given (indices), drawn from the generator (indices NULL,
+// fixed_slot < 0) or one fixed slot. Rows of at least 1 KB go through the wide-row kernel
+// (a workgroup per row part, all loads before the first store), narrow rows through the
+// flat kernel.
+int gather_rows(const RowStore& r, const int64_t* indices, int64_t fixed_slot, int64_t count, uint64_t seed,
+                uint64_t calls, int64_t n, int64_t* out_indices, void* const* dst_fields, uint32_t* err,
+                hipStream_t s) {
+    IoTable t;
+    int rc = make_table(r, dst_fields, n, t);
+    if (rc) return rc;
+    if (widest_field(r) >= 1024 && n <= (1ll << 24)) {
+        SampleArgs a{};
+        a.batch = n;
+        a.seed = seed;
+        a.calls = calls;
+        a.capacity = r.capacity;
+        a.out_idx = out_indices;
+        a.err = err;
+        a.mode = fixed_slot >= 0 ? kFromFixedSlot : (indices ? kFromIndices : kFromGenerator);
+        a.given = indices;
+        a.fixed_slot = fixed_slot;
+        a.count = count;
+        return launch_wide(r, a, t, s);
+    }
+    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, r.capacity, count,
+                       indices, fixed_slot, seed, calls, out_indices, err);
+    LAUNCH_CHECK("k_rows_gather");
+    return MRB_OK;
+}
+
 struct Urb {
     RowStore rows;
     int64_t count = 0, head = 0;
@@ -398,13 +456,7 @@ int mrb_urb_append_from(int64_t h, int64_t src, int64_t first_logical, int64_t n
 
 static int urb_gather_impl(Urb& b, const int64_t* indices, int64_t fixed_slot, int64_t n, int64_t* out_indices,
                            void* const* dst_fields, hipStream_t s) {
-    IoTable t;
-    int rc = make_table(b.rows, dst_fields, n, t);
-    if (rc) return rc;
-    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, b.rows.capacity,
-                       b.count, indices, fixed_slot, b.seed, b.calls, out_indices, b.err);
-    LAUNCH_CHECK("k_rows_gather");
-    return MRB_OK;
+    return gather_rows(b.rows, indices, fixed_slot, b.count, b.seed, b.calls, n, out_indices, dst_fields, b.err, s);
 }
 
 int mrb_urb_get_item(int64_t h, int64_t logical_index, void* const* dst_fields, void* stream) {
@@ -661,29 +713,13 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, 
     a.out_idx = out_indices;
     a.out_w = out_weights;
     a.err = b->err;
-    uint32_t max_units = 0;
-    int64_t max_bytes = 0;
-    for (int i = 0; i < b->rows.nfields; ++i) {
-        if (b->rows.units[i] > max_units) max_units = b->rows.units[i];
-        if (b->rows.bytes[i] > max_bytes) max_bytes = b->rows.bytes[i];
-    }
+    a.mode = kFromTree;
+    const int64_t max_bytes = widest_field(b->rows);
     int path = (int)g_opt.sample_path;
     if (path == 0) path = (batch >= 8192 && max_bytes <= 256) ? 2 : 1;
     if (path == 1) {
-        int split = (int)g_opt.row_split;
-        if (split <= 0) {
-            // one pass of kInFlight granules per thread covers the widest field (measured best on
-            // 28 KB rows: 2 workgroups per row; more workgroups only repeat the tree walk)
-            split = (int)((max_units + kInFlight * kWG - 1) / (kInFlight * kWG));
-            if (split < 1) split = 1;
-            if (split > 16) split = 16;
-        }
-        SplitPlan plan{};
-        plan.split = split;
-        for (int i = 0; i < b->rows.nfields; ++i) plan.per[i] = (b->rows.units[i] + split - 1) / split;
-        hipLaunchKernelGGL(k_per_sample_wide, dim3((uint32_t)(batch * split)), dim3(kWG), 0, s, a.sum, a.uniforms,
-                           a.depth, split, a.batch, a.seed, a.calls, a, t, plan);
-        LAUNCH_CHECK("k_per_sample_wide");
+        rc = launch_wide(b->rows, a, t, s);
+        if (rc) return rc;
     } else {
         int levels = g_opt.lds_levels > 0 ? (int)g_opt.lds_levels : 12;
         if (levels > b->depth) levels = b->depth;
@@ -701,14 +737,8 @@ int mrb_per_gather(int64_t h, const int64_t* indices, int64_t n, void* const* ds
     if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
     if (!indices) return fail(MRB_EINVAL, "indices is NULL");
     if (b->size <= 0) return fail(MRB_ESTATE, "gather from an empty buffer");
-    IoTable t;
-    int rc = make_table(b->rows, dst_fields, n, t);
-    if (rc) return rc;
-    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0,
-                       static_cast<hipStream_t>(stream), t, b->rows.capacity, b->size, indices, (int64_t)-1,
-                       (uint64_t)0, (uint64_t)0, static_cast<int64_t*>(nullptr), b->err);
-    LAUNCH_CHECK("k_rows_gather");
-    return MRB_OK;
+    return gather_rows(b->rows, indices, -1, b->size, 0, 0, n, nullptr, dst_fields, b->err,
+                       static_cast<hipStream_t>(stream));
 }
 
 int mrb_per_export_tree(int64_t h, float* sum_heap, float* min_heap, int64_t* leaves, void* stream) {
@@ -810,13 +840,9 @@ int mrb_res_sample(int64_t h, int64_t n, int64_t* out_indices, void* const* dst_
     GET_RES(b, h);
     if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
     if (b->size <= 0) return fail(MRB_ESTATE, "sample from an empty buffer");
-    IoTable t;
-    int rc = make_table(b->rows, dst_fields, n, t);
+    int rc = gather_rows(b->rows, nullptr, -1, b->size, b->seed, b->calls + 1, n, out_indices, dst_fields, b->err,
+                         static_cast<hipStream_t>(stream));
     if (rc) return rc;
-    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0,
-                       static_cast<hipStream_t>(stream), t, b->rows.capacity, b->size,
-                       static_cast<const int64_t*>(nullptr), (int64_t)-1, b->seed, b->calls + 1, out_indices, b->err);
-    LAUNCH_CHECK("k_rows_gather");
     b->calls += 1;
     return MRB_OK;
 }

@@ -260,7 +260,14 @@ struct SampleArgs {
     int64_t* out_idx;
     float* out_w;
     uint32_t* err;
+    // Where row k comes from. The wide-row kernel also serves plain gathers of wide rows
+    // (BufferSample / BufferGetItem / rows at given slots), which skip the tree altogether.
+    int mode;              // kFromTree, kFromIndices, kFromGenerator, kFromFixedSlot
+    const int64_t* given;  // kFromIndices: slot of row k
+    int64_t fixed_slot;    // kFromFixedSlot
+    int64_t count;         // kFromIndices / kFromGenerator: valid slots are [0, count)
 };
+constexpr int kFromTree = 0, kFromIndices = 1, kFromGenerator = 2, kFromFixedSlot = 3;
 
 // mass of stratum k: (u + k) * (total / batch), each operation rounded once.
 __device__ __forceinline__ float stratum_mass(const SampleArgs& a, float total, int64_t k, float u) {
@@ -321,7 +328,20 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
     const uint32_t split = (uint32_t)split_arg;
     const int64_t k = blockIdx.x / split;
     const uint32_t part = blockIdx.x % split;
-    if (threadIdx.x < 64) {
+    if (a.mode != kFromTree) {
+        // plain gather: the slot is given, drawn, or fixed; out-of-range slots are clamped and flagged
+        if (threadIdx.x == 0) {
+            int64_t slot = a.mode == kFromFixedSlot ? a.fixed_slot
+                           : a.mode == kFromIndices ? a.given[k]
+                                                    : rng_below(seed, calls, (uint64_t)k, a.count);
+            if (a.mode != kFromFixedSlot && (slot < 0 || slot >= a.count)) {
+                if (part == 0) atomicOr(a.err, MRB_DERR_INDEX);
+                slot = slot < 0 ? 0 : (a.count > 0 ? a.count - 1 : 0);
+            }
+            s_idx = slot;
+            s_picked = 0.0f;
+        }
+    } else if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
         const int ngroups = group_count(depth);
         int g = ngroups ? group_levels(depth, ngroups, 0) : 0;
@@ -355,7 +375,9 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
             s_idx = (int64_t)node - a.leaves;
             s_picked = picked;
         }
-    } else if (threadIdx.x < 64 + MRB_MAX_FIELDS) {
+    }
+    // (separate from the chain above: in the gather modes every thread takes its first branch)
+    if (threadIdx.x >= 64 && threadIdx.x < 64 + MRB_MAX_FIELDS) {
         const int f = threadIdx.x - 64;
         uint32_t cnt = 0, vl = 0;
         if (f < t.nfields) {
@@ -442,7 +464,9 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
             for (int i = 0; i < 8; ++i) nb[i] = nsrc[(uint32_t)i < nbytes ? i : 0];
         }
         // ---- importance weight, computed while the loads are in flight
-        if (wfirst == 0 && part == 0 && threadIdx.x < 2) {
+        if (a.mode != kFromTree) {
+            if (wfirst == 0 && part == 0 && threadIdx.x == 0 && a.out_idx) a.out_idx[k] = idx;
+        } else if (wfirst == 0 && part == 0 && threadIdx.x < 2) {
             // lane 0: (p / total * size)^-beta, lane 1: (pmin / total * size)^-beta
             const float total = a.sum[1];
             const float x = threadIdx.x == 0 ? s_picked : a.mn[1];
