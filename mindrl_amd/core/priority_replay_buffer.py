@@ -206,5 +206,13 @@ class PriorityReplayBuffer:
             raise ValueError("sample: total priority is not positive and finite")
         return f
 
+    def __del__(self):
+        # the native buffer (rows, trees) is released with the Python object if destroy() was not called
+        try:
+            if getattr(self, "_h", 0):
+                self.destroy()
+        except Exception:  # interpreter shutdown: the library or torch may already be gone
+            pass
+
     def __repr__(self):
         return "PriorityReplayBuffer<>"

@@ -102,5 +102,13 @@ class ReservoirReplayBuffer:
             views.append(view_of(p.value, (self._capacity,) + s, d, self, self._dev))
         return tuple(views)
 
+    def __del__(self):
+        # the native buffer (rows, trees) is released with the Python object if destroy() was not called
+        try:
+            if getattr(self, "_h", 0):
+                self.destroy()
+        except Exception:  # interpreter shutdown: the library or torch may already be gone
+            pass
+
     def __repr__(self):
         return "ReservoirReplayBuffer<>"

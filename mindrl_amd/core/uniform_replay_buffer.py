@@ -150,5 +150,13 @@ class UniformReplayBuffer:
             h, self._h = self._h, 0
             _lib.check(_lib.lib().mrb_urb_destroy(h))
 
+    def __del__(self):
+        # the native buffer (rows, trees) is released with the Python object if destroy() was not called
+        try:
+            if getattr(self, "_h", 0):
+                self.destroy()
+        except Exception:  # interpreter shutdown: the library or torch may already be gone
+            pass
+
     def __repr__(self):
         return "UniformReplayBuffer<>"

@@ -425,6 +425,58 @@ def test_per_error_paths(mrb):
         mrb.PER(0.6, -5, 4, [(1,)], [torch.int32])
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_randomised_differential(mrb, orc, seed):
+    """Random buffer shapes, capacities (trees of 0..18 levels), alphas and operation mixes,
+    the HIP buffer and the oracle fed the same calls; everything observable compared after each."""
+    rng = np.random.default_rng(9000 + seed)
+    cap = int(rng.choice([1, 2, 3, 7, 64, 65, 1000, 4097, 9999, 40000, 150000]))
+    nf = int(rng.integers(1, 5))
+    pool = [((1,), np.uint8), ((3,), np.int16), ((2, 2), np.float32), ((5,), np.float64), ((64,), np.float32),
+            ((300,), np.uint8), ((1,), np.bool_), ((1,), np.int64)]
+    picks = [pool[i] for i in rng.integers(0, len(pool), nf)]
+    shapes, dtypes = [p[0] for p in picks], [p[1] for p in picks]
+    alpha = float(rng.choice([0.0, 0.3, 0.6, 1.0]))
+    batch = int(rng.choice([1, 5, 64, 300]))
+    mrb.lib.set_option("sample_path", int(rng.integers(0, 3)))
+    mrb.lib.set_option("row_split", int(rng.choice([0, 0, 1, 3])))
+    g, c = make_pair(mrb, orc, alpha, cap, batch, seed=seed + 1, shapes=shapes, dtypes=dtypes)
+    for step in range(25):
+        op = rng.integers(0, 4) if c.size else 0
+        if op == 0:
+            n = int(rng.integers(1, min(2 * cap + 2, 5000)))
+            rows = random_rows(rng, n, shapes, dtypes)
+            if rng.random() < 0.4:
+                pr = (rng.pareto(1.2, n) + 1e-6).astype(np.float32)
+                g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda())
+                c.push(rows, n, pr)
+            else:
+                g.insert(*to_dev(rows))
+                c.push(rows, n)
+        elif op == 1:
+            n = int(rng.integers(1, min(3 * cap + 2, 6000)))
+            idx = rng.integers(0, cap, n)
+            pr = np.where(rng.random(n) < 0.05, 0.0, rng.lognormal(0, 2, n)).astype(np.float32)
+            g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda())
+            c.update(idx, pr)
+        elif c.export_tree()[0][1] > 0:
+            beta = float(rng.uniform(0, 1))
+            if op == 2:
+                u = rng.random(batch).astype(np.float32)
+                assert_sample_equal(g.sample(beta, uniforms=torch.from_numpy(u).cuda()), c.sample(batch, beta, u),
+                                    "seed %d step %d" % (seed, step))
+            else:
+                assert_sample_equal(g.sample(beta), c.sample(batch, beta), "seed %d step %d rng" % (seed, step))
+        assert_tree_equal(g, c, "seed %d step %d" % (seed, step))
+        assert g.size() == c.size and np.float32(g.max_priority) == np.float32(c.max_priority)
+    for f, view in enumerate(g.storage()):
+        assert np.array_equal(t2n(view).view(np.uint8), c.field(f).view(np.uint8)), f
+    mrb.lib.set_option("sample_path", 0)
+    mrb.lib.set_option("row_split", 0)
+    g.check()
+    g.destroy()
+
+
 @pytest.mark.parametrize("path", [1, 2])
 def test_sixteen_fields_of_odd_sizes(mrb, orc, path):
     """The maximum of 16 fields, row sizes 1..4100 bytes covering every copy granule (1, 2, 4, 8,
