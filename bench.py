@@ -435,7 +435,7 @@ def main():
     # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this very command, scaled by what the
     # same counters read for the ring-append copy kernel; only valid for
     # the default workload and library defaults.
-    traffic = 33.85e6 if (a.workload == "c3" and not a.capacity and not a.row_split and not a.sample_path) else None
+    traffic = 33.6e6 if (a.workload == "c3" and not a.capacity and not a.row_split and not a.sample_path) else None
     row_bytes = sum(buf._layout.bytes)
     algo_bytes = batch * (2 * row_bytes + 12)  # rows read + rows written + index (8) + weight (4)
     kern_s = dev_ms * 1e-3 / K
