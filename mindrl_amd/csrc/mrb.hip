@@ -113,19 +113,29 @@ uint32_t grid_for(uint64_t work, uint32_t per_thread = 1) {
 // One thread per entry, no grid-stride loop (n < 2^32, so the grid fits).
 uint32_t grid_exact(uint64_t n) { return (uint32_t)((n + kWG - 1) / kWG); }
 
-// Appends rows [skip, nrows) of the caller's matrices at ring position first_slot.
-int rows_put(const RowStore& r, const void* const* src, int64_t skip, int64_t n, int64_t first_slot, hipStream_t s) {
-    IoTable t;
+// Describes the append of rows [skip, skip + n) of the caller's matrices at ring position first_slot.
+int put_args(const RowStore& r, const void* const* src, int64_t skip, int64_t n, int64_t first_slot, PutArgs& p) {
     const void* shifted[MRB_MAX_FIELDS];
     if (!src) return fail(MRB_EINVAL, "field pointer array is NULL");
     for (int i = 0; i < r.nfields; ++i) {
         if (!src[i]) return fail(MRB_EINVAL, "field %d pointer is NULL", i);
         shifted[i] = static_cast<const uint8_t*>(src[i]) + skip * r.bytes[i];
     }
-    int rc = make_table(r, shifted, n, t);
+    int rc = make_table(r, shifted, n, p.t);
     if (rc) return rc;
-    hipLaunchKernelGGL(k_rows_put, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, r.capacity, first_slot,
-                       (int64_t)0, (int64_t)0);
+    p.capacity = r.capacity;
+    p.first_slot = first_slot;
+    p.src_capacity = 0;
+    p.src_first = 0;
+    p.blocks = grid_for(p.t.prefix[p.t.nfields]);
+    return MRB_OK;
+}
+
+int rows_put(const RowStore& r, const void* const* src, int64_t skip, int64_t n, int64_t first_slot, hipStream_t s) {
+    PutArgs p{};
+    int rc = put_args(r, src, skip, n, first_slot, p);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_rows_put, dim3(p.blocks), dim3(kWG), 0, s, p);
     LAUNCH_CHECK("k_rows_put");
     return MRB_OK;
 }
@@ -312,14 +322,18 @@ int read_and_clear_flags(uint32_t* d_err, uint32_t* flags, hipStream_t s) {
     return MRB_OK;
 }
 
-// Rebuilds the tree above the leaves that `a` writes: one launch per round, then the top.
-int tree_rebuild(Per& b, const UpdateArgs& a, hipStream_t s) {
+// Rebuilds the tree above the leaves that `a` writes: one launch per round, then the top. A push hands
+// its row copy over (`ride`): it is done by extra workgroups of the first launch.
+int tree_rebuild(Per& b, const UpdateArgs& a, hipStream_t s, const PutArgs* ride = nullptr) {
+    PutArgs none{};  // blocks == 0: no copy rides along
     for (int r = 0; r < b.nrounds; ++r) {
         const uint32_t tiles = (1u << b.lo[r]) / kBlockNodes;
-        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r);
+        const PutArgs& put = (r == 0 && ride) ? *ride : none;
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4 + put.blocks), dim3(kWG), 0, s, a, r, put);
         LAUNCH_CHECK("k_tree_update");
     }
-    hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a);
+    const PutArgs& put = (b.nrounds == 0 && ride) ? *ride : none;
+    hipLaunchKernelGGL(k_tree_top, dim3(1 + put.blocks), dim3(kTopWG), 0, s, a, put);
     LAUNCH_CHECK("k_tree_top");
     return MRB_OK;
 }
@@ -442,13 +456,17 @@ int mrb_urb_append_from(int64_t h, int64_t src, int64_t first_logical, int64_t n
     const bool growing = b->count < cap && b->head == 0;
     const int64_t w = growing ? b->count : b->head;
     const int64_t skip = n > cap ? n - cap : 0;
-    IoTable t;
+    PutArgs p{};
     const void* io[MRB_MAX_FIELDS];
     for (int i = 0; i < b->rows.nfields; ++i) io[i] = from->rows.data[i];
-    int rc = make_table(b->rows, io, n - skip, t);
+    int rc = make_table(b->rows, io, n - skip, p.t);
     if (rc) return rc;
-    hipLaunchKernelGGL(k_rows_put, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, static_cast<hipStream_t>(stream),
-                       t, cap, (w + skip) % cap, from->rows.capacity, (src_first + skip) % from->rows.capacity);
+    p.capacity = cap;
+    p.first_slot = (w + skip) % cap;
+    p.src_capacity = from->rows.capacity;
+    p.src_first = (src_first + skip) % from->rows.capacity;
+    p.blocks = grid_for(p.t.prefix[p.t.nfields]);
+    hipLaunchKernelGGL(k_rows_put, dim3(p.blocks), dim3(kWG), 0, static_cast<hipStream_t>(stream), p);
     LAUNCH_CHECK("k_rows_put");
     urb_advance(*b, n);
     return MRB_OK;
@@ -616,8 +634,15 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     const int64_t skip = nrows > cap ? nrows - cap : 0;  // rows overwritten within this very call
     const int64_t n = nrows - skip;
     const int64_t first = (b->pushes + skip) % cap;
-    int rc = rows_put(b->rows, src_fields, skip, n, first, s);
+    PutArgs put{};
+    int rc = put_args(b->rows, src_fields, skip, n, first, put);
     if (rc) return rc;
+    if (put.blocks > 2048) {
+        // a large copy gets its own launch; a small one rides along in the first tree launch
+        hipLaunchKernelGGL(k_rows_put, dim3(put.blocks), dim3(kWG), 0, s, put);
+        LAUNCH_CHECK("k_rows_put");
+        put.blocks = 0;
+    }
     rc = next_epoch(*b, s);
     if (rc) return rc;
     UpdateArgs a = update_args(*b);
@@ -631,7 +656,7 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     }
     a.first_slot = first;
     a.n = n;
-    rc = tree_rebuild(*b, a, s);
+    rc = tree_rebuild(*b, a, s, put.blocks ? &put : nullptr);
     if (rc) return rc;
     b->pushes += nrows;
     b->size = b->size + nrows < cap ? b->size + nrows : cap;
@@ -678,12 +703,13 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     if (!sparse) return tree_rebuild(*b, a, s);
     hipLaunchKernelGGL(k_tree_sparse, dim3(grid_exact((uint64_t)n << (b->s_g0 - 2))), dim3(kWG), 0, s, a);
     LAUNCH_CHECK("k_tree_sparse");
+    const PutArgs none{};
     for (int r = 0; r < b->s_rounds; ++r) {
         const uint32_t tiles = (1u << b->s_lo[r]) / kBlockNodes;
-        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r);
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r, none);
         LAUNCH_CHECK("k_tree_update");
     }
-    hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a);
+    hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a, none);
     LAUNCH_CHECK("k_tree_top");
     return MRB_OK;
 }

@@ -145,21 +145,28 @@ __device__ __forceinline__ void split_work(uint64_t local, uint32_t units, uint6
 // ---------------------------------------------------------------------------
 // src_capacity > 0: the source is itself a ring of that many rows and row r is read from its
 // slot (src_first + r) mod src_capacity (buffer-to-buffer copy); 0: the source is contiguous.
-__global__ __launch_bounds__(kWG) void k_rows_put(IoTable t, int64_t capacity, int64_t first_slot,
-                                                  int64_t src_capacity, int64_t src_first) {
+struct PutArgs {
+    IoTable t;
+    int64_t capacity, first_slot, src_capacity, src_first;
+    uint32_t blocks;  // workgroups doing this copy when it rides along in another kernel's launch (0: none)
+};
+
+// The copy itself, by workgroup `block` of `nblocks` (grid-stride over the granules).
+__device__ __forceinline__ void rows_put_part(const PutArgs& p, uint32_t block, uint32_t nblocks) {
+    const IoTable& t = p.t;
     const uint64_t total = t.prefix[t.nfields];
-    const uint64_t stride = (uint64_t)gridDim.x * kWG;
-    for (uint64_t w = (uint64_t)blockIdx.x * kWG + threadIdx.x; w < total; w += stride) {
+    const uint64_t stride = (uint64_t)nblocks * blockDim.x;
+    for (uint64_t w = (uint64_t)block * blockDim.x + threadIdx.x; w < total; w += stride) {
         const int f = field_of(t, w);
         uint64_t row;
         uint32_t unit;
         split_work(w - t.prefix[f], t.units[f], row, unit);
-        int64_t slot = first_slot + (int64_t)row;
-        if (slot >= capacity) slot -= capacity;
+        int64_t slot = p.first_slot + (int64_t)row;
+        if (slot >= p.capacity) slot -= p.capacity;
         uint64_t src_row = row;
-        if (src_capacity > 0) {
-            int64_t q = src_first + (int64_t)row;
-            if (q >= src_capacity) q -= src_capacity;
+        if (p.src_capacity > 0) {
+            int64_t q = p.src_first + (int64_t)row;
+            if (q >= p.src_capacity) q -= p.src_capacity;
             src_row = (uint64_t)q;
         }
         const uint32_t vl = t.vec_log2[f];
@@ -168,6 +175,8 @@ __global__ __launch_bounds__(kWG) void k_rows_put(IoTable t, int64_t capacity, i
                      as_global(t.io[f]) + src_row * t.row_bytes[f] + off, vl);
     }
 }
+
+__global__ __launch_bounds__(kWG) void k_rows_put(PutArgs p) { rows_put_part(p, blockIdx.x, gridDim.x); }
 
 // ---------------------------------------------------------------------------
 // Gather: io_f[k] = store_f[slot_k]. slot_k is `fixed_slot` when that is >= 0
@@ -877,8 +886,14 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top) {
     }
 }
 
-// One wave per tile of round `round` (>= 0).
-__global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round) {
+// One wave per tile of round `round` (>= 0). A push lets its row copy ride along in the same
+// launch (the copy and the tree work touch different memory): workgroups past the tiles do it.
+__global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, PutArgs put) {
+    const uint32_t tile_blocks = gridDim.x - put.blocks;
+    if (blockIdx.x >= tile_blocks) {
+        rows_put_part(put, blockIdx.x - tile_blocks, put.blocks);
+        return;
+    }
     const uint32_t lane = threadIdx.x & 63;
     const int lo = a.lo[round], g = a.g[round];
     const uint32_t tile = blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
@@ -889,11 +904,18 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round) {
 }
 
 // The top of the tree (everything above a.top_depth; the whole tree, leaves included, when it has
-// no rounds), one workgroup. A separate launch rather than a continuation of the last round by
-// its last workgroup: publishing the rounds' stores to that workgroup needs an agent-scope
-// fence per workgroup, which on this multi-die part costs far more than a launch.
+// no rounds), one workgroup; further workgroups carry a push's row copy when the tree has no rounds.
+// A separate launch rather than a continuation of the last round by its last workgroup: publishing
+// the rounds' stores to that workgroup needs an agent-scope fence per workgroup, which on this
+// multi-die part costs far more than a launch.
 constexpr int kTopWG = 1024;
-__global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a) { top_rebuild(a, a.top_depth); }
+__global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) {
+    if (blockIdx.x >= 1) {
+        rows_put_part(put, blockIdx.x - 1, put.blocks);
+        return;
+    }
+    top_rebuild(a, a.top_depth);
+}
 
 // ---------------------------------------------------------------------------
 // Discounted return (mindspore_rl/utils/discounted_return.py:84-92): one thread per
