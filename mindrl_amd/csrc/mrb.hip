@@ -646,18 +646,23 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     rc = next_epoch(*b, s);
     if (rc) return rc;
     UpdateArgs a = update_args(*b);
+    // push-then-update: the running max sees every priority of the call, surviving or not, and is
+    // raised only after the tree work (a fresh slot with an invalid priority keeps the old running max)
+    const bool fold = opt_priorities && skip == 0 && nrows <= 1024;  // few enough for the top workgroup
     if (opt_priorities) {
-        // push-then-update: the running max sees every priority of the call, surviving or not
-        a.priorities = opt_priorities;
-        a.n = nrows;
-        hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)nrows)), dim3(kWG), 0, s, a);
-        LAUNCH_CHECK("k_update_stamp");
         a.priorities = opt_priorities + skip;
+        a.fold_max = fold ? 1 : 0;
     }
     a.first_slot = first;
     a.n = n;
     rc = tree_rebuild(*b, a, s, put.blocks ? &put : nullptr);
     if (rc) return rc;
+    if (opt_priorities && !fold) {
+        a.priorities = opt_priorities;
+        a.n = nrows;
+        hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)nrows)), dim3(kWG), 0, s, a);
+        LAUNCH_CHECK("k_update_stamp");
+    }
     b->pushes += nrows;
     b->size = b->size + nrows < cap ? b->size + nrows : cap;
     return MRB_OK;

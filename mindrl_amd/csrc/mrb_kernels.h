@@ -655,6 +655,7 @@ struct UpdateArgs {
     uint32_t* dirty[kMaxRounds];  // per round: one epoch word per block of 1 << g[r] nodes at depth lo[r]
     // sparse updates of very large trees: the lowest sparse_g0 levels are rebuilt per entry
     // (k_tree_sparse) instead of per tile; owner[block] elects one entry per block of leaves
+    int fold_max;                // push with priorities: k_tree_top also folds them into the running max
     int sparse_g0;               // 0 = not used
     unsigned long long* owner;   // [leaves >> sparse_g0]
 };
@@ -915,6 +916,22 @@ __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) 
         return;
     }
     top_rebuild(a, a.top_depth);
+    if (a.fold_max) {
+        // The rounds before this launch read the running max as it was before the call (fresh slots
+        // with an invalid priority take it), so it is raised only now.
+        float q = 0.0f;
+        for (int64_t j = threadIdx.x; j < a.n; j += kTopWG) {
+            const float p = a.priorities[j];
+            if (valid_priority(p)) {
+                q = fmaxf(q, powf_det(p, a.alpha));
+            } else {
+                atomicOr(a.err, MRB_DERR_PRIORITY);
+            }
+        }
+        for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+        if ((threadIdx.x & 63) == 0 && q > 0.0f)
+            atomicMax(reinterpret_cast<unsigned int*>(a.maxp), __float_as_uint(q));
+    }
 }
 
 // ---------------------------------------------------------------------------
