@@ -10,6 +10,40 @@ from ._rows import (FieldLayout, device, get_counters, load_fields, pointers, sa
                     view_of)
 
 
+class _BufferAppend:
+    """Stands in for P.BufferAppend (uniform_replay_buffer.py:82): called as
+    buffer_append(buffer, exp, count, head); buffer, count and head are the owner's own state."""
+
+    def __init__(self, owner):
+        self._owner_ref = owner
+
+    def __call__(self, buffer, exp, count=None, head=None):
+        self._owner_ref.insert(exp)
+        return True
+
+
+class _BufferSample:
+    """Stands in for P.BufferSample (uniform_replay_buffer.py:87-89): batch_size attribute,
+    called as buffer_sample(buffer, count, head)."""
+
+    def __init__(self, owner):
+        self._owner_ref = owner
+        self.batch_size = owner._sample_size
+
+    def __call__(self, buffer=None, count=None, head=None):
+        return self._owner_ref.sample()
+
+
+class _BufferGet:
+    """Stands in for P.BufferGetItem (uniform_replay_buffer.py:83): buffer_get(buffer, count, head, index)."""
+
+    def __init__(self, owner):
+        self._owner_ref = owner
+
+    def __call__(self, buffer, count, head, index):
+        return self._owner_ref.get_item(index)
+
+
 class UniformReplayBuffer:
     """FIFO replay buffer resident in HBM.
 
@@ -41,6 +75,13 @@ class UniformReplayBuffer:
             _lib.check(_lib.lib().mrb_urb_field_ptr(self._h, i, C.byref(p)))
             views.append(view_of(p.value, (self._capacity,) + s, d, self, self._dev))
         self.buffer = tuple(views)
+        # Attributes that subclasses and callers of the reference class reach into: the append and sample
+        # primitives (mindspore_rl/algorithm/mappo/mappo_replaybuffer.py:43 calls
+        # `self.buffer_append(self.buffer, exp, self.count, self.head)`;
+        # mindspore_rl/algorithm/gail/gail.py:163-164 reads `buffer_sample.batch_size`).
+        self.buffer_append = _BufferAppend(self)
+        self.buffer_sample = _BufferSample(self)
+        self.buffer_get = _BufferGet(self)
 
     # -- reference methods ---------------------------------------------------
     def insert(self, exp):

@@ -78,6 +78,26 @@ def test_uniform_ring_random_ops(mrb, orc, layout, cap):
     g.destroy()
 
 
+def test_uniform_primitive_attributes_used_by_reference_callers(mrb):
+    """A subclass written like mindspore_rl/algorithm/mappo/mappo_replaybuffer.py:23-44 works unchanged,
+    and buffer_sample.batch_size is readable (mindspore_rl/algorithm/gail/gail.py:163-164)."""
+
+    class ConditionalBuffer(mrb.URB):
+        def construct(self, exp, command):
+            if command:
+                self.buffer_append(self.buffer, exp, self.count, self.head)
+            return self.buffer
+
+    b = ConditionalBuffer(4, 10, [(2,)], [torch.float32])
+    b.construct([torch.ones(2).cuda()], False)
+    assert int(b.count) == 0
+    out = b.construct([torch.ones(2).cuda() * 3], True)
+    assert int(b.count) == 1 and float(out[0][0, 0]) == 3.0
+    assert b.buffer_sample.batch_size == 4
+    assert float(b.buffer_get(b.buffer, b.count, b.head, 0)[0][1]) == 3.0
+    b.destroy()
+
+
 def test_uniform_successive_samples_differ_and_errors(mrb):
     g = mrb.URB(32, 200, [(1,)], [torch.int32], seed=5)
     with pytest.raises(ValueError):
