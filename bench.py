@@ -328,7 +328,8 @@ def bench_discounted_return(a):
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "DiscountedReturn, reward [1000, %d, 1] f32, gamma 0.99, 1 %% dones" % b},
         "roofline": {"bound": "hbm", "achieved": algo / kern_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "k_discounted_return",
+                     "frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "k_discounted_return_tiled" if b * inner <= 16384 else "k_discounted_return",
                      "algorithmic_bytes_per_launch": algo, "avg_launch_us": kern_s * 1e6},
         "cpu_baseline": None,
     }

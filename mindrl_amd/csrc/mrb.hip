@@ -999,6 +999,15 @@ int mrb_discounted_return(const float* reward, const uint8_t* done, const float*
         return fail(MRB_EINVAL, "The discounted factor should be a number in range [0, 1], but got %g.", (double)gamma);
     const int64_t cols = batch * inner;
     if (cols > (1ll << 40) / timesteps) return fail(MRB_EINVAL, "problem too large");
+    if (cols <= 256 * kDrCols) {
+        // few columns (at most one 64-column tile per compute unit): a thread per column cannot keep
+        // enough loads in flight; stage chunks through LDS
+        hipLaunchKernelGGL(k_discounted_return_tiled, dim3((uint32_t)((cols + kDrCols - 1) / kDrCols)), dim3(kDrWG), 0,
+                           static_cast<hipStream_t>(stream), reward, done, last_value, out, timesteps, batch, inner,
+                           gamma);
+        LAUNCH_CHECK("k_discounted_return_tiled");
+        return MRB_OK;
+    }
     hipLaunchKernelGGL(k_discounted_return, dim3(grid_exact((uint64_t)cols)), dim3(kWG), 0,
                        static_cast<hipStream_t>(stream), reward, done, last_value, out, timesteps, batch, inner, gamma);
     LAUNCH_CHECK("k_discounted_return");

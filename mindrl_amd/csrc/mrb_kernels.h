@@ -975,6 +975,95 @@ __global__ __launch_bounds__(kWG) void k_discounted_return(const float* __restri
     }
 }
 
+// The same recurrence for inputs with few columns, where a thread per column leaves the memory
+// system idle: a workgroup takes 64 columns and walks the time axis in chunks of kDrChunk steps.
+// All sixteen waves load a chunk's rewards and done flags into LDS (independent, fully coalesced
+// loads), wave 0 runs the recurrence over the chunk out of LDS (lane = column), all waves store
+// the results. The arithmetic and its order are those of k_discounted_return.
+constexpr int kDrChunk = 256;
+constexpr int kDrCols = 64;
+constexpr int kDrWG = 1024;  // 16 waves: each thread moves 16 rows of a chunk, all 16 loads in flight at once
+__global__ __launch_bounds__(kDrWG) void k_discounted_return_tiled(const float* __restrict__ reward,
+                                                                 const uint8_t* __restrict__ done,
+                                                                 const float* __restrict__ last_value,
+                                                                 float* __restrict__ out, int64_t timesteps,
+                                                                 int64_t batch, int64_t inner, float gamma) {
+    __shared__ float s_val[kDrChunk * kDrCols];    // rewards in, returns out
+    __shared__ uint8_t s_done[kDrChunk * kDrCols];
+    const int64_t cols = batch * inner;
+    const int64_t c0 = (int64_t)blockIdx.x * kDrCols;
+    const int ncols = (int)(cols - c0 < kDrCols ? cols - c0 : kDrCols);
+    const int lane = threadIdx.x & 63;
+    float last = 0.0f;
+    if (threadIdx.x < ncols) last = last_value[c0 + threadIdx.x];
+    for (int64_t hi = timesteps; hi > 0; hi -= kDrChunk) {
+        const int64_t t0 = hi > kDrChunk ? hi - kDrChunk : 0;
+        const int steps = (int)(hi - t0);
+        // thread -> column cc, time rows tr, tr + 16, ...: 16 loads are issued before the first LDS write
+        {
+            constexpr int BATCH = 16, ROWS = kDrWG / kDrCols;
+            const int cc = threadIdx.x % kDrCols, tr = threadIdx.x / kDrCols;
+            const int64_t c = c0 + (cc < ncols ? cc : 0);
+            const int64_t b = c / inner;
+            for (int base = tr; base < steps; base += ROWS * BATCH) {
+                float r[BATCH];
+                uint8_t d[BATCH];
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u) {
+                    const int tt = base + u * ROWS < steps ? base + u * ROWS : tr;  // clamped: always a valid row
+                    r[u] = __builtin_nontemporal_load(reward + (t0 + tt) * cols + c);
+                    d[u] = done[(t0 + tt) * batch + b];
+                }
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u) {
+                    const int tt = base + u * ROWS;
+                    if (tt < steps) {
+                        s_val[tt * kDrCols + cc] = r[u];
+                        s_done[tt * kDrCols + cc] = d[u];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x < 64 && lane < ncols) {
+            // 32 steps at a time through registers, so that the LDS reads are not serialised
+            // behind the recurrence's stores
+            constexpr int STEP = 32;
+            int tt = steps - 1;
+            for (; tt >= STEP - 1; tt -= STEP) {
+                float r[STEP];
+                uint8_t d[STEP];
+#pragma unroll
+                for (int u = 0; u < STEP; ++u) {
+                    r[u] = s_val[(tt - u) * kDrCols + lane];
+                    d[u] = s_done[(tt - u) * kDrCols + lane];
+                }
+#pragma unroll
+                for (int u = 0; u < STEP; ++u) {
+                    const float scaled = (1.0f - (d[u] ? 1.0f : 0.0f)) * gamma;
+                    last = r[u] + scaled * last;
+                    r[u] = last;
+                }
+#pragma unroll
+                for (int u = 0; u < STEP; ++u) s_val[(tt - u) * kDrCols + lane] = r[u];
+            }
+            for (; tt >= 0; --tt) {
+                const float scaled = (1.0f - (s_done[tt * kDrCols + lane] ? 1.0f : 0.0f)) * gamma;
+                last = s_val[tt * kDrCols + lane] + scaled * last;
+                s_val[tt * kDrCols + lane] = last;
+            }
+        }
+        __syncthreads();
+        {
+            const int cc = threadIdx.x % kDrCols, tr = threadIdx.x / kDrCols;
+            if (cc < ncols)
+                for (int tt = tr; tt < steps; tt += kDrWG / kDrCols)
+                    __builtin_nontemporal_store(s_val[tt * kDrCols + cc], out + (t0 + tt) * cols + c0 + cc);
+        }
+        __syncthreads();
+    }
+}
+
 // Fills a float array with one value (tree initialisation: sums 0, mins FLT_MAX).
 __global__ __launch_bounds__(kWG) void k_fill_f32(float* p, float v, uint64_t n) {
     const uint64_t stride = (uint64_t)gridDim.x * kWG;

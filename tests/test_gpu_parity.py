@@ -199,7 +199,8 @@ def test_discounted_return_reference_vectors(mrb):
         DiscountedReturn(gamma=1.5)
 
 
-@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 1, 1), (37, 3, 1), (100, 64, 5), (1000, 256, 1), (9, 1000, 17)])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 1, 1), (37, 3, 1), (100, 64, 5), (1000, 256, 1), (9, 1000, 17),
+                                   (300, 65, 1), (257, 130, 3), (40, 70000, 1), (33, 9000, 8)])
 def test_discounted_return_bit_exact(mrb, orc, shape):
     from mindrl_amd.utils import DiscountedReturn
     t, b, inner = shape
