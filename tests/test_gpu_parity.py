@@ -215,6 +215,36 @@ def test_discounted_return_bit_exact(mrb, orc, shape):
         assert got.shape == r.shape and np.array_equal(got.view(np.int32), want.view(np.int32)), gamma
 
 
+def test_discounted_return_backward_matches_autograd_of_the_reference_loop(mrb):
+    """need_bprop=True: gradients equal those torch's autograd gives for the reference's own loop
+    (mindspore_rl/utils/discounted_return.py:84-92) evaluated with torch ops in float32."""
+    from mindrl_amd.utils import DiscountedReturn
+    torch.manual_seed(3)
+    for t, b, inner in [(7, 1, 1), (50, 9, 1), (33, 5, 4)]:
+        shape = (t, b) + ((inner,) if inner > 1 else ())
+        r0 = torch.randn(shape, device="cuda")
+        v0 = torch.randn(shape[1:], device="cuda")
+        d = torch.rand(t, b, device="cuda") < 0.15
+        w = torch.randn(shape, device="cuda")
+        r1, v1 = r0.clone().requires_grad_(True), v0.clone().requires_grad_(True)
+        out = DiscountedReturn(0.97, need_bprop=True)(r1, d, v1)
+        (out * w).sum().backward()
+        r2, v2 = r0.clone().requires_grad_(True), v0.clone().requires_grad_(True)
+        last, rows = v2, [None] * t
+        for step in range(t - 1, -1, -1):
+            keep = (1 - d[step].float())
+            keep = keep.reshape(keep.shape + (1,) * (last.dim() - keep.dim()))
+            last = r2[step] + keep * 0.97 * last
+            rows[step] = last
+        ref = torch.stack(rows)
+        (ref * w).sum().backward()
+        assert torch.allclose(out, ref, rtol=1e-6, atol=1e-6)
+        assert torch.allclose(r1.grad, r2.grad, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(v1.grad, v2.grad, rtol=1e-5, atol=1e-6)
+    # without need_bprop the result carries no graph
+    assert not DiscountedReturn(0.97)(r0.clone().requires_grad_(True), d, v0).requires_grad
+
+
 # -------------------------------------------------------------- n-step buffer
 class OracleNStep:
     """The reference's NStepBuffer, line for line, over two oracle ring buffers
