@@ -569,6 +569,31 @@ def test_sixteen_fields_of_odd_sizes(mrb, orc, path):
         b.destroy()
 
 
+@pytest.mark.parametrize("path", [1, 2])
+def test_out_of_domain_inputs_are_clamped_and_flagged(mrb, orc, path):
+    """Draws outside [0, 1), NaN draws, and slots far outside the buffer: the oracle defines what comes
+    back (the descent has no clamp), the row copies stay inside the storage, and flags are raised."""
+    mrb.lib.set_option("sample_path", path)
+    shapes, dtypes = [(600,), (1,)], [np.float32, np.int32]  # one wide and one narrow field
+    rng = np.random.default_rng(4)
+    cap = 1500
+    g, c = make_pair(mrb, orc, 0.6, cap, 8, seed=5, shapes=shapes, dtypes=dtypes)
+    rows = random_rows(rng, cap, shapes, dtypes)
+    g.insert(*to_dev(rows)), c.push(rows, cap)
+    u = np.array([0.0, 0.999, 1.0, 7.5, -3.0, np.nan, np.inf, 1e30], np.float32)
+    assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(8, 0.5, u), "odd draws")
+    assert g.check() & 8  # the descent ended past the filled leaves at least once
+    wild = torch.tensor([0, cap - 1, cap, 10 ** 12, -1, -2 ** 62, 2 ** 62, 5], dtype=torch.int64).cuda()
+    got = g.gather(wild)
+    want = np.clip(t2n(wild), 0, cap - 1)
+    assert np.array_equal(t2n(got[1])[:, 0], c.field(1)[want, 0])
+    assert np.array_equal(t2n(got[0]), c.field(0)[want])
+    with pytest.raises(IndexError):
+        g.check()
+    mrb.lib.set_option("sample_path", 0)
+    g.destroy()
+
+
 # ----------------------------------------------- the five benchmark configurations
 def test_config1_dqn_per_cartpole_full_loop(mrb, orc):
     """Config 1: capacity 10 000, alpha .6, beta .4, eps 1e-6; fill, then 1000 x
