@@ -703,6 +703,12 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
             a.g[r] = b->s_g[r];
         }
     }
+    // A small call on a tree of at least four leaves needs no stamp pass: the leaf-level waves scan the
+    // entries themselves (one launch less).
+    if (!sparse && n <= 1024 && b->depth >= 2) {
+        a.inline_election = 1;
+        return tree_rebuild(*b, a, s);
+    }
     hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
     LAUNCH_CHECK("k_update_stamp");
     if (!sparse) return tree_rebuild(*b, a, s);

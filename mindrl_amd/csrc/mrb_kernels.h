@@ -656,6 +656,7 @@ struct UpdateArgs {
     // sparse updates of very large trees: the lowest sparse_g0 levels are rebuilt per entry
     // (k_tree_sparse) instead of per tile; owner[block] elects one entry per block of leaves
     int fold_max;                // push with priorities: k_tree_top also folds them into the running max
+    int inline_election;         // small update_priorities: no stamp pass, the leaf-level waves scan the entries
     int sparse_g0;               // 0 = not used
     unsigned long long* owner;   // [leaves >> sparse_g0]
 };
@@ -726,11 +727,15 @@ __device__ __forceinline__ bool range_meets(const UpdateArgs& a, int64_t lo, int
 //              a block is dirty if its word in dirty_in carries this call's epoch or, at the
 //              leaf level of a push (dirty_in NULL), if it meets the pushed slot range
 //   dirty_out  next round's words, marked for every block rebuilt here (may be NULL)
+//   win        this wave's 256 ints of LDS, used at the leaf level of a small update
+//              (a.inline_election): the wave scans the call's entries itself, the last entry
+//              aimed at each of its leaves wins through an LDS integer max (last write wins),
+//              and the blocks holding a winner are the dirty ones
 // Lanes of clean blocks neither load nor store; the shuffles of a dirty block only mix
 // lanes of that block.
 __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, uint32_t tile, bool sparse,
                                            const uint32_t* __restrict__ dirty_in, uint32_t* __restrict__ dirty_out,
-                                           int g_next, uint32_t lane) {
+                                           int g_next, uint32_t lane, int* win = nullptr) {
     const uint32_t level_nodes = 1u << lo;
     const bool leaf_level = lo == a.depth;
     if (level_nodes < 4) {
@@ -761,7 +766,35 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
     const uint32_t off = tile * kBlockNodes + 4 * lane;  // this lane's first node within the level
     const uint32_t first = level_nodes + tile * kBlockNodes;  // heap index of the tile's first node
     bool active = 4 * lane < tile_nodes;
-    if (active && sparse) {
+    const bool elect = leaf_level && a.inline_election && win != nullptr;
+    int jw0 = -1, jw1 = -1, jw2 = -1, jw3 = -1;  // winning entry of each of this lane's leaves
+    if (elect) {
+        win[4 * lane + 0] = -1;
+        win[4 * lane + 1] = -1;
+        win[4 * lane + 2] = -1;
+        win[4 * lane + 3] = -1;
+        __builtin_amdgcn_wave_barrier();
+        for (int64_t base = 0; base < a.n; base += 64) {
+            const int64_t j = base + lane;
+            if (j < a.n) {
+                const int64_t idx = a.indices[j];
+                if (idx >= 0 && idx < a.capacity && valid_priority(a.priorities[j]) &&
+                    (uint32_t)((uint64_t)idx / kBlockNodes) == tile)
+                    atomicMax(&win[idx % kBlockNodes], (int)j);
+            }
+        }
+        __threadfence_block();  // LDS operations of a wave complete in order; this also stops the compiler
+        __builtin_amdgcn_wave_barrier();
+        jw0 = win[4 * lane + 0];
+        jw1 = win[4 * lane + 1];
+        jw2 = win[4 * lane + 2];
+        jw3 = win[4 * lane + 3];
+        const unsigned long long hit = __ballot(jw0 >= 0 || jw1 >= 0 || jw2 >= 0 || jw3 >= 0);
+        const uint32_t lanes_per_block = g >= 8 ? 64u : (1u << g) / 4u;
+        const unsigned long long block_lanes =
+            lanes_per_block >= 64 ? ~0ull : ((1ull << lanes_per_block) - 1) << (lane & ~(lanes_per_block - 1));
+        active = active && (hit & block_lanes) != 0;
+    } else if (active && sparse) {
         if (dirty_in) {
             active = dirty_in[off >> g] == a.epoch;
         } else if (leaf_level && !a.indices) {
@@ -776,10 +809,17 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
         if (leaf_level) {
             float q;
             bool wrote = false;
-            if (leaf_value(a, off + 0, q)) { vs.x = vm.x = q; wrote = true; }
-            if (leaf_value(a, off + 1, q)) { vs.y = vm.y = q; wrote = true; }
-            if (leaf_value(a, off + 2, q)) { vs.z = vm.z = q; wrote = true; }
-            if (leaf_value(a, off + 3, q)) { vs.w = vm.w = q; wrote = true; }
+            if (elect) {
+                if (jw0 >= 0) { vs.x = vm.x = powf_det(a.priorities[jw0], a.alpha); wrote = true; }
+                if (jw1 >= 0) { vs.y = vm.y = powf_det(a.priorities[jw1], a.alpha); wrote = true; }
+                if (jw2 >= 0) { vs.z = vm.z = powf_det(a.priorities[jw2], a.alpha); wrote = true; }
+                if (jw3 >= 0) { vs.w = vm.w = powf_det(a.priorities[jw3], a.alpha); wrote = true; }
+            } else {
+                if (leaf_value(a, off + 0, q)) { vs.x = vm.x = q; wrote = true; }
+                if (leaf_value(a, off + 1, q)) { vs.y = vm.y = q; wrote = true; }
+                if (leaf_value(a, off + 2, q)) { vs.z = vm.z = q; wrote = true; }
+                if (leaf_value(a, off + 3, q)) { vs.w = vm.w = q; wrote = true; }
+            }
             if (wrote) {
                 *reinterpret_cast<float4*>(a.sum + first + 4 * lane) = vs;
                 *reinterpret_cast<float4*>(a.mn + first + 4 * lane) = vm;
@@ -873,13 +913,36 @@ __global__ __launch_bounds__(kWG) void k_tree_sparse(UpdateArgs a) {
     }
 }
 
+// Small update without a stamp pass: what k_update_stamp does besides electing — flag invalid
+// entries and fold every valid p^alpha into the running max — is shared out among the waves,
+// 64 entries at a time.
+__device__ __forceinline__ void entry_duty(const UpdateArgs& a, uint32_t wave_id, uint32_t nwaves, uint32_t lane) {
+    for (int64_t base = (int64_t)wave_id * 64; base < a.n; base += (int64_t)nwaves * 64) {
+        const int64_t j = base + lane;
+        float q = 0.0f;
+        if (j < a.n) {
+            const int64_t idx = a.indices[j];
+            const float p = a.priorities[j];
+            const bool idx_ok = idx >= 0 && idx < a.capacity;
+            if (!idx_ok) atomicOr(a.err, MRB_DERR_INDEX);
+            if (!valid_priority(p)) atomicOr(a.err, MRB_DERR_PRIORITY);
+            if (idx_ok && valid_priority(p)) q = powf_det(p, a.alpha);
+        }
+        for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+        if (lane == 0 && q > 0.0f) atomicMax(reinterpret_cast<unsigned int*>(a.maxp), __float_as_uint(q));
+    }
+}
+
 // Rebuilds everything above depth `top` (<= 12) with one workgroup: first up to 8 levels
 // over the 1..16 tiles of that depth (one wave each), then the rest in one tile.
-__device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top) {
+// `win`: 256 ints of LDS per wave (see tile_round).
+__device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, int* win) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int g1 = top < kRoundLevels ? top : kRoundLevels;
     const uint32_t tiles = (1u << top) <= (uint32_t)kBlockNodes ? 1u : (1u << top) / kBlockNodes;
-    for (uint32_t t = wave; t < tiles; t += nwaves) tile_round(a, top, g1, t, false, nullptr, nullptr, 0, lane);
+    if (a.inline_election && top == a.depth) entry_duty(a, wave, nwaves, lane);
+    for (uint32_t t = wave; t < tiles; t += nwaves)
+        tile_round(a, top, g1, t, false, nullptr, nullptr, 0, lane, win + wave * kBlockNodes);
     if (top > g1) {
         __threadfence_block();  // the tiles' parents, written by other waves of this workgroup, are read below
         __syncthreads();
@@ -890,6 +953,7 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top) {
 // One wave per tile of round `round` (>= 0). A push lets its row copy ride along in the same
 // launch (the copy and the tree work touch different memory): workgroups past the tiles do it.
 __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, PutArgs put) {
+    __shared__ int s_win[kWG / 64][kBlockNodes];
     const uint32_t tile_blocks = gridDim.x - put.blocks;
     if (blockIdx.x >= tile_blocks) {
         rows_put_part(put, blockIdx.x - tile_blocks, put.blocks);
@@ -898,10 +962,14 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, Pu
     const uint32_t lane = threadIdx.x & 63;
     const int lo = a.lo[round], g = a.g[round];
     const uint32_t tile = blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
+    const uint32_t ntiles = (1u << lo) / kBlockNodes;
     const bool last_round = round + 1 == a.nrounds;
-    if (tile < (1u << lo) / kBlockNodes)
-        tile_round(a, lo, g, tile, true, (round == 0 && !a.indices) ? nullptr : a.dirty[round],
-                   last_round ? nullptr : a.dirty[round + 1], last_round ? 0 : a.g[round + 1], lane);
+    if (tile >= ntiles) return;
+    const bool elect = round == 0 && a.inline_election;
+    if (elect) entry_duty(a, tile, ntiles, lane);
+    tile_round(a, lo, g, tile, true, (elect || (round == 0 && !a.indices)) ? nullptr : a.dirty[round],
+               last_round ? nullptr : a.dirty[round + 1], last_round ? 0 : a.g[round + 1], lane,
+               s_win[threadIdx.x >> 6]);
 }
 
 // The top of the tree (everything above a.top_depth; the whole tree, leaves included, when it has
@@ -911,11 +979,12 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, Pu
 // multi-die part costs far more than a launch.
 constexpr int kTopWG = 1024;
 __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) {
+    __shared__ int s_win[kTopWG / 64][kBlockNodes];
     if (blockIdx.x >= 1) {
         rows_put_part(put, blockIdx.x - 1, put.blocks);
         return;
     }
-    top_rebuild(a, a.top_depth);
+    top_rebuild(a, a.top_depth, &s_win[0][0]);
     if (a.fold_max) {
         // The rounds before this launch read the running max as it was before the call (fresh slots
         // with an invalid priority take it), so it is raised only now.

@@ -108,7 +108,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
         if "k_per_sample_wide" in name:
             assert lds <= 1024, (name, lds)
         if "k_tree_update" in name:
-            assert lds <= 64, (name, lds)
+            assert lds == 4096, (name, lds)
 
 
 def test_create_replay_buffer_follows_the_reference_config_entry():
