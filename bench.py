@@ -108,19 +108,31 @@ def cpu_baseline(workload, shapes, np_dtypes, batch, seed):
     w = np.empty(batch, np.float32)
     dst = per._dst(batch)
     dptr = orc._ptr_array(dst)
-    calls, t_end = 0, time.perf_counter() + 12.0
     u_all = rng.random((64, batch)).astype(np.float32)
-    t0 = time.perf_counter()
-    while time.perf_counter() < t_end:
-        u = u_all[calls % 64]
-        rc = L.orc_per_sample(per.h, batch, 0.4, u.ctypes.data, idx.ctypes.data, w.ctypes.data, dptr)
-        assert rc == 0
-        calls += 1
-    dt = time.perf_counter() - t0
+
+    def timed(seconds):
+        calls, t_end = 0, time.perf_counter() + seconds
+        t0 = time.perf_counter()
+        while time.perf_counter() < t_end:
+            u = u_all[calls % 64]
+            rc = L.orc_per_sample(per.h, batch, 0.4, u.ctypes.data, idx.ctypes.data, w.ctypes.data, dptr)
+            assert rc == 0
+            calls += 1
+        return calls, time.perf_counter() - t0
+
+    calls, dt = timed(10.0)
+    # all host cores: the tree walk stays sequential, the row copies are shared out with OpenMP
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = max(1, min(cores, 16))
+    orc.set_threads(cores)
+    calls_mt, dt_mt = timed(4.0)
+    orc.set_threads(1)
     return {
         "value": calls * batch / dt, "unit": "transitions/s", "cores": 1, "kind": "port",
         "sample": "%d sample calls (batch %d, same row shape) in %.1f s on a capacity-%d buffer, 1 thread" % (
             calls, batch, dt, cap),
+        "all_cores": {"value": calls_mt * batch / dt_mt, "cores": cores,
+                      "sample": "%d calls in %.1f s, row copies on %d OpenMP threads" % (calls_mt, dt_mt, cores)},
     }
 
 

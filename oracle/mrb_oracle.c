@@ -137,6 +137,11 @@ int64_t orc_rng_below(uint64_t seed, uint64_t counter, uint64_t k, int64_t bound
     return (int64_t)(((unsigned __int128)orc_rng_u64(seed, counter, k) * (unsigned __int128)(uint64_t)bound) >> 64);
 }
 
+/* Threads used for the row copies of orc_per_sample / orc_urb_gather (1 = the
+ * sequential restatement; more only for the "all host cores" timing baseline). */
+static int orc_threads = 1;
+void orc_set_threads(int n) { orc_threads = n < 1 ? 1 : n; }
+
 /* ------------------------------------------------------------------------
  * Row storage: structure of arrays, field i = [capacity, bytes_i]
  * (mindspore_rl/core/uniform_replay_buffer.py:26-47).
@@ -239,10 +244,10 @@ int orc_urb_get_item(const orc_urb *b, int64_t index, void *const *dst) {
 
 /* Gather half of sample(): uniform_replay_buffer.py:130-139. */
 int orc_urb_gather(const orc_urb *b, const int64_t *indices, int64_t n, void *const *dst) {
-    for (int64_t k = 0; k < n; ++k) {
+    for (int64_t k = 0; k < n; ++k)
         if (indices[k] < 0 || indices[k] >= b->count) return 1;
-        rows_get(&b->rows, indices[k], dst, k);
-    }
+#pragma omp parallel for num_threads(orc_threads) schedule(static) if (orc_threads > 1)
+    for (int64_t k = 0; k < n; ++k) rows_get(&b->rows, indices[k], dst, k);
     return 0;
 }
 
@@ -470,7 +475,16 @@ int orc_per_sample(orc_per *b, int64_t batch, float beta, const float *uniforms,
         /* No clamp on the index: rounding in the last stratum can carry the
          * descent onto an unfilled leaf, and that index is returned as it is.
          * Only the row copy is kept inside the storage. */
-        if (out_fields) rows_get(&b->rows, idx < b->rows.capacity ? idx : b->rows.capacity - 1, out_fields, k);
+        if (out_fields && orc_threads <= 1)
+            rows_get(&b->rows, idx < b->rows.capacity ? idx : b->rows.capacity - 1, out_fields, k);
+    }
+    if (out_fields && orc_threads > 1) {
+        /* the all-cores baseline: the descent stays sequential, the row copies are shared out */
+#pragma omp parallel for num_threads(orc_threads) schedule(static)
+        for (int64_t k = 0; k < batch; ++k) {
+            int64_t idx = out_indices[k];
+            rows_get(&b->rows, idx < b->rows.capacity ? idx : b->rows.capacity - 1, out_fields, k);
+        }
     }
     if (!uniforms) b->calls += 1;
     return 0;

@@ -34,6 +34,7 @@ def lib():
     vp, i64, u64, f32 = C.c_void_p, C.c_int64, C.c_uint64, C.c_float
     pvp = C.POINTER(C.c_void_p)
     sig = {
+        "orc_set_threads": (None, [C.c_int]),
         "orc_powf": (f32, [f32, f32]),
         "orc_powf_n": (None, [vp, f32, vp, i64]),
         "orc_rng_u64": (u64, [u64, u64, u64]),
@@ -76,6 +77,11 @@ def lib():
         fn.argtypes = args
     _lib = L
     return L
+
+
+def set_threads(n):
+    """Threads for the row copies of sample / gather (1 = sequential; more only for timing baselines)."""
+    lib().orc_set_threads(int(n))
 
 
 def powf(x, a):
