@@ -233,6 +233,37 @@ __device__ __forceinline__ uint32_t group_walk(f32x16 v, int g, int lane, float&
     return 16u * w + (uint32_t)__builtin_amdgcn_readlane((int)in, (int)w);
 }
 
+// Four levels in one thread: `v` holds the 16 great-great-grandchildren of a node (64 contiguous
+// bytes); the three levels between are rebuilt with the additions the tree was built with and
+// walked with selects. Returns the offset of the node reached among the 16; `picked` is its value.
+__device__ __forceinline__ uint32_t walk16(f32x16 v, float& mass, float& picked) {
+    const f32x8 q8 = __builtin_shufflevector(v, v, 0, 2, 4, 6, 8, 10, 12, 14) +
+                     __builtin_shufflevector(v, v, 1, 3, 5, 7, 9, 11, 13, 15);
+    const f32x4 q4 = __builtin_shufflevector(q8, q8, 0, 2, 4, 6) + __builtin_shufflevector(q8, q8, 1, 3, 5, 7);
+    const float q2a = q4.x + q4.y;
+    bool r = !(mass <= q2a);
+    mass = r ? mass - q2a : mass;
+    uint32_t p = r ? 8u : 0u;
+    const float h4a = r ? q4.z : q4.x;
+    const f32x4 h8 = r ? q8.hi : q8.lo;
+    const f32x8 hv = r ? v.hi : v.lo;
+    r = !(mass <= h4a);
+    mass = r ? mass - h4a : mass;
+    p += r ? 4u : 0u;
+    const float g8a = r ? h8.z : h8.x;
+    const f32x4 gv = r ? hv.hi : hv.lo;
+    r = !(mass <= g8a);
+    mass = r ? mass - g8a : mass;
+    p += r ? 2u : 0u;
+    const float fa = r ? gv.z : gv.x;
+    const float fb = r ? gv.w : gv.y;
+    r = !(mass <= fa);
+    mass = r ? mass - fa : mass;
+    p += r ? 1u : 0u;
+    picked = r ? fb : fa;
+    return p;
+}
+
 // Number of round trips and the levels taken by each for a tree of `depth` levels.
 __device__ __forceinline__ int group_count(int depth) { return (depth + kGroupMaxLevels - 1) / kGroupMaxLevels; }
 __device__ __forceinline__ int group_levels(int depth, int count, int i) {

@@ -539,10 +539,18 @@ __global__ __launch_bounds__(kWG) void k_per_sample_lds(SampleArgs a, IoTable t,
                 node = 2 * node + 1;
             }
         }
-        // Below the staged levels every dependent load brings three levels at once: the 8
-        // great-grandchildren of `node` are 32 contiguous, aligned bytes; the two levels
-        // between are rebuilt with the additions the tree was built with.
+        // Below the staged levels every dependent load brings several levels at once: the 16
+        // (or 8) descendants of `node` four (three) levels down are 64 (32) contiguous, aligned
+        // bytes; the levels between are rebuilt with the additions the tree was built with.
         float picked = a.depth <= lds_levels ? s_top[node] : 0.0f;
+        for (; d + 4 <= a.depth; d += 4) {
+            const f32x4* src = reinterpret_cast<const f32x4*>(a.sum + ((uint64_t)node << 4));
+            const f32x4 t0 = src[0], t1 = src[1], t2 = src[2], t3 = src[3];
+            const f32x16 v = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
+                                                     __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2,
+                                                     3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+            node = (node << 4) + walk16(v, mass, picked);
+        }
         for (; d + 3 <= a.depth; d += 3) {
             const float4* src = reinterpret_cast<const float4*>(a.sum + ((uint64_t)node << 3));
             const float4 lo = src[0], hi = src[1];
