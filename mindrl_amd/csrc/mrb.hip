@@ -240,7 +240,6 @@ struct Per {
     int s_g0 = 0, s_rounds = 0, s_top = 0;
     int s_lo[kMaxRounds] = {}, s_g[kMaxRounds] = {};
     uint32_t* s_dirty[kMaxRounds] = {};
-    unsigned long long* owner = nullptr;
     float* powered = nullptr;  // scratch of the last update_priorities call, grown on demand
     int64_t powered_cap = 0;
     uint32_t* err = nullptr;
@@ -257,7 +256,6 @@ struct Per {
         if (stamp) (void)hipFree(stamp);
         if (maxp) (void)hipFree(maxp);
         if (powered) (void)hipFree(powered);
-        if (owner) (void)hipFree(owner);
         for (auto* d : s_dirty)
             if (d) (void)hipFree(d);
         if (err) (void)hipFree(err);
@@ -349,7 +347,6 @@ int next_epoch(Per& b, hipStream_t s) {
             HIP_TRY(hipMemsetAsync(b.dirty[r], 0, sizeof(uint32_t) * ((size_t)1 << (b.lo[r] - b.g[r])), s));
         for (int r = 0; r < b.s_rounds; ++r)
             HIP_TRY(hipMemsetAsync(b.s_dirty[r], 0, sizeof(uint32_t) * ((size_t)1 << (b.s_lo[r] - b.s_g[r])), s));
-        if (b.owner) HIP_TRY(hipMemsetAsync(b.owner, 0, sizeof(unsigned long long) * ((size_t)b.leaves >> b.s_g0), s));
         b.epoch += 1;
     }
     return MRB_OK;
@@ -610,9 +607,6 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
             HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->s_dirty[r]), nblocks * sizeof(uint32_t)));
             HIP_TRY(hipMemset(b->s_dirty[r], 0, nblocks * sizeof(uint32_t)));
         }
-        const size_t nown = (size_t)b->leaves >> b->s_g0;
-        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->owner), nown * sizeof(unsigned long long)));
-        HIP_TRY(hipMemset(b->owner, 0, nown * sizeof(unsigned long long)));
     }
     hipLaunchKernelGGL(k_fill_f32, dim3(grid_for(nodes)), dim3(kWG), 0, nullptr, b->mn, FLT_MAX, (uint64_t)nodes);
     LAUNCH_CHECK("k_fill_f32");
@@ -694,7 +688,6 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     const bool sparse = b->s_g0 > 0 && n <= (b->leaves >> 8);
     if (sparse) {
         a.sparse_g0 = b->s_g0;
-        a.owner = b->owner;
         a.nrounds = b->s_rounds;
         a.top_depth = b->s_top;
         for (int r = 0; r < kMaxRounds; ++r) {

@@ -661,12 +661,11 @@ struct UpdateArgs {
     int g[kMaxRounds];
     int top_depth;
     uint32_t* dirty[kMaxRounds];  // per round: one epoch word per block of 1 << g[r] nodes at depth lo[r]
-    // sparse updates of very large trees: the lowest sparse_g0 levels are rebuilt per entry
-    // (k_tree_sparse) instead of per tile; owner[block] elects one entry per block of leaves
     int fold_max;                // push with priorities: k_tree_top also folds them into the running max
     int inline_election;         // small update_priorities: no stamp pass, the leaf-level waves scan the entries
+    // sparse updates of very large trees: the lowest sparse_g0 levels are rebuilt per entry
+    // (k_tree_sparse) instead of per tile
     int sparse_g0;               // 0 = not used
-    unsigned long long* owner;   // [leaves >> sparse_g0]
 };
 
 __device__ __forceinline__ bool valid_priority(float p) { return p >= 0.0f && p <= 3.0e38f; }
@@ -685,10 +684,7 @@ __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
             if (a.indices) {
                 a.powered[j] = q;
                 atomicMax(&a.stamp[idx], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
-                if (a.sparse_g0)
-                    atomicMax(&a.owner[idx >> a.sparse_g0], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
-                else if (a.nrounds)
-                    a.dirty[0][idx >> a.g[0]] = a.epoch;
+                if (!a.sparse_g0 && a.nrounds) a.dirty[0][idx >> a.g[0]] = a.epoch;
             }
         }
     }
@@ -863,7 +859,7 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
 // Sparse lowest round for very large trees (e.g. 2^24 leaves, 65,536 entries): scanning
 // every 256-leaf tile costs more in wave launches than the update itself, so here the
 // ENTRIES drive the work. A group of L = 2^(g0-2) lanes (g0 = 4..6) takes one entry; if
-// that entry owns its block of 2^g0 leaves (integer-max election in k_update_stamp), the
+// that entry owns its block of 2^g0 leaves (it holds the largest of the block's stamps), the
 // group loads the block, replaces the leaves the stamps name, rebuilds the g0 levels
 // above with the same pairwise operations as tile_round and marks the next round's block.
 // ---------------------------------------------------------------------------
@@ -877,11 +873,25 @@ __global__ __launch_bounds__(kWG) void k_tree_sparse(UpdateArgs a) {
     int64_t idx = 0;
     if (active) {
         idx = a.indices[j];
-        active = idx >= 0 && idx < a.capacity && valid_priority(a.priorities[j]) &&
-                 a.owner[idx >> g0] == (((unsigned long long)a.epoch << 32) | (unsigned long long)j);
+        active = idx >= 0 && idx < a.capacity && valid_priority(a.priorities[j]);
     }
     const uint64_t block = (uint64_t)idx >> g0;
     const uint64_t first = (uint64_t)a.leaves + (block << g0);  // heap index of the block's first leaf
+    // The block's owner is the entry with the largest stamp of this call among its leaves: every
+    // group aimed at the block reads the same 2^g0 stamps and only the owner's group goes on.
+    unsigned long long top = 0;
+    if (active) {
+        const unsigned long long* st = a.stamp + (block << g0) + 4 * sub;
+        const unsigned long long s0 = st[0], s1 = st[1], s2 = st[2], s3 = st[3];
+        top = s0 > s1 ? s0 : s1;
+        top = top > s2 ? top : s2;
+        top = top > s3 ? top : s3;
+    }
+    for (uint32_t m = 1; m < group; m <<= 1) {
+        const unsigned long long o = __shfl_xor(top, (int)m);
+        top = top > o ? top : o;
+    }
+    active = active && top == (((unsigned long long)a.epoch << 32) | (unsigned long long)j);
     float4 vs = make_float4(0.f, 0.f, 0.f, 0.f), vm = vs;
     if (active) {
         vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * sub);
