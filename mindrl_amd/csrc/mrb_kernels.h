@@ -670,6 +670,13 @@ struct UpdateArgs {
 
 __device__ __forceinline__ bool valid_priority(float p) { return p >= 0.0f && p <= 3.0e38f; }
 
+// Folds q into the running max priority. Atomics on one address are serialised by the memory
+// system (~11 ns each), so the wave first looks at the current value: the max only grows, hence a
+// q that does not exceed what is already there can never matter, and nearly every wave skips.
+__device__ __forceinline__ void raise_max(float* maxp, float q) {
+    if (q > *reinterpret_cast<volatile float*>(maxp)) atomicMax(reinterpret_cast<unsigned int*>(maxp), __float_as_uint(q));
+}
+
 __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
     const int64_t j = (int64_t)blockIdx.x * kWG + threadIdx.x;
     float q = 0.0f;
@@ -690,7 +697,7 @@ __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
     }
     // wave max, then one integer atomic per wave
     for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
-    if ((threadIdx.x & 63) == 0 && q > 0.0f) atomicMax(reinterpret_cast<unsigned int*>(a.maxp), __float_as_uint(q));
+    if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
 }
 
 // New value of leaf `leaf`, if this call writes it.
@@ -947,7 +954,7 @@ __device__ __forceinline__ void entry_duty(const UpdateArgs& a, uint32_t wave_id
             if (idx_ok && valid_priority(p)) q = powf_det(p, a.alpha);
         }
         for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
-        if (lane == 0 && q > 0.0f) atomicMax(reinterpret_cast<unsigned int*>(a.maxp), __float_as_uint(q));
+        if (lane == 0 && q > 0.0f) raise_max(a.maxp, q);
     }
 }
 
@@ -1016,8 +1023,7 @@ __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) 
             }
         }
         for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
-        if ((threadIdx.x & 63) == 0 && q > 0.0f)
-            atomicMax(reinterpret_cast<unsigned int*>(a.maxp), __float_as_uint(q));
+        if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
     }
 }
 
