@@ -325,9 +325,15 @@ int read_and_clear_flags(uint32_t* d_err, uint32_t* flags, hipStream_t s) {
 int tree_rebuild(Per& b, const UpdateArgs& a, hipStream_t s, const PutArgs* ride = nullptr) {
     PutArgs none{};  // blocks == 0: no copy rides along
     for (int r = 0; r < b.nrounds; ++r) {
-        const uint32_t tiles = (1u << b.lo[r]) / kBlockNodes;
+        uint32_t tiles = (1u << b.lo[r]) / kBlockNodes;
+        uint32_t tile_base = 0;
+        if (r == 0 && !a.indices && a.first_slot + a.n <= a.capacity) {
+            // a push that does not wrap: only the leaf tiles under its slot range need a wave
+            tile_base = (uint32_t)(a.first_slot / kBlockNodes);
+            tiles = (uint32_t)((a.first_slot + a.n - 1) / kBlockNodes) - tile_base + 1;
+        }
         const PutArgs& put = (r == 0 && ride) ? *ride : none;
-        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4 + put.blocks), dim3(kWG), 0, s, a, r, put);
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4 + put.blocks), dim3(kWG), 0, s, a, r, tile_base, put);
         LAUNCH_CHECK("k_tree_update");
     }
     const PutArgs& put = (b.nrounds == 0 && ride) ? *ride : none;
@@ -710,7 +716,7 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     const PutArgs none{};
     for (int r = 0; r < b->s_rounds; ++r) {
         const uint32_t tiles = (1u << b->s_lo[r]) / kBlockNodes;
-        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r, none);
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r, 0u, none);
         LAUNCH_CHECK("k_tree_update");
     }
     hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a, none);

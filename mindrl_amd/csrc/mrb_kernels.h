@@ -977,7 +977,9 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, int* w
 
 // One wave per tile of round `round` (>= 0). A push lets its row copy ride along in the same
 // launch (the copy and the tree work touch different memory): workgroups past the tiles do it.
-__global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, PutArgs put) {
+// `tile_base`: the launch covers tiles tile_base, tile_base + 1, ... only (a push knows which leaf
+// tiles its slot range meets).
+__global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, uint32_t tile_base, PutArgs put) {
     __shared__ int s_win[kWG / 64][kBlockNodes];
     const uint32_t tile_blocks = gridDim.x - put.blocks;
     if (blockIdx.x >= tile_blocks) {
@@ -986,7 +988,7 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, Pu
     }
     const uint32_t lane = threadIdx.x & 63;
     const int lo = a.lo[round], g = a.g[round];
-    const uint32_t tile = blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
+    const uint32_t tile = tile_base + blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
     const uint32_t ntiles = (1u << lo) / kBlockNodes;
     const bool last_round = round + 1 == a.nrounds;
     if (tile >= ntiles) return;
