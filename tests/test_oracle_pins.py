@@ -465,3 +465,20 @@ def test_discounted_return_closed_forms(orc):
     r2[21:] += 5.0
     a2 = orc.discounted_return(r2, d2, v * 3, g)
     assert np.array_equal(a1[:21], a2[:21]) and not np.array_equal(a1[21:], a2[21:])
+
+
+def test_all_cores_mode_of_the_timing_baseline_changes_nothing(orc):
+    """The OpenMP mode used for the "all host cores" baseline only shares out the row copies."""
+    rng = np.random.default_rng(8)
+    per = orc.OraclePER(0.6, 500, [(33,), (1,)], [np.float32, np.int32], seed=2)
+    per.push([rng.normal(size=(500, 33)).astype(np.float32), np.arange(500, dtype=np.int32)[:, None]], 500)
+    per.update(np.arange(500), rng.lognormal(size=500).astype(np.float32))
+    u = rng.random(64).astype(np.float32)
+    one = per.sample(64, 0.5, u)
+    orc.set_threads(4)
+    try:
+        many = per.sample(64, 0.5, u)
+    finally:
+        orc.set_threads(1)
+    assert np.array_equal(one[0], many[0]) and np.array_equal(one[1], many[1])
+    assert all(np.array_equal(a, b) for a, b in zip(one[2], many[2]))
