@@ -130,3 +130,12 @@ def test_create_replay_buffer_follows_the_reference_config_entry():
     assert with_params.args == (2, 5, ((1,),), ("float32",))
     default_size = create_replay_buffer({"type": Fake, "capacity": 7, "data_shape": [(1,)], "data_type": ["int32"]})
     assert default_size.args[0] == 1
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """Every box has one GPU: `bench.py --gpus N` with N > 1 exits non-zero with a message, before touching a device."""
+    import subprocess
+    import sys
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                         stderr=subprocess.PIPE, text=True, timeout=120)
+    assert res.returncode != 0 and "one GPU" in res.stderr and res.stdout.strip() == ""
