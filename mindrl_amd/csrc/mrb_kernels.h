@@ -958,16 +958,17 @@ __device__ __forceinline__ void entry_duty(const UpdateArgs& a, uint32_t wave_id
     }
 }
 
-// Rebuilds everything above depth `top` (<= 12) with one workgroup: first up to 8 levels
-// over the 1..16 tiles of that depth (one wave each), then the rest in one tile.
-// `win`: 256 ints of LDS per wave (see tile_round).
+// Rebuilds everything above depth `top` (<= 16) with one workgroup: first up to 8 levels over
+// the tiles of that depth (shared out among the waves), then the rest in one tile. When `top`
+// is the leaf level, clean tiles are skipped like in a round. `win`: 256 ints of LDS per wave
+// (see tile_round).
 __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, int* win) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int g1 = top < kRoundLevels ? top : kRoundLevels;
     const uint32_t tiles = (1u << top) <= (uint32_t)kBlockNodes ? 1u : (1u << top) / kBlockNodes;
     if (a.inline_election && top == a.depth) entry_duty(a, wave, nwaves, lane);
     for (uint32_t t = wave; t < tiles; t += nwaves)
-        tile_round(a, top, g1, t, false, nullptr, nullptr, 0, lane, win + wave * kBlockNodes);
+        tile_round(a, top, g1, t, top == a.depth && g1 >= 2, nullptr, nullptr, 0, lane, win + wave * kBlockNodes);
     if (top > g1) {
         __threadfence_block();  // the tiles' parents, written by other waves of this workgroup, are read below
         __syncthreads();
