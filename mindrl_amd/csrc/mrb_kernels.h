@@ -13,7 +13,7 @@ namespace mrb {
 constexpr int kWG = 256;          // threads per workgroup of the row and sample kernels
 constexpr int kRoundLevels = 8;   // most tree levels rebuilt by one round of k_tree_update
 constexpr int kBlockNodes = 256;  // nodes per wave tile in k_tree_update (float4 per lane)
-constexpr int kTopMaxDepth = 12;  // deepest level the last workgroup's top rebuild starts from (4096 nodes)
+constexpr int kTopMaxDepth = 12;  // deepest level k_tree_top normally starts from (4096 nodes)
 
 // Per-call table of the fields of a row, passed to kernels by value.
 // `store` is the buffer's [capacity, row_bytes] matrix, `io` the caller's
@@ -63,60 +63,7 @@ __device__ __forceinline__ void copy_granule(gbyte* dst, const gbyte* src, uint3
     }
 }
 
-using granule_t = __attribute__((ext_vector_type(4))) uint32_t;
-
-// Load / store halves of copy_granule, for kernels that keep several granules
-// in flight per thread (all loads issued before the first store).
-__device__ __forceinline__ granule_t load_granule(const gbyte* src, uint32_t vl) {
-    granule_t r = 0;
-    switch (vl) {
-        case 4:
-            r = __builtin_nontemporal_load((const __attribute__((address_space(1))) granule_t*)src);
-            break;
-        case 3: {
-            using v2 = __attribute__((ext_vector_type(2))) uint32_t;
-            const v2 t = __builtin_nontemporal_load((const __attribute__((address_space(1))) v2*)src);
-            r.x = t.x;
-            r.y = t.y;
-            break;
-        }
-        case 2:
-            r.x = *(const __attribute__((address_space(1))) uint32_t*)src;
-            break;
-        case 1:
-            r.x = *(const __attribute__((address_space(1))) uint16_t*)src;
-            break;
-        default:
-            r.x = *src;
-            break;
-    }
-    return r;
-}
-
-__device__ __forceinline__ void store_granule(gbyte* dst, granule_t r, uint32_t vl) {
-    switch (vl) {
-        case 4:
-            __builtin_nontemporal_store(r, (__attribute__((address_space(1))) granule_t*)dst);
-            break;
-        case 3: {
-            using v2 = __attribute__((ext_vector_type(2))) uint32_t;
-            v2 t;
-            t.x = r.x;
-            t.y = r.y;
-            __builtin_nontemporal_store(t, (__attribute__((address_space(1))) v2*)dst);
-            break;
-        }
-        case 2:
-            *(__attribute__((address_space(1))) uint32_t*)dst = r.x;
-            break;
-        case 1:
-            *(__attribute__((address_space(1))) uint16_t*)dst = (uint16_t)r.x;
-            break;
-        default:
-            *dst = (uint8_t)r.x;
-            break;
-    }
-}
+using granule_t = __attribute__((ext_vector_type(4))) uint32_t;  // one 16-byte copy granule
 
 __device__ __forceinline__ int field_of(const IoTable& t, uint64_t w) {
     int f = 0;
