@@ -233,6 +233,22 @@ __device__ __forceinline__ uint32_t group_walk(f32x16 v, int g, int lane, float&
     return 16u * w + (uint32_t)__builtin_amdgcn_readlane((int)in, (int)w);
 }
 
+// Sum of all the nodes a wave holds in `v` (16 per lane), paired exactly as group_walk pairs them,
+// i.e. the value the tree stores in the node ten levels above a full group.
+__device__ __forceinline__ float group_total(f32x16 v) {
+    const f32x8 q8 = __builtin_shufflevector(v, v, 0, 2, 4, 6, 8, 10, 12, 14) +
+                     __builtin_shufflevector(v, v, 1, 3, 5, 7, 9, 11, 13, 15);
+    const f32x4 q4 = __builtin_shufflevector(q8, q8, 0, 2, 4, 6) + __builtin_shufflevector(q8, q8, 1, 3, 5, 7);
+    float c = (q4.x + q4.y) + (q4.z + q4.w);
+    c = c + dpp_move<0xB1>(c);
+    c = c + dpp_move<0x4E>(c);
+    c = c + dpp_move<0x141>(c);
+    c = c + dpp_move<0x140>(c);
+    c = c + __shfl_xor(c, 16);
+    c = c + __shfl_xor(c, 32);
+    return c;
+}
+
 // Four levels in one thread: `v` holds the 16 great-great-grandchildren of a node (64 contiguous
 // bytes); the three levels between are rebuilt with the additions the tree was built with and
 // walked with selects. Returns the offset of the node reached among the 16; `picked` is its value.

@@ -297,6 +297,57 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
             s_idx = slot;
             s_picked = 0.0f;
         }
+    } else if (depth == 21 || depth == 22) {
+        // Trees of 21 and 22 levels would need three dependent node groups of <= 10 levels. Instead
+        // two (four) waves share the 2048 (4096) nodes at depth 11 (12), whose address is known: each
+        // reduces its 1024 nodes, the wave totals - the tree's nodes at depth 1 (2) - meet in LDS, every
+        // wave takes the one (two) top steps of the walk from them, and the wave the walk enters goes on
+        // through its ten levels and the ten below. Two dependent loads again, one barrier more.
+        __shared__ float s_tot[4];
+        const int share = depth - 20;  // log2 of the waves sharing the top group
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        f32x16 v = 0.0f;
+        float total = 0.0f, u = 0.0f;
+        if (wave < (1 << share)) {
+            f32x4 r0, r1, r2, r3;
+            group_request(sum, (1u << share) + wave, kGroupMaxLevels, lane, r0, r1, r2, r3);
+            total = sum[1];
+            u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
+            __builtin_amdgcn_sched_barrier(0);
+            v = group_finish(kGroupMaxLevels, lane, r0, r1, r2, r3);
+            const float mine = group_total(v);
+            if (lane == 0) s_tot[wave] = mine;
+        }
+        __syncthreads();
+        if (wave < (1 << share)) {
+            float mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
+            uint32_t q = 0;
+            if (share == 2) {
+                const float left = s_tot[0] + s_tot[1];  // the node at depth 1
+                if (!(mass <= left)) {
+                    mass -= left;
+                    q = 2;
+                }
+            }
+            const float left = s_tot[q];
+            if (!(mass <= left)) {
+                mass -= left;
+                q += 1;
+            }
+            if ((uint32_t)wave == q) {
+                float picked;
+                uint32_t node = (((1u << share) + q) << kGroupMaxLevels) + group_walk(v, kGroupMaxLevels, lane, mass, picked);
+                f32x4 r0, r1, r2, r3;
+                group_request(sum, node, kGroupMaxLevels, lane, r0, r1, r2, r3);
+                __builtin_amdgcn_sched_barrier(0);
+                node = (node << kGroupMaxLevels) +
+                       group_walk(group_finish(kGroupMaxLevels, lane, r0, r1, r2, r3), kGroupMaxLevels, lane, mass, picked);
+                if (lane == 0) {
+                    s_idx = (int64_t)node - a.leaves;
+                    s_picked = picked;
+                }
+            }
+        }
     } else if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
         const int ngroups = group_count(depth);
