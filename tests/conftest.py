@@ -10,6 +10,10 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a HIP device (MI355X); run with -m gpu")
+    # the tests load what is built; only a tree with nothing built (a fresh checkout) compiles here
+    from mindrl_amd import _lib, build
+    if not os.path.exists(_lib.LIB_PATH):
+        build.build()
 
 
 @pytest.fixture(scope="session")
