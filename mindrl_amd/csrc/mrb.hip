@@ -162,8 +162,13 @@ int launch_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, hipStr
     SplitPlan plan{};
     plan.split = wide_split(r);
     for (int i = 0; i < r.nfields; ++i) plan.per[i] = (r.units[i] + plan.split - 1) / plan.split;
-    hipLaunchKernelGGL(k_per_sample_wide, dim3((uint32_t)(a.batch * plan.split)), dim3(kWG), 0, s, a.sum, a.uniforms,
-                       a.depth, plan.split, a.batch, a.seed, a.calls, a, t, plan);
+    if (a.mode == kFromTree) {
+        hipLaunchKernelGGL(k_per_sample_wide<true>, dim3((uint32_t)(a.batch * plan.split)), dim3(kWG), 0, s, a.sum,
+                           a.uniforms, a.depth, plan.split, a.batch, a.seed, a.calls, a, t, plan);
+    } else {
+        hipLaunchKernelGGL(k_per_sample_wide<false>, dim3((uint32_t)(a.batch * plan.split)), dim3(kWG), 0, s, a.sum,
+                           a.uniforms, a.depth, plan.split, a.batch, a.seed, a.calls, a, t, plan);
+    }
     LAUNCH_CHECK("k_per_sample_wide");
     return MRB_OK;
 }

@@ -101,7 +101,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
         kernels[name] = (int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
-    assert len(kernels) == 13, sorted(kernels)
+    assert len(kernels) == 14, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)
