@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
                                                          int depth, int split_arg, int64_t batch, uint64_t seed,
                                                          uint64_t calls, SampleArgs a, IoTable t, SplitPlan plan) {
     __shared__ int64_t s_idx;
-    __shared__ float s_picked;
+    __shared__ float s_picked, s_total, s_pmin;
     // this workgroup's share of each field, filled by wave 1 while wave 0 walks the tree
     __shared__ const gbyte* s_src[MRB_MAX_FIELDS];  // store_f + first granule's byte offset
     __shared__ gbyte* s_dst[MRB_MAX_FIELDS];          // io_f + k * row_bytes + the same offset
@@ -350,6 +350,7 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
                 if (lane == 0) {
                     s_idx = (int64_t)node - a.leaves;
                     s_picked = picked;
+                    s_total = total;
                 }
             }
         }
@@ -358,7 +359,7 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
         const int ngroups = group_count(depth);
         int g = ngroups ? group_levels(depth, ngroups, 0) : 0;
         uint32_t node;
-        float picked, mass;
+        float picked, mass, total_w0;
         if (depth >= 2) {
             // The first group hangs under the root: its address is known, so it is requested
             // together with the total and the draw; the scheduling barrier keeps every
@@ -368,6 +369,7 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
             const float total = sum[1];
             const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
             __builtin_amdgcn_sched_barrier(0);
+            total_w0 = total;
             mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
             node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
             for (int i = 1; i < ngroups; ++i) {
@@ -379,6 +381,7 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
         } else {
             // one or two leaves
             const float total = sum[1];
+            total_w0 = total;
             mass = stratum_mass(a, total, k);
             picked = total;
             node = (1u << g) + (g ? group_walk(group_load_tiny(sum, 1u, g, lane), g, lane, mass, picked) : 0u);
@@ -386,8 +389,10 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
         if (lane == 0) {
             s_idx = (int64_t)node - a.leaves;
             s_picked = picked;
+            s_total = total_w0;
         }
     }
+    if (kTree && threadIdx.x == 64 + MRB_MAX_FIELDS) s_pmin = a.mn[1];  // for the weight, fetched while wave 0 walks
     // (separate from the chain above: in the gather modes every thread takes its first branch)
     if (threadIdx.x >= 64 && threadIdx.x < 64 + MRB_MAX_FIELDS) {
         const int f = threadIdx.x - 64;
@@ -480,8 +485,8 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
             if (wfirst == 0 && part == 0 && threadIdx.x == 0 && a.out_idx) a.out_idx[k] = idx;
         } else if (wfirst == 0 && part == 0 && threadIdx.x < 2) {
             // lane 0: (p / total * size)^-beta, lane 1: (pmin / total * size)^-beta
-            const float total = a.sum[1];
-            const float x = threadIdx.x == 0 ? s_picked : a.mn[1];
+            const float total = s_total;
+            const float x = threadIdx.x == 0 ? s_picked : s_pmin;
             const float r = powf_det(x / total * (float)a.size, -a.beta);
             const float max_w = __shfl(r, 1);
             if (threadIdx.x == 0) {
