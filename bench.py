@@ -381,14 +381,14 @@ def main():
     if a.workload == "dr":
         return bench_discounted_return(a)
     capacity, batch, shapes, np_dtypes, upd_n, ins_n, desc = WORKLOADS[a.workload]
-    _lib.set_option("row_split", a.row_split)
-    _lib.set_option("sample_path", a.sample_path)
     if a.capacity:
         capacity = a.capacity
         desc += " [capacity overridden to %d]" % capacity
     seed = 1000 + int(a.workload[1])
     t_types = [getattr(torch, d) for d in np_dtypes]
     buf = PriorityReplayBuffer(0.6, capacity, batch, shapes, t_types, seed0=seed)
+    buf.set_option("row_split", a.row_split)
+    buf.set_option("sample_path", a.sample_path)
     t0 = time.perf_counter()
     fill_per(buf, torch, capacity, shapes, np_dtypes, seed)
     fill_s = time.perf_counter() - t0

@@ -60,11 +60,12 @@ const char *mrb_last_error(void);
 int mrb_backend(void);
 /* ABI version of this header. */
 int mrb_version(void);
-/* Tuning knobs; unknown names return MRB_EINVAL.
- *   "sample_path"  0 = choose by row size, 1 = force wide-row kernel, 2 = force LDS-top kernel
- *   "row_split"    workgroups per sampled row in the wide-row kernel (0 = auto)
- *   "lds_levels"   tree levels staged in LDS by the LDS-top kernel (0 = auto, max 12) */
-int mrb_set_option(const char *name, int64_t value);
+/* Tuning knobs of ONE buffer (any kind of handle); they change how its kernels are launched, never a
+ * result. Unknown names return MRB_EINVAL. Set them while no call on the handle is in progress.
+ *   "row_split"    least number of workgroups per row in the wide-row kernel (0 = auto, max 64)
+ *   "sample_path"  prioritized buffers: 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
+ *   "lds_levels"   prioritized buffers: tree levels staged in LDS by the LDS-top kernel (0 = auto, max 12) */
+int mrb_set_option(int64_t h, const char *name, int64_t value);
 
 /* ---- uniform FIFO ring buffer ----------------------------------------- */
 

@@ -21,7 +21,7 @@ _pi64 = C.POINTER(C.c_int64)
 SIGNATURES = {
     "mrb_backend": [],
     "mrb_version": [],
-    "mrb_set_option": [C.c_char_p, _i64],
+    "mrb_set_option": [_i64, C.c_char_p, _i64],
     "mrb_urb_create": [_i64, _int, _pi64, _pi64],
     "mrb_urb_append": [_i64, _pvp, _i64, _vp],
     "mrb_urb_append_from": [_i64, _i64, _i64, _i64, _vp],
@@ -101,8 +101,9 @@ def check(rc):
     raise MrbError(rc, msg)
 
 
-def set_option(name, value):
-    check(lib().mrb_set_option(name.encode(), int(value)))
+def set_option(handle, name, value):
+    """Sets a launch option of one buffer (see mrb_set_option in include/mrb.h)."""
+    check(lib().mrb_set_option(int(handle), name.encode(), int(value)))
 
 
 def ptr_array(pointers):

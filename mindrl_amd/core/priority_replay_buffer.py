@@ -206,6 +206,11 @@ class PriorityReplayBuffer:
             raise ValueError("sample: total priority is not positive and finite")
         return f
 
+    def set_option(self, name, value):
+        """Sets a launch option of this buffer ("row_split"; prioritized buffers also "sample_path",
+        "lds_levels"). Options change how kernels are launched, never a result."""
+        _lib.set_option(self._h, name, value)
+
     def __del__(self):
         # the native buffer (rows, trees) is released with the Python object if destroy() was not called
         try:

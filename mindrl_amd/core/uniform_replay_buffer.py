@@ -191,6 +191,11 @@ class UniformReplayBuffer:
             h, self._h = self._h, 0
             _lib.check(_lib.lib().mrb_urb_destroy(h))
 
+    def set_option(self, name, value):
+        """Sets a launch option of this buffer ("row_split"; prioritized buffers also "sample_path",
+        "lds_levels"). Options change how kernels are launched, never a result."""
+        _lib.set_option(self._h, name, value)
+
     def __del__(self):
         # the native buffer (rows, trees) is released with the Python object if destroy() was not called
         try:

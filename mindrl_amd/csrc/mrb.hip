@@ -40,12 +40,6 @@ int fail(int code, const char* fmt, ...) {
         if (e_ != hipSuccess) return fail(MRB_EHIP, "launch %s: %s", name, hipGetErrorString(e_)); \
     } while (0)
 
-struct Options {
-    int64_t sample_path = 0;
-    int64_t row_split = 0;
-    int64_t lds_levels = 0;
-} g_opt;
-
 // Row storage: structure of arrays, field i = [capacity, bytes_i]
 // (reference layout: mindspore_rl/core/uniform_replay_buffer.py:26-47).
 struct RowStore {
@@ -55,6 +49,7 @@ struct RowStore {
     uint8_t* data[MRB_MAX_FIELDS] = {};
     uint32_t vec_log2[MRB_MAX_FIELDS] = {};
     uint32_t units[MRB_MAX_FIELDS] = {};
+    int64_t row_split = 0;  // option "row_split": least number of workgroups per row in the wide-row kernel (0 = auto)
 
     ~RowStore() {
         for (int i = 0; i < nfields; ++i)
@@ -140,17 +135,6 @@ int rows_put(const RowStore& r, const void* const* src, int64_t skip, int64_t n,
     return MRB_OK;
 }
 
-// Workgroups per row for the wide-row kernel: one pass of kInFlight granules per thread covers the
-// widest field (measured best on 28 KB rows: 2 workgroups per row).
-int wide_split(const RowStore& r) {
-    if (g_opt.row_split > 0) return (int)g_opt.row_split;
-    uint32_t max_units = 0;
-    for (int i = 0; i < r.nfields; ++i)
-        if (r.units[i] > max_units) max_units = r.units[i];
-    int split = (int)((max_units + kInFlight * kWG - 1) / (kInFlight * kWG));
-    return split < 1 ? 1 : (split > 16 ? 16 : split);
-}
-
 int64_t widest_field(const RowStore& r) {
     int64_t m = 0;
     for (int i = 0; i < r.nfields; ++i)
@@ -158,25 +142,89 @@ int64_t widest_field(const RowStore& r) {
     return m;
 }
 
-int launch_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, hipStream_t s) {
-    SplitPlan plan{};
-    plan.split = wide_split(r);
-    for (int i = 0; i < r.nfields; ++i) plan.per[i] = (r.units[i] + plan.split - 1) / plan.split;
-    if (a.mode == kFromTree) {
-        hipLaunchKernelGGL(k_per_sample_wide<true>, dim3((uint32_t)(a.batch * plan.split)), dim3(kWG), 0, s, a.sum,
-                           a.uniforms, a.depth, plan.split, a.batch, a.seed, a.calls, a, t, plan);
-    } else {
-        hipLaunchKernelGGL(k_per_sample_wide<false>, dim3((uint32_t)(a.batch * plan.split)), dim3(kWG), 0, s, a.sum,
-                           a.uniforms, a.depth, plan.split, a.batch, a.seed, a.calls, a, t, plan);
+// Describes n rows of `r` for the wide-row kernels: one workgroup per row unless a row holds more than
+// kMaxInFlight * kCopyThreads (2048) wide granules, or the buffer's "row_split" option asks for more.
+// Returns the number of granules a copy thread holds (2 or 8) or 0 on error.
+int wide_plan(const RowStore& r, const IoTable& t, int64_t n, WidePlan& plan, dim3& grid) {
+    plan = WidePlan{};
+    for (int i = 0; i < r.nfields; ++i) plan.nwide += r.vec_log2[i] == 4;
+    plan.nnarrow = r.nfields - plan.nwide;
+    int w = 0, m = plan.nwide;
+    for (int i = 0; i < r.nfields; ++i) {
+        const bool wide = r.vec_log2[i] == 4;
+        const int q = wide ? w++ : m++;
+        plan.f[q].src = t.store[i];
+        plan.f[q].dst = t.io[i];
+        plan.f[q].rb = t.row_bytes[i];
+        uint32_t& items = wide ? plan.wide_items : plan.narrow_items;
+        plan.f[q].first = items;
+        items += wide ? r.units[i] : t.row_bytes[i];
+    }
+    const uint32_t per_wg = (uint32_t)kMaxInFlight * kCopyThreads;
+    uint32_t split = (plan.wide_items + per_wg - 1) / per_wg;
+    if (r.row_split > (int64_t)split) split = (uint32_t)r.row_split;
+    if (split < 1) split = 1;
+    plan.split = (int)split;
+    plan.share = (plan.wide_items + split - 1) / split;
+    if (n > 0x7fffffffll || split > 65535u) {
+        fail(MRB_EINVAL, "%lld rows of %u workgroups each exceed one launch", (long long)n, split);
+        return 0;
+    }
+    grid = dim3((uint32_t)n, split);
+    const uint32_t per_thread = (plan.share + kCopyThreads - 1) / kCopyThreads;  // <= kMaxInFlight
+    return per_thread <= 2 ? 2 : 8;
+}
+
+// The descent plan of a tree of `depth` levels as the wide-row sample kernel takes it: bits 0-3 the
+// number of node groups (one dependent load each), then 5 bits per group with its levels (<= 10).
+uint32_t pack_groups(int depth) {
+    const int count = (depth + kGroupMaxLevels - 1) / kGroupMaxLevels;
+    uint32_t packed = (uint32_t)count;
+    for (int i = 0; i < count; ++i) packed |= (uint32_t)(depth / count + (i < depth % count ? 1 : 0)) << (4 + 5 * i);
+    return packed;
+}
+
+template <int kInF, bool kTen, bool kOneWide>
+void launch_sample_wide(dim3 grid, const SampleArgs& a, const WidePlan& plan, hipStream_t s) {
+    const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
+    hipLaunchKernelGGL((k_per_sample_wide<kInF, kTen, kOneWide>), grid, dim3(kWideWG), 0, s, a.sum, a.uniforms, a.depth,
+                       pack_groups(a.depth), (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, tail, plan);
+}
+
+template <int kInF>
+void launch_sample_wide_as(dim3 grid, const SampleArgs& a, const WidePlan& plan, hipStream_t s) {
+    const bool ten = a.depth > 0 && a.depth % kGroupMaxLevels == 0;  // every node group takes 10 levels
+    const bool one = plan.nwide == 1;
+    if (ten) one ? launch_sample_wide<kInF, true, true>(grid, a, plan, s) : launch_sample_wide<kInF, true, false>(grid, a, plan, s);
+    else one ? launch_sample_wide<kInF, false, true>(grid, a, plan, s) : launch_sample_wide<kInF, false, false>(grid, a, plan, s);
+}
+
+int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, hipStream_t s) {
+    WidePlan plan;
+    dim3 grid;
+    switch (wide_plan(r, t, a.batch, plan, grid)) {
+        case 0: return MRB_EINVAL;
+        case 2: launch_sample_wide_as<2>(grid, a, plan, s); break;
+        default: launch_sample_wide_as<8>(grid, a, plan, s); break;
     }
     LAUNCH_CHECK("k_per_sample_wide");
     return MRB_OK;
 }
 
+template <int kInF>
+void launch_gather_wide(dim3 grid, const int64_t* indices, int mode, int64_t count, int64_t fixed_slot, uint64_t seed,
+                        uint64_t calls, int64_t* out_indices, uint32_t* err, const WidePlan& plan, hipStream_t s) {
+    if (plan.nwide == 1)
+        hipLaunchKernelGGL((k_rows_gather_wide<kInF, true>), grid, dim3(kWideWG), 0, s, indices, mode, count, fixed_slot, seed,
+                           calls, out_indices, err, plan);
+    else
+        hipLaunchKernelGGL((k_rows_gather_wide<kInF, false>), grid, dim3(kWideWG), 0, s, indices, mode, count, fixed_slot, seed,
+                           calls, out_indices, err, plan);
+}
+
 // Gather of n rows whose slots are given (indices), drawn from the generator (indices NULL,
-// fixed_slot < 0) or one fixed slot. Rows of at least 1 KB go through the wide-row kernel
-// (a workgroup per row part, all loads before the first store), narrow rows through the
-// flat kernel.
+// fixed_slot < 0) or one fixed slot. Rows with a field of at least 1 KB go through the wide-row
+// kernel (a workgroup per row, all loads before the first store), narrow rows through the flat kernel.
 int gather_rows(const RowStore& r, const int64_t* indices, int64_t fixed_slot, int64_t count, uint64_t seed,
                 uint64_t calls, int64_t n, int64_t* out_indices, void* const* dst_fields, uint32_t* err,
                 hipStream_t s) {
@@ -184,18 +232,16 @@ int gather_rows(const RowStore& r, const int64_t* indices, int64_t fixed_slot, i
     int rc = make_table(r, dst_fields, n, t);
     if (rc) return rc;
     if (widest_field(r) >= 1024 && n <= (1ll << 24)) {
-        SampleArgs a{};
-        a.batch = n;
-        a.seed = seed;
-        a.calls = calls;
-        a.capacity = r.capacity;
-        a.out_idx = out_indices;
-        a.err = err;
-        a.mode = fixed_slot >= 0 ? kFromFixedSlot : (indices ? kFromIndices : kFromGenerator);
-        a.given = indices;
-        a.fixed_slot = fixed_slot;
-        a.count = count;
-        return launch_wide(r, a, t, s);
+        const int mode = fixed_slot >= 0 ? kFromFixedSlot : (indices ? kFromIndices : kFromGenerator);
+        WidePlan plan;
+        dim3 grid;
+        switch (wide_plan(r, t, n, plan, grid)) {
+            case 0: return MRB_EINVAL;
+            case 2: launch_gather_wide<2>(grid, indices, mode, count, fixed_slot, seed, calls, out_indices, err, plan, s); break;
+            default: launch_gather_wide<8>(grid, indices, mode, count, fixed_slot, seed, calls, out_indices, err, plan, s); break;
+        }
+        LAUNCH_CHECK("k_rows_gather_wide");
+        return MRB_OK;
     }
     hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, r.capacity, count,
                        indices, fixed_slot, seed, calls, out_indices, err);
@@ -255,6 +301,8 @@ struct Per {
     int top_depth = 0;
     uint64_t epoch = 0;
     uint64_t seed = 0, calls = 0;
+    int64_t sample_path = 0;  // option "sample_path": 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
+    int64_t lds_levels = 0;   // option "lds_levels": tree levels staged in LDS by the LDS-top kernel (0 = auto)
     ~Per() {
         if (sum) (void)hipFree(sum);
         if (mn) (void)hipFree(mn);
@@ -402,17 +450,27 @@ const char* mrb_last_error(void) { return g_err; }
 int mrb_backend(void) { return 1; }
 int mrb_version(void) { return 1; }
 
-int mrb_set_option(const char* name, int64_t value) {
+int mrb_set_option(int64_t h, const char* name, int64_t value) {
     if (!name) return fail(MRB_EINVAL, "option name is NULL");
-    if (!strcmp(name, "sample_path")) {
-        if (value < 0 || value > 2) return fail(MRB_EINVAL, "sample_path must be 0, 1 or 2");
-        g_opt.sample_path = value;
-    } else if (!strcmp(name, "row_split")) {
+    RowStore* rows = nullptr;
+    std::shared_ptr<Per> per = find_per(h);
+    std::shared_ptr<Urb> urb = per ? nullptr : find_urb(h);
+    std::shared_ptr<Res> res = (per || urb) ? nullptr : find_res(h);
+    if (per) rows = &per->rows;
+    if (urb) rows = &urb->rows;
+    if (res) rows = &res->rows;
+    if (!rows) return fail(MRB_EHANDLE, "unknown buffer handle %lld", (long long)h);
+    if (!strcmp(name, "row_split")) {
         if (value < 0 || value > 64) return fail(MRB_EINVAL, "row_split must be in [0, 64]");
-        g_opt.row_split = value;
+        rows->row_split = value;
+    } else if (!strcmp(name, "sample_path")) {
+        if (!per) return fail(MRB_EINVAL, "sample_path is an option of prioritized buffers");
+        if (value < 0 || value > 2) return fail(MRB_EINVAL, "sample_path must be 0, 1 or 2");
+        per->sample_path = value;
     } else if (!strcmp(name, "lds_levels")) {
+        if (!per) return fail(MRB_EINVAL, "lds_levels is an option of prioritized buffers");
         if (value < 0 || value > 12) return fail(MRB_EINVAL, "lds_levels must be in [0, 12]");
-        g_opt.lds_levels = value;
+        per->lds_levels = value;
     } else {
         return fail(MRB_EINVAL, "unknown option '%s'", name);
     }
@@ -763,15 +821,14 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, 
     a.out_idx = out_indices;
     a.out_w = out_weights;
     a.err = b->err;
-    a.mode = kFromTree;
     const int64_t max_bytes = widest_field(b->rows);
-    int path = (int)g_opt.sample_path;
+    int path = (int)b->sample_path;
     if (path == 0) path = (batch >= 8192 && max_bytes <= 256) ? 2 : 1;
     if (path == 1) {
-        rc = launch_wide(b->rows, a, t, s);
+        rc = sample_wide(b->rows, a, t, s);
         if (rc) return rc;
     } else {
-        int levels = g_opt.lds_levels > 0 ? (int)g_opt.lds_levels : 12;
+        int levels = b->lds_levels > 0 ? (int)b->lds_levels : 12;
         if (levels > b->depth) levels = b->depth;
         const uint32_t ntop = (2u << levels) < 4 ? 4 : (2u << levels);
         const size_t lds = ntop * sizeof(float) + kWG * sizeof(int64_t);

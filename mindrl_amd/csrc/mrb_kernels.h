@@ -200,8 +200,8 @@ __global__ __launch_bounds__(kWG) void k_res_put(IoTable t, const unsigned long 
     }
 }
 
-// Arguments common to both sample kernels (the wide-row kernel additionally takes the
-// fields its tree descent needs first as plain leading parameters).
+// Arguments of a PER sample (the wide-row kernel takes what its tree walk needs as plain leading
+// parameters instead).
 struct SampleArgs {
     const float* sum;       // sum tree, heap order
     const float* uniforms;  // f32[batch] or NULL -> generator
@@ -216,14 +216,7 @@ struct SampleArgs {
     int64_t* out_idx;
     float* out_w;
     uint32_t* err;
-    // Where row k comes from. The wide-row kernel also serves plain gathers of wide rows
-    // (BufferSample / BufferGetItem / rows at given slots), which skip the tree altogether.
-    int mode;              // kFromTree, kFromIndices, kFromGenerator, kFromFixedSlot
-    const int64_t* given;  // kFromIndices: slot of row k
-    int64_t fixed_slot;    // kFromFixedSlot
-    int64_t count;         // kFromIndices / kFromGenerator: valid slots are [0, count)
 };
-constexpr int kFromTree = 0, kFromIndices = 1, kFromGenerator = 2, kFromFixedSlot = 3;
 
 // mass of stratum k: (u + k) * (total / batch), each operation rounded once.
 __device__ __forceinline__ float stratum_mass(const SampleArgs& a, float total, int64_t k, float u) {
@@ -245,86 +238,302 @@ __device__ __forceinline__ void sample_flags(const SampleArgs& a, float total, i
     if (idx >= a.size) atomicOr(a.err, MRB_DERR_UNFILLED);
 }
 
-// How the wide-row sample kernel divides a row among `split` workgroups:
-// workgroup `part` copies granules [part * per[f], (part + 1) * per[f]) of field f.
-struct SplitPlan {
-    int split;
-    uint32_t per[MRB_MAX_FIELDS];
+// ---------------------------------------------------------------------------
+// Wide rows (at least one field of 1 KB or more): k_per_sample_wide (PER sample)
+// and k_rows_gather_wide (gather at given / drawn / fixed slots).
+//
+// A row's fields are of two kinds: "wide" fields, whose rows are multiples of
+// 16 bytes and are copied in 16-byte granules, and "narrow" fields (the
+// others: scalars and short vectors), copied byte by byte. The granules
+// (bytes) of each kind are numbered consecutively over the fields. `split` workgroups share a row (one unless a
+// row has more than 2048 wide granules); workgroup `part` copies wide granules
+// [part * share, (part + 1) * share), the row's first workgroup also the
+// narrow ones. A workgroup is one "walker" wave and four copy waves:
+//   walker   finds the row's slot - for a sample by walking the sum tree with
+//            group_request / group_walk (one dependent load per 10 levels; the
+//            first group sits under the root, so it is requested together with
+//            the total and the uniform draw) - using nothing but kernel
+//            arguments preloaded into scalar registers, and publishes it
+//            through LDS. Afterwards it copies the narrow fields, computes the
+//            importance weight (the two powers in two lanes of one instruction
+//            stream) and writes index and weight, off the copy waves' path.
+//   copy     meanwhile every copy thread works out where its up to kInF
+//            granules lie within a row (field, offset, destination) from the
+//            field table, and the first copy wave stages in LDS what the
+//            walker needs afterwards (narrow-field table, output pointers,
+//            the minimum priority). After the barrier one multiply-add per
+//            granule gives the source address; all loads are issued before
+//            the first store: a row costs one memory round trip, not one per
+//            field.
+// Everything read from the kernel-argument segment costs a memory round trip
+// of its own when a kernel starts (nothing is cached across launches), which
+// is why the walker touches none of it before the barrier and the copy waves
+// fetch the table in one round.
+// Sampling reads its rows non-temporally so that they do not push the tree
+// out of the caches; the gathered batch is stored with ordinary stores (it is
+// what the caller reads next).
+// ---------------------------------------------------------------------------
+struct WideField {  // one table entry, 32 bytes
+    const uint8_t* src;  // storage [capacity, row_bytes]
+    uint8_t* dst;        // the caller's [batch, row_bytes] matrix
+    uint32_t rb;         // row_bytes
+    uint32_t first;      // wide field: number of its first granule among the wide ones; narrow: of its first byte
+    uint32_t pad[2];
+};
+struct WidePlan {
+    int split;              // workgroups per row
+    uint32_t share;         // wide granules per workgroup
+    uint32_t wide_items;    // wide granules per row
+    uint32_t narrow_items;  // bytes of narrow fields per row
+    int nwide, nnarrow;     // fields of each kind
+    uint32_t pad[2];
+    WideField f[MRB_MAX_FIELDS];  // the wide fields first, then the narrow ones
 };
 
-constexpr int kInFlight = 4;  // granules a thread holds between its loads and its stores
+// What the walker of a sample needs after the descent.
+struct SampleTail {
+    const float* mn;  // min tree, heap order
+    int64_t* out_idx;
+    float* out_w;
+    uint32_t* err;
+    int64_t size;
+    float beta;
+};
 
-// ---------------------------------------------------------------------------
-// PER sample, wide rows: `split` workgroups per sampled row. Wave 0 of every
-// workgroup walks the sum tree for its stratum with group_request / group_walk
-// (one dependent load per 10 levels; the first group sits under the root, so it
-// is requested together with the total and the uniform draw) and publishes the
-// slot through LDS. The workgroup's share of the row — granules of all
-// fields, numbered consecutively — is then copied with every load issued
-// before the first store, so a row costs one memory round trip, not one per
-// field. The row's first workgroup computes the importance weight while its
-// loads are in flight (the two powers in two lanes of one instruction stream).
-// Replaces PriorityReplayBufferSample
-// (mindspore_rl/core/priority_replay_buffer.py:70,92-106).
-// ---------------------------------------------------------------------------
-// kTree: sample through the sum tree (a.mode == kFromTree); otherwise a plain gather, compiled
-// without the descent and with ordinary row loads (sampling reads its rows non-temporally so
-// that they do not push the tree out of L2: 9.5 vs 10.1 us per config-3 call; a gather has no
-// tree to protect and is faster with ordinary loads: 6.1 vs 6.7 us for the same rows).
-template <bool kTree>
-__global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict__ sum, const float* __restrict__ uniforms,
-                                                         int depth, int split_arg, int64_t batch, uint64_t seed,
-                                                         uint64_t calls, SampleArgs a, IoTable t, SplitPlan plan) {
+#ifdef MRB_PROBE
+__device__ uint64_t g_probe[16384 * 16];
+#define MRB_TS(var) const uint64_t var = wall_clock64()
+#define MRB_TS_OUT(slot, var) do { if ((threadIdx.x & 63) == 0) g_probe[(blockIdx.x * 16 + (slot)) & (16384 * 16 - 1)] = (var); } while (0)
+#else
+#define MRB_TS(var) do { } while (0)
+#define MRB_TS_OUT(slot, var) do { } while (0)
+#endif
+
+constexpr int kCopyWaves = 4;
+constexpr int kCopyThreads = 64 * kCopyWaves;
+constexpr int kWideWG = 64 + kCopyThreads;  // the walker wave, then four copy waves
+constexpr int kMaxInFlight = 8;             // most granules a copy thread holds between its loads and its stores
+constexpr int kFastWide = 2;                // wide fields whose table entries are fetched unconditionally, in one round
+
+using g16 = __attribute__((address_space(1))) granule_t;
+
+constexpr int kNarrowInF = 2;  // narrow bytes a thread of the first copy wave holds beside its wide granules
+
+__device__ __forceinline__ uint32_t lane_u32(uint32_t x, int src_lane) {
+    return (uint32_t)__builtin_amdgcn_readlane((int)x, src_lane);
+}
+__device__ __forceinline__ uint64_t lane_u64(uint64_t x, int src_lane) {
+    return ((uint64_t)lane_u32((uint32_t)(x >> 32), src_lane) << 32) | lane_u32((uint32_t)x, src_lane);
+}
+
+// The narrow fields of a row, copied byte by byte by the first copy wave of the row's first
+// workgroup: lane l takes bytes l, l + 64, ... of the narrow fields' bytes, numbered consecutively
+// over the fields; the first kNarrowInF of them are loaded ahead of the wave's wide granules and
+// stored after them. Narrow fields are small (scalars such as action, reward, done); byte
+// granularity keeps their copy free of branches on a granule size.
+struct NarrowWork {
+    const gbyte* base[kNarrowInF];
+    gbyte* dst[kNarrowInF];
+    uint32_t rb[kNarrowInF];
+    uint32_t live;  // bit j: position j holds a byte
+    // the table entry of field `lane` (lanes 0 .. MRB_MAX_FIELDS - 1), kept for bytes past the first ones
+    uint64_t e_src, e_dst;
+    uint32_t e_rb, e_first;
+
+    // Lane q fetches table entry q, needed or not: the address depends on nothing loaded, so the
+    // table costs one round trip. Each lane then finds its bytes' fields from the entries held by
+    // the other lanes (the loops are wave-uniform).
+    __device__ __forceinline__ void prepare(const WidePlan& plan, int64_t k, uint32_t lane) {
+        const WideField e = plan.f[lane < MRB_MAX_FIELDS ? lane : 0];
+        e_src = (uint64_t)e.src;
+        e_dst = (uint64_t)e.dst + (uint64_t)k * e.rb;
+        e_rb = e.rb;
+        e_first = e.first;
+        live = 0;
+#pragma unroll
+        for (int j = 0; j < kNarrowInF; ++j) {
+            base[j] = nullptr;
+            dst[j] = nullptr;
+            rb[j] = 0;
+            if (lane + 64 * j < plan.narrow_items) live |= 1u << j;
+        }
+        for (int q = plan.nwide; q < plan.nwide + plan.nnarrow; ++q) {
+            const uint64_t src_q = lane_u64(e_src, q), dst_q = lane_u64(e_dst, q);
+            const uint32_t rb_q = lane_u32(e_rb, q), first_q = lane_u32(e_first, q);
+#pragma unroll
+            for (int j = 0; j < kNarrowInF; ++j) {
+                const uint32_t rel = ((live >> j) & 1u ? lane + 64 * j : 0u) - first_q;  // wraps for bytes of earlier fields
+                if (rel < rb_q) {
+                    base[j] = (const gbyte*)(src_q + rel);
+                    dst[j] = (gbyte*)(dst_q + rel);
+                    rb[j] = rb_q;
+                }
+            }
+        }
+    }
+    __device__ __forceinline__ void load(uint32_t slot, uint8_t (&held)[kNarrowInF]) const {
+#pragma unroll
+        for (int j = 0; j < kNarrowInF; ++j) held[j] = *(base[j] + (uint64_t)slot * rb[j]);
+    }
+    __device__ __forceinline__ void store(uint32_t slot, const uint8_t (&held)[kNarrowInF], const WidePlan& plan, uint32_t lane) const {
+#pragma unroll
+        for (int j = 0; j < kNarrowInF; ++j)
+            if (live & (1u << j)) *dst[j] = held[j];
+        if (plan.narrow_items > 64u * kNarrowInF) {  // wave-uniform; rows with many narrow bytes
+            for (int q = plan.nwide; q < plan.nwide + plan.nnarrow; ++q) {
+                const uint64_t src_q = lane_u64(e_src, q) + (uint64_t)slot * lane_u32(e_rb, q), dst_q = lane_u64(e_dst, q);
+                const uint32_t rb_q = lane_u32(e_rb, q), first_q = lane_u32(e_first, q);
+                // bytes of this field numbered 64 * kNarrowInF or more among the narrow bytes
+                uint32_t rel = (first_q >= 64u * kNarrowInF ? 0u : 64u * kNarrowInF - first_q) + lane;
+                for (; rel < rb_q; rel += 64) *((gbyte*)dst_q + rel) = *((const gbyte*)src_q + rel);
+            }
+        }
+    }
+};
+
+// Copy thread `tid` (0 .. kCopyThreads - 1) of workgroup `part` of row k: up to kInF wide granules.
+// A thread without a granule in some position re-reads the workgroup's first granule (a valid
+// address) and skips the store, so that the loads are unconditional and all in flight together.
+// kOneWide: the row has a single wide field (e.g. an image observation beside a few scalars); all
+// addresses are then a wave-uniform row base plus a 32-bit offset, which costs a tenth of the
+// general path's address arithmetic - work that would otherwise compete with the walker for
+// the SIMD's issue slots.
+template <int kInF, bool kOneWide>
+struct CopyWork {
+    const gbyte* base[kOneWide ? 1 : kInF];  // general: field storage + offset of the granule within a row
+    g16* dst[kOneWide ? 1 : kInF];
+    uint32_t rb[kOneWide ? 1 : kInF];
+    uint32_t off[kOneWide ? kInF : 1];       // one wide field: byte offset of the granule within a row
+    const uint8_t* src0;                     // one wide field: storage, destination row, row size (wave-uniform)
+    uint8_t* dst0;
+    uint32_t rb0;
+    uint32_t live;  // bit j: position j holds a granule of this workgroup
+
+    __device__ __forceinline__ void prepare(const WidePlan& plan, int64_t k, uint32_t part, uint32_t tid) {
+        const uint32_t lo = part * plan.share;
+        const uint32_t hi = min(plan.wide_items, lo + plan.share);
+        uint32_t it[kInF];
+        live = 0;
+#pragma unroll
+        for (int j = 0; j < kInF; ++j) {
+            it[j] = lo + j * kCopyThreads + tid;
+            if (it[j] < hi) live |= 1u << j;
+            else it[j] = lo;
+        }
+        if (lo >= hi) live = 0;
+        if (kOneWide) {
+            const WideField e = plan.f[0];
+            src0 = e.src;
+            rb0 = e.rb;
+            dst0 = e.dst + (uint64_t)k * e.rb;
+#pragma unroll
+            for (int j = 0; j < kInF; ++j) off[j] = it[j] << 4;
+            return;
+        }
+#pragma unroll
+        for (int j = 0; j < (kOneWide ? 1 : kInF); ++j) {
+            base[j] = nullptr;
+            dst[j] = nullptr;
+            rb[j] = 0;
+        }
+        auto take = [&](int q) {
+            const WideField e = plan.f[q];
+            const uint32_t units = q < plan.nwide ? e.rb >> 4 : 0u;
+            const gbyte* s = as_global(e.src);
+            gbyte* d = as_global(e.dst) + (uint64_t)k * e.rb;
+#pragma unroll
+            for (int j = 0; j < (kOneWide ? 1 : kInF); ++j) {
+                const uint32_t rel = it[j] - e.first;  // wraps for granules of earlier fields
+                if (rel < units) {
+                    base[j] = s + ((uint64_t)rel << 4);
+                    dst[j] = (g16*)(d + ((uint64_t)rel << 4));
+                    rb[j] = e.rb;
+                }
+            }
+        };
+        // the first entries unconditionally: their (wave-uniform) loads go out together at once
+#pragma unroll
+        for (int q = 0; q < kFastWide; ++q) take(q);
+        for (int q = kFastWide; q < plan.nwide; ++q) take(q);
+    }
+
+    // `narrow`: this thread also carries narrow bytes (first copy wave of the row's first workgroup)
+    __device__ __forceinline__ void run(uint32_t slot, const WidePlan& plan, bool narrow, const NarrowWork& nw, uint32_t lane) const {
+        uint8_t nheld[kNarrowInF];
+        granule_t held[kInF];
+        if (narrow) nw.load(slot, nheld);  // ahead of the wide loads in the memory pipeline
+        if (live) {
+            if (kOneWide) {
+                const gbyte* row = as_global(src0) + (uint64_t)slot * rb0;  // wave-uniform
+#pragma unroll
+                for (int j = 0; j < kInF; ++j) held[j] = __builtin_nontemporal_load((const g16*)(row + off[j]));
+            } else {
+#pragma unroll
+                for (int j = 0; j < kInF; ++j)
+                    held[j] = __builtin_nontemporal_load((const g16*)(base[j < (kOneWide ? 1 : kInF) ? j : 0] + (uint64_t)slot * rb[j < (kOneWide ? 1 : kInF) ? j : 0]));
+            }
+            // every load is issued before the first store (the compiler would otherwise move a load
+            // next to its conditional store, behind the other stores' waits)
+#pragma unroll
+            for (int j = 0; j < kInF; ++j) asm volatile("" : "+v"(held[j]));
+            MRB_TS(ts_loaded);
+            MRB_TS_OUT(threadIdx.x < 128 ? 6 : (threadIdx.x < 192 ? 11 : 15), ts_loaded);
+#pragma unroll
+            for (int j = 0; j < kInF; ++j) {
+                if (live & (1u << j)) {
+                    if (kOneWide) *(g16*)(as_global(dst0) + off[j]) = held[j];
+                    else *dst[j < (kOneWide ? 1 : kInF) ? j : 0] = held[j];
+                }
+            }
+        }
+        if (narrow) nw.store(slot, nheld, plan, lane);
+    }
+};
+
+// Replaces PriorityReplayBufferSample (mindspore_rl/core/priority_replay_buffer.py:70,92-106).
+// sum .. calls are the arguments the tree walk needs; they are preloaded into scalar registers.
+// `groups` packs the descent plan: bits 0-3 the number of node groups, then 5 bits per group
+// with the levels it takes. kTen: every group takes 10 levels (trees of 10, 20 or 30 levels); the
+// walk is then compiled for that size, which shortens it by a third.
+template <int kInF, bool kTen, bool kOneWide>
+__global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __restrict__ sum, const float* __restrict__ uniforms,
+                                                             int depth, uint32_t groups, int batch, uint32_t capacity,
+                                                             uint64_t seed, uint64_t calls, SampleTail tail, WidePlan plan) {
     __shared__ int64_t s_idx;
     __shared__ float s_picked, s_total, s_pmin;
-    // this workgroup's share of each field, filled by wave 1 while wave 0 walks the tree
-    __shared__ const gbyte* s_src[MRB_MAX_FIELDS];  // store_f + first granule's byte offset
-    __shared__ gbyte* s_dst[MRB_MAX_FIELDS];          // io_f + k * row_bytes + the same offset
-    __shared__ uint32_t s_wide[MRB_MAX_FIELDS];       // 16-byte granules of field f copied here
-    __shared__ uint32_t s_narrow[MRB_MAX_FIELDS];     // smaller granules (field rows not a multiple of 16 bytes)
-    __shared__ uint32_t s_vl[MRB_MAX_FIELDS];
-    __shared__ uint32_t s_rb[MRB_MAX_FIELDS];
-    // sum, uniforms, depth, split, batch, seed and calls repeat fields of `a` and `plan` as plain
-    // leading parameters: those are preloaded into scalar registers when the wave starts.
-    const uint32_t split = (uint32_t)split_arg;
-    const int64_t k = blockIdx.x / split;
-    const uint32_t part = blockIdx.x % split;
-    if (!kTree) {
-        // plain gather: the slot is given, drawn, or fixed; out-of-range slots are clamped and flagged
-        if (threadIdx.x == 0) {
-            int64_t slot = a.mode == kFromFixedSlot ? a.fixed_slot
-                           : a.mode == kFromIndices ? a.given[k]
-                                                    : rng_below(seed, calls, (uint64_t)k, a.count);
-            if (a.mode != kFromFixedSlot && (slot < 0 || slot >= a.count)) {
-                if (part == 0) atomicOr(a.err, MRB_DERR_INDEX);
-                slot = slot < 0 ? 0 : (a.count > 0 ? a.count - 1 : 0);
-            }
-            s_idx = slot;
-            s_picked = 0.0f;
-        }
-    } else if (depth == 21 || depth == 22) {
+    __shared__ float s_tot[4];
+    __shared__ SampleTail s_tail;
+    const int64_t k = blockIdx.x;      // row
+    const uint32_t part = blockIdx.y;  // which of the row's workgroups
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const bool walker = wave == 0;
+    const bool deep = depth == 21 || depth == 22;
+    const uint32_t ctid = threadIdx.x - 64;  // copy thread number
+    MRB_TS(ts_start);
+
+    if (deep) {
         // Trees of 21 and 22 levels would need three dependent node groups of <= 10 levels. Instead
-        // two (four) waves share the 2048 (4096) nodes at depth 11 (12), whose address is known: each
+        // two (four) copy waves share the 2048 (4096) nodes at depth 11 (12), whose address is known: each
         // reduces its 1024 nodes, the wave totals - the tree's nodes at depth 1 (2) - meet in LDS, every
         // wave takes the one (two) top steps of the walk from them, and the wave the walk enters goes on
         // through its ten levels and the ten below. Two dependent loads again, one barrier more.
-        __shared__ float s_tot[4];
         const int share = depth - 20;  // log2 of the waves sharing the top group
-        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        const int w = wave - 1;
+        const bool mine = !walker && w < (1 << share);
+        f32x4 r0, r1, r2, r3;
         f32x16 v = 0.0f;
         float total = 0.0f, u = 0.0f;
-        if (wave < (1 << share)) {
-            f32x4 r0, r1, r2, r3;
-            group_request(sum, (1u << share) + wave, kGroupMaxLevels, lane, r0, r1, r2, r3);
+        if (mine) {
+            group_request(sum, (1u << share) + w, kGroupMaxLevels, lane, r0, r1, r2, r3);
             total = sum[1];
             u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
             __builtin_amdgcn_sched_barrier(0);
             v = group_finish(kGroupMaxLevels, lane, r0, r1, r2, r3);
-            const float mine = group_total(v);
-            if (lane == 0) s_tot[wave] = mine;
+            const float t = group_total(v);
+            if (lane == 0) s_tot[w] = t;
         }
         __syncthreads();
-        if (wave < (1 << share)) {
+        if (mine) {
             float mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
             uint32_t q = 0;
             if (share == 2) {
@@ -339,178 +548,169 @@ __global__ __launch_bounds__(kWG) void k_per_sample_wide(const float* __restrict
                 mass -= left;
                 q += 1;
             }
-            if ((uint32_t)wave == q) {
+            if ((uint32_t)w == q) {
                 float picked;
                 uint32_t node = (((1u << share) + q) << kGroupMaxLevels) + group_walk(v, kGroupMaxLevels, lane, mass, picked);
-                f32x4 r0, r1, r2, r3;
                 group_request(sum, node, kGroupMaxLevels, lane, r0, r1, r2, r3);
                 __builtin_amdgcn_sched_barrier(0);
                 node = (node << kGroupMaxLevels) +
                        group_walk(group_finish(kGroupMaxLevels, lane, r0, r1, r2, r3), kGroupMaxLevels, lane, mass, picked);
                 if (lane == 0) {
-                    s_idx = (int64_t)node - a.leaves;
+                    s_idx = (int64_t)node - ((int64_t)1 << depth);
                     s_picked = picked;
                     s_total = total;
                 }
             }
         }
-    } else if (threadIdx.x < 64) {
-        const int lane = threadIdx.x;
-        const int ngroups = group_count(depth);
-        int g = ngroups ? group_levels(depth, ngroups, 0) : 0;
-        uint32_t node;
-        float picked, mass, total_w0;
+    } else if (walker) {
+        // the walk is a chain of dependent instructions: it goes ahead of the copy waves' address
+        // arithmetic on the SIMD they share
+        __builtin_amdgcn_s_setprio(3);
+        const int ngroups = (int)(groups & 15u);
+        uint32_t node = 1;
+        float picked, mass = 0.0f, total;
         if (depth >= 2) {
-            // The first group hangs under the root: its address is known, so it is requested
-            // together with the total and the draw; the scheduling barrier keeps every
-            // request ahead of the first use.
+            // The first group hangs under the root: its address is known, so it is requested at once,
+            // together with the total and the draw (read from a valid address also when the generator
+            // supplies the draw: no branch sits between the requests); the scheduling barrier keeps
+            // every request ahead of the first use and of the generator's arithmetic.
+            uint32_t packed = groups >> 4;
+            int g = kTen ? kGroupMaxLevels : (int)(packed & 31u);
             f32x4 r0, r1, r2, r3;
             group_request(sum, 1u, g, lane, r0, r1, r2, r3);
-            const float total = sum[1];
-            const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
+            total = sum[1];
+            const float u_given = *(uniforms ? uniforms + k : sum + 1);
             __builtin_amdgcn_sched_barrier(0);
-            total_w0 = total;
+            const float u = uniforms ? u_given : rng_uniform(seed, calls, (uint64_t)k);
             mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
             node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
+#pragma nounroll
             for (int i = 1; i < ngroups; ++i) {
-                g = group_levels(depth, ngroups, i);  // >= 5 once there are two groups
+                packed >>= 5;
+                g = kTen ? kGroupMaxLevels : (int)(packed & 31u);
                 group_request(sum, node, g, lane, r0, r1, r2, r3);
                 __builtin_amdgcn_sched_barrier(0);
                 node = (node << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
             }
         } else {
             // one or two leaves
-            const float total = sum[1];
-            total_w0 = total;
-            mass = stratum_mass(a, total, k);
+            total = sum[1];
+            const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
+            mass = (u + (float)k) * (total / (float)batch);
             picked = total;
-            node = (1u << g) + (g ? group_walk(group_load_tiny(sum, 1u, g, lane), g, lane, mass, picked) : 0u);
+            node = (1u << depth) + (depth ? group_walk(group_load_tiny(sum, 1u, depth, lane), depth, lane, mass, picked) : 0u);
         }
         if (lane == 0) {
-            s_idx = (int64_t)node - a.leaves;
+            s_idx = (int64_t)node - ((int64_t)1 << depth);
             s_picked = picked;
-            s_total = total_w0;
+            s_total = total;
+        }
+        __builtin_amdgcn_s_setprio(0);
+    }
+    // ---- copy waves, while the walker walks
+    CopyWork<kInF, kOneWide> work;
+    NarrowWork nw;
+    const bool narrow = wave == 1 && part == 0 && plan.narrow_items;
+    if (!walker) {
+        if (narrow) nw.prepare(plan, k, lane);
+        work.prepare(plan, k, part, ctid);
+        if (part == 0 && wave == 2) {
+            // what the walker needs after the barrier (member by member: a whole-struct copy would go
+            // through private memory)
+            if (lane == 0) {
+                s_tail.out_idx = tail.out_idx;
+                s_tail.out_w = tail.out_w;
+                s_tail.err = tail.err;
+                s_tail.size = tail.size;
+                s_tail.beta = tail.beta;
+            } else if (lane == 1) {
+                s_pmin = tail.mn[1];
+            }
         }
     }
-    if (kTree && threadIdx.x == 64 + MRB_MAX_FIELDS) s_pmin = a.mn[1];  // for the weight, fetched while wave 0 walks
-    // (separate from the chain above: in the gather modes every thread takes its first branch)
-    if (threadIdx.x >= 64 && threadIdx.x < 64 + MRB_MAX_FIELDS) {
-        const int f = threadIdx.x - 64;
-        uint32_t cnt = 0, vl = 0;
-        if (f < t.nfields) {
-            const uint32_t lo = part * plan.per[f];
-            vl = t.vec_log2[f];
-            const uint64_t off = (uint64_t)lo << vl;
-            cnt = lo < t.units[f] ? min(plan.per[f], t.units[f] - lo) : 0u;
-            s_vl[f] = vl;
-            s_rb[f] = t.row_bytes[f];
-            s_src[f] = as_global(t.store[f]) + off;
-            s_dst[f] = as_global(t.io[f]) + (uint64_t)k * t.row_bytes[f] + off;
+    MRB_TS(ts_at_barrier);
+    __syncthreads();
+    MRB_TS(ts_past_barrier);
+    const int64_t idx = s_idx;
+    if (!walker) {
+        // the descent can end on an unfilled leaf past the last row (flagged by the walker)
+        const uint32_t slot = (uint32_t)(idx < (int64_t)capacity ? idx : (int64_t)capacity - 1);
+        work.run((uint32_t)__builtin_amdgcn_readfirstlane((int)slot), plan, narrow, nw, lane);
+        MRB_TS(ts_end);
+        if (wave == 1) {
+            MRB_TS_OUT(0, ts_start);
+            MRB_TS_OUT(2, ts_at_barrier);
+            MRB_TS_OUT(4, ts_past_barrier);
+            MRB_TS_OUT(7, ts_end);
+        } else if (wave == 2) {
+            MRB_TS_OUT(9, ts_at_barrier);
+            MRB_TS_OUT(10, ts_past_barrier);
+            MRB_TS_OUT(12, ts_end);
         }
-        s_wide[f] = vl == 4 ? cnt : 0u;
-        s_narrow[f] = vl == 4 ? 0u : cnt;
+        return;
+    }
+    // ---- walker of the row's first workgroup: index and importance weight
+    if (part != 0) return;
+    // lane 0: (p / total * size)^-beta, lane 1: (pmin / total * size)^-beta
+    const float total = s_total;
+    const float fsize = (float)s_tail.size;
+    const float x = lane == 0 ? s_picked : s_pmin;
+    float r = 0.0f;
+    if (lane < 2) r = powf_det(x / total * fsize, -s_tail.beta);
+    const float max_w = __shfl(r, 1);
+    if (lane == 0) {
+        s_tail.out_idx[k] = idx;
+        s_tail.out_w[k] = r / max_w;
+        if (!(total > 0.0f) || total > 3.0e38f) atomicOr(s_tail.err, MRB_DERR_TOTAL);
+        if (idx >= s_tail.size) atomicOr(s_tail.err, MRB_DERR_UNFILLED);
+    }
+    MRB_TS(ts_wend);
+    MRB_TS_OUT(1, ts_start);
+    MRB_TS_OUT(3, ts_at_barrier);
+    MRB_TS_OUT(5, ts_past_barrier);
+    MRB_TS_OUT(8, ts_wend);
+}
+
+// Gather of wide rows: io_f[k] = store_f[slot_k], slot_k being `fixed_slot` (mode kFromFixedSlot, a
+// single-row read), given[k] (kFromIndices) or drawn by the counter-based generator uniformly in
+// [0, count) (kFromGenerator). Replaces P.BufferSample / P.BufferGetItem
+// (mindspore_rl/core/uniform_replay_buffer.py:83-89,128,139) for wide rows.
+constexpr int kFromIndices = 1, kFromGenerator = 2, kFromFixedSlot = 3;
+
+template <int kInF, bool kOneWide>
+__global__ __launch_bounds__(kWideWG) void k_rows_gather_wide(const int64_t* __restrict__ given, int mode,
+                                                              int64_t count, int64_t fixed_slot, uint64_t seed,
+                                                              uint64_t calls, int64_t* __restrict__ out_idx,
+                                                              uint32_t* __restrict__ err, WidePlan plan) {
+    __shared__ int64_t s_idx;
+    const int64_t k = blockIdx.x;      // row
+    const uint32_t part = blockIdx.y;  // which of the row's workgroups
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const bool walker = wave == 0;
+    const uint32_t ctid = threadIdx.x - 64;
+    CopyWork<kInF, kOneWide> work;
+    NarrowWork nw;
+    const bool narrow = wave == 1 && part == 0 && plan.narrow_items;
+    if (walker) {
+        if (lane == 0) {
+            // out-of-range slots are clamped and flagged (a fixed slot was range-checked by the host
+            // against the ring: it may lie above `count` after a reset)
+            int64_t slot = mode == kFromFixedSlot ? fixed_slot
+                           : mode == kFromIndices ? given[k]
+                                                  : rng_below(seed, calls, (uint64_t)k, count);
+            if (mode != kFromFixedSlot && (slot < 0 || slot >= count)) {
+                if (part == 0) atomicOr(err, MRB_DERR_INDEX);
+                slot = slot < 0 ? 0 : (count > 0 ? count - 1 : 0);
+            }
+            s_idx = slot;
+            if (part == 0 && out_idx) out_idx[k] = slot;
+        }
+    } else {
+        if (narrow) nw.prepare(plan, k, lane);
+        work.prepare(plan, k, part, ctid);
     }
     __syncthreads();
-    const int64_t idx = s_idx;
-    const uint64_t slot = (uint64_t)(idx < a.capacity ? idx : a.capacity - 1);
-    // This workgroup's granules, numbered consecutively over the fields: 16-byte ones
-    // ("wide") and the granules of fields whose rows are not multiples of 16 bytes ("narrow").
-    uint32_t wide_items = 0, narrow_items = 0;
-#pragma unroll
-    for (int f = 0; f < MRB_MAX_FIELDS; ++f) {
-        wide_items += s_wide[f];
-        narrow_items += s_narrow[f];
-    }
-    using g16 = __attribute__((address_space(1))) granule_t;
-    uint32_t wfirst = 0, nfirst = 0;
-    do {
-        // ---- addresses first. A thread without a granule in this pass re-reads granule 0
-        // (a valid address) and skips the store, so that the loads below are unconditional
-        // and can all be in flight together.
-        const g16* wsrc[kInFlight];
-        g16* wdst[kInFlight];
-        bool wlive[kInFlight];
-#pragma unroll
-        for (int j = 0; j < kInFlight; ++j) {
-            uint32_t it = wfirst + j * kWG + threadIdx.x;
-            wlive[j] = it < wide_items;
-            if (!wlive[j]) it = 0;
-            int f = 0;
-            if (wide_items) {
-                uint32_t cnt = s_wide[0];
-                while (it >= cnt) {
-                    it -= cnt;
-                    cnt = s_wide[++f];
-                }
-            }
-            const uint64_t off = (uint64_t)it << 4;
-            wsrc[j] = (const g16*)(s_src[f] + slot * s_rb[f] + off);
-            wdst[j] = (g16*)(s_dst[f] + off);
-        }
-        const gbyte* nsrc;
-        gbyte* ndst;
-        uint32_t nbytes;
-        bool nlive;
-        {
-            uint32_t it = nfirst + threadIdx.x;
-            nlive = it < narrow_items;
-            if (!nlive) it = 0;
-            int f = 0;
-            if (narrow_items) {
-                uint32_t cnt = s_narrow[0];
-                while (it >= cnt) {
-                    it -= cnt;
-                    cnt = s_narrow[++f];
-                }
-            }
-            const uint32_t vl = s_vl[f];
-            const uint64_t off = (uint64_t)it << vl;
-            nsrc = s_src[f] + slot * s_rb[f] + off;
-            ndst = s_dst[f] + off;
-            nbytes = 1u << vl;
-        }
-        // ---- loads
-        granule_t held[kInFlight];
-        uint8_t nb[8];
-        if (wide_items) {
-#pragma unroll
-            for (int j = 0; j < kInFlight; ++j) held[j] = kTree ? __builtin_nontemporal_load(wsrc[j]) : *wsrc[j];
-        }
-        if (narrow_items) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) nb[i] = nsrc[(uint32_t)i < nbytes ? i : 0];
-        }
-        // ---- importance weight, computed while the loads are in flight
-        if (!kTree) {
-            if (wfirst == 0 && part == 0 && threadIdx.x == 0 && a.out_idx) a.out_idx[k] = idx;
-        } else if (wfirst == 0 && part == 0 && threadIdx.x < 2) {
-            // lane 0: (p / total * size)^-beta, lane 1: (pmin / total * size)^-beta
-            const float total = s_total;
-            const float x = threadIdx.x == 0 ? s_picked : s_pmin;
-            const float r = powf_det(x / total * (float)a.size, -a.beta);
-            const float max_w = __shfl(r, 1);
-            if (threadIdx.x == 0) {
-                a.out_idx[k] = idx;
-                a.out_w[k] = r / max_w;
-                sample_flags(a, total, idx);
-            }
-        }
-        // ---- stores: plain (cached) ones, unlike the row loads. The gathered batch is what the
-        // caller reads next, and on the measured 28 KB-row workload cached stores are faster by
-        // 0.6 us per launch than non-temporal ones.
-        if (wide_items) {
-#pragma unroll
-            for (int j = 0; j < kInFlight; ++j)
-                if (wlive[j]) *wdst[j] = held[j];
-        }
-        if (narrow_items && nlive) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if ((uint32_t)i < nbytes) ndst[i] = nb[i];
-        }
-        wfirst += kWG * kInFlight;
-        nfirst += kWG;
-    } while (wfirst < wide_items || nfirst < narrow_items);
+    if (!walker) work.run((uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)s_idx), plan, narrow, nw, lane);
 }
 
 // ---------------------------------------------------------------------------

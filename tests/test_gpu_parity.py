@@ -26,9 +26,6 @@ def mrb():
     ns = NS()
     ns.lib, ns.PER, ns.URB, ns.RES = _lib, PriorityReplayBuffer, UniformReplayBuffer, ReservoirReplayBuffer
     yield ns
-    _lib.set_option("sample_path", 0)
-    _lib.set_option("row_split", 0)
-    _lib.set_option("lds_levels", 0)
 
 
 # ------------------------------------------------------------------ uniform
@@ -371,10 +368,10 @@ def test_per_random_ops_bit_exact(mrb, orc, cap, path):
     duplicates and samples; after every step both trees, indices, rows, size, head and
     running max are compared. Capacities cover tree depths 0..17, i.e. the top kernel
     alone (<= 4096 leaves) and one rebuild round."""
-    mrb.lib.set_option("sample_path", path)
     rng = np.random.default_rng(cap + path)
     batch = 32
     g, c = make_pair(mrb, orc, 0.6, cap, batch)
+    g.set_option("sample_path", path)
     serial, exact_w = 0, 0
     for step in range(12):
         n = int(rng.integers(1, min(2 * cap + 3, 3000)))
@@ -489,9 +486,10 @@ def test_randomised_differential(mrb, orc, seed):
     shapes, dtypes = [p[0] for p in picks], [p[1] for p in picks]
     alpha = float(rng.choice([0.0, 0.3, 0.6, 1.0]))
     batch = int(rng.choice([1, 5, 64, 300]))
-    mrb.lib.set_option("sample_path", int(rng.integers(0, 3)))
-    mrb.lib.set_option("row_split", int(rng.choice([0, 0, 1, 3])))
+    path, split = int(rng.integers(0, 3)), int(rng.choice([0, 0, 1, 3]))
     g, c = make_pair(mrb, orc, alpha, cap, batch, seed=seed + 1, shapes=shapes, dtypes=dtypes)
+    g.set_option("sample_path", path)
+    g.set_option("row_split", split)
     for step in range(25):
         op = rng.integers(0, 4) if c.size else 0
         if op == 0:
@@ -522,8 +520,6 @@ def test_randomised_differential(mrb, orc, seed):
         assert g.size() == c.size and np.float32(g.max_priority) == np.float32(c.max_priority)
     for f, view in enumerate(g.storage()):
         assert np.array_equal(t2n(view).view(np.uint8), c.field(f).view(np.uint8)), f
-    mrb.lib.set_option("sample_path", 0)
-    mrb.lib.set_option("row_split", 0)
     g.check()
     g.destroy()
 
@@ -537,9 +533,9 @@ def test_sixteen_fields_of_odd_sizes(mrb, orc, path):
     shapes[7], dtypes[7] = (4,), np.float32   # 16 bytes
     shapes[9], dtypes[9] = (3,), np.int64     # 24 bytes
     rng = np.random.default_rng(16)
-    mrb.lib.set_option("sample_path", path)
     cap, batch = 300, 40
     g, c = make_pair(mrb, orc, 0.7, cap, batch, seed=2, shapes=shapes, dtypes=dtypes)
+    g.set_option("sample_path", path)
     u = mrb.URB(batch, cap, shapes, torch_types(dtypes), seed=8)
     cu = orc.OracleUniform(cap, shapes, dtypes, seed=8)
     r = mrb.RES(cap, batch, shapes, torch_types(dtypes), seed1=8)
@@ -564,7 +560,6 @@ def test_sixteen_fields_of_odd_sizes(mrb, orc, path):
             assert np.array_equal(t2n(uf[f]).view(np.uint8), cf[f].view(np.uint8)), (step, f)
             assert np.array_equal(t2n(rf[f]).view(np.uint8), kf[f].view(np.uint8)), (step, f)
             assert np.array_equal(t2n(u.buffer[f]).view(np.uint8), cu.field(f).view(np.uint8)), (step, f)
-    mrb.lib.set_option("sample_path", 0)
     for b in (g, u, r):
         b.destroy()
 
@@ -573,11 +568,11 @@ def test_sixteen_fields_of_odd_sizes(mrb, orc, path):
 def test_out_of_domain_inputs_are_clamped_and_flagged(mrb, orc, path):
     """Draws outside [0, 1), NaN draws, and slots far outside the buffer: the oracle defines what comes
     back (the descent has no clamp), the row copies stay inside the storage, and flags are raised."""
-    mrb.lib.set_option("sample_path", path)
     shapes, dtypes = [(600,), (1,)], [np.float32, np.int32]  # one wide and one narrow field
     rng = np.random.default_rng(4)
     cap = 1500
     g, c = make_pair(mrb, orc, 0.6, cap, 8, seed=5, shapes=shapes, dtypes=dtypes)
+    g.set_option("sample_path", path)
     rows = random_rows(rng, cap, shapes, dtypes)
     g.insert(*to_dev(rows)), c.push(rows, cap)
     u = np.array([0.0, 0.999, 1.0, 7.5, -3.0, np.nan, np.inf, 1e30], np.float32)
@@ -590,7 +585,6 @@ def test_out_of_domain_inputs_are_clamped_and_flagged(mrb, orc, path):
     assert np.array_equal(t2n(got[0]), c.field(0)[want])
     with pytest.raises(IndexError):
         g.check()
-    mrb.lib.set_option("sample_path", 0)
     g.destroy()
 
 
@@ -652,10 +646,10 @@ def test_config4_apex_high_churn(mrb, orc):
         c.update(idx, up)
         u = rng.random(batch).astype(np.float32)
         for path in (1, 2):
-            mrb.lib.set_option("sample_path", path)
+            g.set_option("sample_path", path)
             assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(batch, 0.5, u),
                                 "step %d path %d" % (step, path))
-        mrb.lib.set_option("sample_path", 0)
+        g.set_option("sample_path", 0)
     assert_tree_equal(g, c, "config 4")
     assert g.check() == 0
     g.destroy()
@@ -680,11 +674,11 @@ def test_config5_tree_descent_stress(mrb, orc):
         c.update(idx, up)
         u = rng.random(batch).astype(np.float32)
         for path in (2, 1):
-            mrb.lib.set_option("sample_path", path)
+            g.set_option("sample_path", path)
             out = g.sample(0.7, uniforms=torch.from_numpy(u).cuda())
             assert_sample_equal(out, c.sample(batch, 0.7, u), "step %d path %d" % (step, path))
             assert np.array_equal(t2n(out[2])[:, 0], t2n(out[0]))  # row k holds its own slot number
-        mrb.lib.set_option("sample_path", 0)
+        g.set_option("sample_path", 0)
     assert_tree_equal(g, c, "config 5")
     assert g.check() == 0
     g.destroy()

@@ -37,9 +37,7 @@ def test_status_codes_without_a_device():
     assert L.mrb_urb_state(123456, None, None) == _lib.MRB_EHANDLE
     assert b"123456" in L.mrb_last_error()
     assert L.mrb_per_destroy(42) == _lib.MRB_EHANDLE
-    assert L.mrb_set_option(b"no_such_option", 1) == _lib.MRB_EINVAL
-    assert L.mrb_set_option(b"row_split", 1000) == _lib.MRB_EINVAL
-    assert L.mrb_set_option(b"row_split", 0) == _lib.MRB_OK
+    assert L.mrb_set_option(42, b"row_split", 0) == _lib.MRB_EHANDLE  # options belong to a buffer
     h = C.c_int64(0)
     fb = (C.c_int64 * 1)(4)
     assert L.mrb_urb_create(0, 1, fb, C.byref(h)) == _lib.MRB_EINVAL
@@ -101,12 +99,13 @@ def test_kernels_use_no_scratch_memory(tmp_path):
         kernels[name] = (int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
-    assert len(kernels) == 14, sorted(kernels)
+    assert sum("k_per_sample_wide" in k for k in kernels) == 8 and sum("k_rows_gather_wide" in k for k in kernels) == 4
+    assert len(kernels) == 24, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)
-        if "k_per_sample_wide" in name:
-            assert lds <= 1024, (name, lds)
+        if "k_per_sample_wide" in name or "k_rows_gather_wide" in name:
+            assert lds <= 256, (name, lds)  # a private array turned into LDS would show here
         if "k_tree_update" in name:
             assert lds == 4096, (name, lds)
 
