@@ -135,6 +135,14 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float *uniforms, 
  * duplicates), every ancestor of a touched leaf recomputed from its final
  * children; max priority = max(old, all priorities[j]^alpha). */
 int mrb_per_update(int64_t h, const int64_t *indices, const float *priorities, int64_t n, void *stream);
+/* mrb_per_update for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments, same result
+ * bit for bit; the scratch that mrb_per_update keeps per buffer (p^alpha of the call's entries) lives
+ * here in a static device array of the library, 1 MiB per GPU, so n is limited to 262,144 entries
+ * (larger n: MRB_EINVAL). The call allocates and frees nothing. All buffers on one GPU share that
+ * array: calls of this function that may run at the same time on one GPU (different streams) race;
+ * calls ordered on one stream do not. The buffer must live on the current device. */
+int mrb_per_update_noalloc(int64_t h, const int64_t *indices, const float *priorities, int64_t n, void *stream);
 /* Rows at the given physical slots (device int64[n], each in [0, size)), gathered like mrb_urb_gather:
  * dst_fields[i][k] = storage_i[indices[k]]. No counterpart among the reference's primitives; it serves
  * transitions that store a slot number instead of a copy of the next observation (a frame-shared

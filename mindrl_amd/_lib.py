@@ -39,6 +39,7 @@ SIGNATURES = {
     "mrb_per_sample": [_i64, _i64, _f32, _vp, _vp, _vp, _pvp, _vp],
     "mrb_per_gather": [_i64, _vp, _i64, _pvp, _vp],
     "mrb_per_update": [_i64, _vp, _vp, _i64, _vp],
+    "mrb_per_update_noalloc": [_i64, _vp, _vp, _i64, _vp],
     "mrb_per_export_tree": [_i64, _vp, _vp, _pi64, _vp],
     "mrb_per_state": [_i64, _pi64, _pi64, C.POINTER(C.c_float), _vp],
     "mrb_per_check": [_i64, C.POINTER(C.c_uint32), _vp],

@@ -11,6 +11,7 @@
 #include <memory>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 #include "mrb_kernels.h"
 
@@ -249,6 +250,37 @@ int gather_rows(const RowStore& r, const int64_t* indices, int64_t fixed_slot, i
     return MRB_OK;
 }
 
+// ---- the allocation-free entry point's scratch (mrb_per_update_noalloc) -------------------------
+// Device memory that exists from the moment the library is loaded: callers that must not allocate
+// (HIP graph capture, serving loops, harnesses that forbid hipMalloc) get the update_priorities
+// scratch from here. Every device holds its own copy at its own address; `scratch` itself is only
+// the host-side name of the symbol and is never passed to a kernel.
+constexpr int64_t kNoAllocMaxEntries = 1 << 18;  // 1 MiB per device
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+}  // namespace
+
+static __device__ __align__(256) float scratch[1 << 18];
+
+namespace {
+
+// Address of the current device's copy of `scratch`, looked up once per device.
+int static_scratch(float** out) {
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(MRB_EINVAL, "device %d outside [0, %d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        float* p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MRB_OK;
+}
+
 struct Urb {
     RowStore rows;
     int64_t count = 0, head = 0;
@@ -291,8 +323,11 @@ struct Per {
     int s_g0 = 0, s_rounds = 0, s_top = 0;
     int s_lo[kMaxRounds] = {}, s_g[kMaxRounds] = {};
     uint32_t* s_dirty[kMaxRounds] = {};
-    float* powered = nullptr;  // scratch of the last update_priorities call, grown on demand
+    // scratch of update_priorities (p^alpha of the call's entries): sized at create; a call with more
+    // entries gets a larger array and the old one is kept until destroy (work may still be queued on it)
+    float* powered = nullptr;
     int64_t powered_cap = 0;
+    std::vector<float*> retired;
     uint32_t* err = nullptr;
     uint32_t* dirty[kMaxRounds] = {};
     int nrounds = 0;
@@ -301,6 +336,7 @@ struct Per {
     int top_depth = 0;
     uint64_t epoch = 0;
     uint64_t seed = 0, calls = 0;
+    int device = 0;           // the HIP device the buffer lives on
     int64_t sample_path = 0;  // option "sample_path": 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
     int64_t lds_levels = 0;   // option "lds_levels": tree levels staged in LDS by the LDS-top kernel (0 = auto)
     ~Per() {
@@ -309,6 +345,7 @@ struct Per {
         if (stamp) (void)hipFree(stamp);
         if (maxp) (void)hipFree(maxp);
         if (powered) (void)hipFree(powered);
+        for (auto* d : retired) (void)hipFree(d);
         for (auto* d : s_dirty)
             if (d) (void)hipFree(d);
         if (err) (void)hipFree(err);
@@ -404,17 +441,24 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
     return MRB_OK;
 }
 
+// Zero-fills `bytes` (a multiple of 4) of device memory with a kernel.
+void fill_zero(void* p, size_t bytes, hipStream_t s) {
+    const uint64_t n = bytes / sizeof(float);
+    hipLaunchKernelGGL(k_fill_f32, dim3(grid_for(n)), dim3(kWG), 0, s, static_cast<float*>(p), 0.0f, n);
+}
+
 // Starts a new tree-update epoch. Epochs tag stamps and dirty words so that
 // neither needs clearing between calls; when the 32-bit tag would wrap, both
 // are cleared once.
 int next_epoch(Per& b, hipStream_t s) {
     b.epoch += 1;
     if ((uint32_t)b.epoch == 0) {
-        HIP_TRY(hipMemsetAsync(b.stamp, 0, sizeof(unsigned long long) * (size_t)b.leaves, s));
-        for (int r = 0; r < b.nrounds; ++r)
-            HIP_TRY(hipMemsetAsync(b.dirty[r], 0, sizeof(uint32_t) * ((size_t)1 << (b.lo[r] - b.g[r])), s));
+        // cleared by a fill kernel, not a memset node: a caller may be capturing this stream (0.0f is all-zero bits)
+        fill_zero(b.stamp, sizeof(unsigned long long) * (size_t)b.leaves, s);
+        for (int r = 0; r < b.nrounds; ++r) fill_zero(b.dirty[r], sizeof(uint32_t) * ((size_t)1 << (b.lo[r] - b.g[r])), s);
         for (int r = 0; r < b.s_rounds; ++r)
-            HIP_TRY(hipMemsetAsync(b.s_dirty[r], 0, sizeof(uint32_t) * ((size_t)1 << (b.s_lo[r] - b.s_g[r])), s));
+            fill_zero(b.s_dirty[r], sizeof(uint32_t) * ((size_t)1 << (b.s_lo[r] - b.s_g[r])), s);
+        LAUNCH_CHECK("k_fill_f32");
         b.epoch += 1;
     }
     return MRB_OK;
@@ -441,6 +485,52 @@ UpdateArgs update_args(Per& b) {
     a.top_depth = b.top_depth;
     return a;
 }
+
+// update_priorities on buffer b with `powered` (device f32[n]) as the scratch that holds the entries'
+// p^alpha between the stamp pass and the leaf writes. Allocates nothing.
+int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t n, float* powered, hipStream_t s) {
+    Per* b = &pb;
+    int rc = next_epoch(*b, s);
+    if (rc) return rc;
+    UpdateArgs a = update_args(*b);
+    a.powered = powered;
+    a.indices = indices;
+    a.priorities = priorities;
+    a.n = n;
+    // Few entries on a very large tree: rebuild the lowest levels per entry, not per tile.
+    const bool sparse = b->s_g0 > 0 && n <= (b->leaves >> 8);
+    if (sparse) {
+        a.sparse_g0 = b->s_g0;
+        a.nrounds = b->s_rounds;
+        a.top_depth = b->s_top;
+        for (int r = 0; r < kMaxRounds; ++r) {
+            a.dirty[r] = b->s_dirty[r];
+            a.lo[r] = b->s_lo[r];
+            a.g[r] = b->s_g[r];
+        }
+    }
+    // A small call on a tree of at least four leaves needs no stamp pass: the leaf-level waves scan the
+    // entries themselves (one launch less).
+    if (!sparse && n <= 1024 && b->depth >= 2) {
+        a.inline_election = 1;
+        return tree_rebuild(*b, a, s);
+    }
+    hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
+    LAUNCH_CHECK("k_update_stamp");
+    if (!sparse) return tree_rebuild(*b, a, s);
+    hipLaunchKernelGGL(k_tree_sparse, dim3(grid_exact((uint64_t)n << (b->s_g0 - 2))), dim3(kWG), 0, s, a);
+    LAUNCH_CHECK("k_tree_sparse");
+    const PutArgs none{};
+    for (int r = 0; r < b->s_rounds; ++r) {
+        const uint32_t tiles = (1u << b->s_lo[r]) / kBlockNodes;
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r, 0u, none);
+        LAUNCH_CHECK("k_tree_update");
+    }
+    hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a, none);
+    LAUNCH_CHECK("k_tree_top");
+    return MRB_OK;
+}
+
 
 }  // namespace
 
@@ -662,6 +752,13 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->stamp), (size_t)b->leaves * sizeof(unsigned long long)));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->maxp), 16));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16));
+    // update_priorities scratch, sized once: a call rarely names more entries than there are rows
+    b->powered_cap = capacity < 4096 ? 4096 : (capacity > (1ll << 20) ? (1ll << 20) : capacity);
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->powered), (size_t)b->powered_cap * sizeof(float)));
+    HIP_TRY(hipGetDevice(&b->device));
+    float* unused = nullptr;
+    rc = static_scratch(&unused);  // set-up of the allocation-free entry point for this device
+    if (rc) return rc;
     HIP_TRY(hipMemset(b->sum, 0, nodes * sizeof(float)));
     HIP_TRY(hipMemset(b->stamp, 0, (size_t)b->leaves * sizeof(unsigned long long)));
     HIP_TRY(hipMemset(b->err, 0, 16));
@@ -747,53 +844,32 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     if (!indices || !priorities) return fail(MRB_EINVAL, "indices or priorities is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (n > b->powered_cap) {
-        // hipFree waits for the device, so no kernel still reads the old scratch
-        if (b->powered) HIP_TRY(hipFree(b->powered));
-        b->powered = nullptr;
-        b->powered_cap = 0;
-        const int64_t want = n > 4096 ? n : 4096;
-        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->powered), (size_t)want * sizeof(float)));
+        // more entries than any call so far (and than the capacity): a larger array, at least twice the
+        // old one; the old one stays allocated, kernels already queued may still use it
+        const int64_t want = n > 2 * b->powered_cap ? n : 2 * b->powered_cap;
+        float* bigger = nullptr;
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&bigger), (size_t)want * sizeof(float)));
+        if (b->powered) b->retired.push_back(b->powered);
+        b->powered = bigger;
         b->powered_cap = want;
     }
-    int rc = next_epoch(*b, s);
+    return per_update(*b, indices, priorities, n, b->powered, s);
+}
+
+int mrb_per_update_noalloc(int64_t h, const int64_t* indices, const float* priorities, int64_t n, void* stream) {
+    GET_PER(b, h);
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (n > kNoAllocMaxEntries)
+        return fail(MRB_EINVAL, "n %lld exceeds the %lld entries the static scratch holds; use mrb_per_update",
+                    (long long)n, (long long)kNoAllocMaxEntries);
+    if (!indices || !priorities) return fail(MRB_EINVAL, "indices or priorities is NULL");
+    float* powered = nullptr;
+    int rc = static_scratch(&powered);
     if (rc) return rc;
-    UpdateArgs a = update_args(*b);
-    a.powered = b->powered;
-    a.indices = indices;
-    a.priorities = priorities;
-    a.n = n;
-    // Few entries on a very large tree: rebuild the lowest levels per entry, not per tile.
-    const bool sparse = b->s_g0 > 0 && n <= (b->leaves >> 8);
-    if (sparse) {
-        a.sparse_g0 = b->s_g0;
-        a.nrounds = b->s_rounds;
-        a.top_depth = b->s_top;
-        for (int r = 0; r < kMaxRounds; ++r) {
-            a.dirty[r] = b->s_dirty[r];
-            a.lo[r] = b->s_lo[r];
-            a.g[r] = b->s_g[r];
-        }
-    }
-    // A small call on a tree of at least four leaves needs no stamp pass: the leaf-level waves scan the
-    // entries themselves (one launch less).
-    if (!sparse && n <= 1024 && b->depth >= 2) {
-        a.inline_election = 1;
-        return tree_rebuild(*b, a, s);
-    }
-    hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, a);
-    LAUNCH_CHECK("k_update_stamp");
-    if (!sparse) return tree_rebuild(*b, a, s);
-    hipLaunchKernelGGL(k_tree_sparse, dim3(grid_exact((uint64_t)n << (b->s_g0 - 2))), dim3(kWG), 0, s, a);
-    LAUNCH_CHECK("k_tree_sparse");
-    const PutArgs none{};
-    for (int r = 0; r < b->s_rounds; ++r) {
-        const uint32_t tiles = (1u << b->s_lo[r]) / kBlockNodes;
-        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r, 0u, none);
-        LAUNCH_CHECK("k_tree_update");
-    }
-    hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a, none);
-    LAUNCH_CHECK("k_tree_top");
-    return MRB_OK;
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev != b->device) return fail(MRB_ESTATE, "the buffer lives on device %d, the current device is %d", b->device, dev);
+    return per_update(*b, indices, priorities, n, powered, static_cast<hipStream_t>(stream));
 }
 
 int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, int64_t* out_indices,
@@ -1046,7 +1122,7 @@ int mrb_per_load_leaves(int64_t h, const float* leaves, int64_t n, float max_pri
     if (!(max_priority >= 0.0f) || max_priority > 3.0e38f) return fail(MRB_EINVAL, "max_priority %g is not a priority", (double)max_priority);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t nodes = 2 * (size_t)b->leaves;
-    HIP_TRY(hipMemsetAsync(b->sum, 0, nodes * sizeof(float), s));
+    fill_zero(b->sum, nodes * sizeof(float), s);
     hipLaunchKernelGGL(k_fill_f32, dim3(grid_for(nodes)), dim3(kWG), 0, s, b->mn, FLT_MAX, (uint64_t)nodes);
     LAUNCH_CHECK("k_fill_f32");
     HIP_TRY(hipMemcpyAsync(b->maxp, &max_priority, sizeof(float), hipMemcpyHostToDevice, s));
