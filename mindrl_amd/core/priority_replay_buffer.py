@@ -180,17 +180,22 @@ class PriorityReplayBuffer:
                 "fields": save_fields(self.storage(), size)}
 
     def load_state_dict(self, state):
-        """Restores a state_dict() taken from a buffer of the same capacity, alpha, shapes and types."""
+        """Restores a state_dict() taken from a buffer of the same capacity, alpha, shapes and types.
+        Nothing of this buffer changes unless the whole state fits."""
         if state.get("kind") != "priority" or state["capacity"] != self._capacity:
             raise ValueError("state does not belong to a PriorityReplayBuffer of capacity %d" % self._capacity)
-        load_fields(self.storage(), state["fields"], self._layout)
+        if np.float32(state["alpha"]) != np.float32(self._alpha):
+            # the saved leaves are priorities ** alpha: they mean something else under another exponent
+            raise ValueError("state was saved with alpha %r, this buffer has alpha %r" % (state["alpha"], self._alpha))
         leaves = torch.as_tensor(state["leaves"]).to(device=self._dev, dtype=torch.float32).contiguous()
-        if leaves.numel() != state["size"]:
-            raise ValueError("state holds %d leaves for %d rows" % (leaves.numel(), state["size"]))
-        set_counters(_lib.lib().mrb_per_set_counters, self._h,
-                     [state["size"], state["pushes"], state["seed"], state["calls"]])
+        size, pushes = int(state["size"]), int(state["pushes"])
+        if leaves.numel() != size or size != min(pushes, self._capacity) or pushes < 0:
+            raise ValueError("state holds %d leaves for size %d after %d pushes" % (leaves.numel(), size, pushes))
+        load_fields(self.storage(), state["fields"], self._layout)
+        # the tree first, the counters last: a failure on the way leaves size and pushes as they were
         _lib.check(_lib.lib().mrb_per_load_leaves(self._h, leaves.data_ptr() if leaves.numel() else None,
                                                   leaves.numel(), float(state["max_priority"]), stream_ptr()))
+        set_counters(_lib.lib().mrb_per_set_counters, self._h, [size, pushes, state["seed"], state["calls"]])
         torch.cuda.current_stream().synchronize()
 
     def check(self):

@@ -577,6 +577,7 @@ int mrb_urb_create(int64_t capacity, int nfields, const int64_t* field_bytes, in
     if (rc) return rc;
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16));
     HIP_TRY(hipMemset(b->err, 0, 16));
+    HIP_TRY(hipDeviceSynchronize());  // the zero-fills ran on the null stream; the caller's stream may not wait for it
     std::lock_guard<std::mutex> lk(g_mu);
     *out_handle = g_next++;
     g_urb[*out_handle] = b;
@@ -984,6 +985,7 @@ int mrb_res_create(int64_t capacity, int nfields, const int64_t* field_bytes, ui
     HIP_TRY(hipMemset(b->stamp, 0, (size_t)capacity * sizeof(unsigned long long)));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16));
     HIP_TRY(hipMemset(b->err, 0, 16));
+    HIP_TRY(hipDeviceSynchronize());  // as in mrb_urb_create
     std::lock_guard<std::mutex> lk(g_mu);
     *out_handle = g_next++;
     g_res[*out_handle] = b;

@@ -19,7 +19,7 @@ namespace mrb {
 // importance-sampling weights (PriorityReplayBufferSample, :92-106).
 __device__ __forceinline__ float powf_det(float x, float a) {
     if (a == 0.0f) return 1.0f;
-    if (x == 0.0f) return 0.0f;
+    if (x == 0.0f) return a < 0.0f ? __builtin_inff() : 0.0f;  // as pow(): 0^-b is +inf
     if (a == 1.0f) return x;
     if (x == 1.0f) return 1.0f;
     unsigned long long bits = (unsigned long long)__double_as_longlong((double)x);

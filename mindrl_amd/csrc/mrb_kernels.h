@@ -1222,6 +1222,9 @@ __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) 
     }
     top_rebuild(a, a.top_depth, &s_win[0][0]);
     if (a.fold_max) {
+        // every wave has finished reading the running max (a fresh slot with an invalid priority takes
+        // its value from before the call) before any wave raises it
+        __syncthreads();
         // The rounds before this launch read the running max as it was before the call (fresh slots
         // with an invalid priority take it), so it is raised only now.
         float q = 0.0f;

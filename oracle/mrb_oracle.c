@@ -68,7 +68,7 @@ static uint64_t orc_double_as_u64(double d) {
 
 float orc_powf(float x, float a) {
     if (a == 0.0f) return 1.0f;
-    if (x == 0.0f) return 0.0f;
+    if (x == 0.0f) return a < 0.0f ? INFINITY : 0.0f; /* as pow(): 0^-b is +inf, so a zero minimum priority gives weights 0, not inf */
     if (a == 1.0f) return x;
     if (x == 1.0f) return 1.0f;
     uint64_t bits = orc_double_as_u64((double)x);
@@ -265,6 +265,16 @@ void orc_urb_reset(orc_urb *b) { b->count = 0; } /* uniform_replay_buffer.py:149
 int64_t orc_urb_count(const orc_urb *b) { return b->count; }
 int64_t orc_urb_head(const orc_urb *b) { return b->head; }
 const void *orc_urb_field(const orc_urb *b, int i) { return b->rows.data[i]; }
+/* Checkpoint counterpart (the reference persists no buffers; the state is what continuing
+ * identically needs): {count, head, seed, calls}. Row storage is reached through orc_urb_field. */
+void orc_urb_get_state(const orc_urb *b, int64_t *out4) {
+    out4[0] = b->count, out4[1] = b->head, out4[2] = (int64_t)b->seed, out4[3] = (int64_t)b->calls;
+}
+int orc_urb_set_state(orc_urb *b, const int64_t *in4) {
+    if (in4[0] < 0 || in4[0] > b->rows.capacity || in4[1] < 0 || in4[1] >= b->rows.capacity) return 1;
+    b->count = in4[0], b->head = in4[1], b->seed = (uint64_t)in4[2], b->calls = (uint64_t)in4[3];
+    return 0;
+}
 
 /* ------------------------------------------------------------------------
  * Discounted return (mindspore_rl/utils/discounted_return.py:84-92, the
@@ -350,6 +360,16 @@ int orc_res_sample(orc_res *b, int64_t n, int64_t *out_indices, void *const *dst
 int64_t orc_res_size(const orc_res *b) { return b->size; }
 int64_t orc_res_total(const orc_res *b) { return b->total; }
 const void *orc_res_field(const orc_res *b, int i) { return b->rows.data[i]; }
+/* {size, total, seed, calls} */
+void orc_res_get_state(const orc_res *b, int64_t *out4) {
+    out4[0] = b->size, out4[1] = b->total, out4[2] = (int64_t)b->seed, out4[3] = (int64_t)b->calls;
+}
+int orc_res_set_state(orc_res *b, const int64_t *in4) {
+    int64_t want = in4[1] < b->rows.capacity ? in4[1] : b->rows.capacity;
+    if (in4[1] < 0 || in4[0] != want) return 1;
+    b->size = in4[0], b->total = in4[1], b->seed = (uint64_t)in4[2], b->calls = (uint64_t)in4[3];
+    return 0;
+}
 
 /* ------------------------------------------------------------------------
  * Prioritized buffer (priority_replay_buffer.py:60-138): FIFO rows + a sum
@@ -499,3 +519,27 @@ int64_t orc_per_size(const orc_per *b) { return b->size; }
 int64_t orc_per_head(const orc_per *b) { return b->pushes % b->rows.capacity; }
 float orc_per_max_priority(const orc_per *b) { return b->max_priority; }
 const void *orc_per_field(const orc_per *b, int i) { return b->rows.data[i]; }
+/* {size, pushes, seed, calls} */
+void orc_per_get_state(const orc_per *b, int64_t *out4) {
+    out4[0] = b->size, out4[1] = b->pushes, out4[2] = (int64_t)b->seed, out4[3] = (int64_t)b->calls;
+}
+/* Loads a saved state: counters, running max and the stored leaves of slots [0, n) (values as
+ * stored, i.e. already raised to alpha); every other leaf becomes empty and every internal node is
+ * recomputed from its two children, bottom-up - the value a leaf-to-root walk after the last write
+ * leaves there. */
+int orc_per_load_state(orc_per *b, const int64_t *in4, const float *leaves, int64_t n, float max_priority) {
+    int64_t cap = b->rows.capacity;
+    int64_t want = in4[1] < cap ? in4[1] : cap;
+    if (in4[1] < 0 || in4[0] != want || n < 0 || n > cap) return 1;
+    b->size = in4[0], b->pushes = in4[1], b->seed = (uint64_t)in4[2], b->calls = (uint64_t)in4[3];
+    b->max_priority = max_priority;
+    for (int64_t i = 0; i < b->leaves; ++i) {
+        b->sum[b->leaves + i] = i < n ? leaves[i] : 0.0f;
+        b->mn[b->leaves + i] = i < n ? leaves[i] : FLT_MAX;
+    }
+    for (int64_t i = b->leaves - 1; i >= 1; --i) {
+        b->sum[i] = b->sum[2 * i] + b->sum[2 * i + 1];
+        b->mn[i] = fminf(b->mn[2 * i], b->mn[2 * i + 1]);
+    }
+    return 0;
+}

@@ -51,6 +51,8 @@ def lib():
         "orc_urb_count": (i64, [vp]),
         "orc_urb_head": (i64, [vp]),
         "orc_urb_field": (vp, [vp, C.c_int]),
+        "orc_urb_get_state": (None, [vp, vp]),
+        "orc_urb_set_state": (C.c_int, [vp, vp]),
         "orc_discounted_return": (None, [vp, vp, vp, vp, i64, i64, i64, f32]),
         "orc_res_create": (vp, [i64, C.c_int, vp, u64]),
         "orc_res_destroy": (None, [vp]),
@@ -59,6 +61,8 @@ def lib():
         "orc_res_size": (i64, [vp]),
         "orc_res_total": (i64, [vp]),
         "orc_res_field": (vp, [vp, C.c_int]),
+        "orc_res_get_state": (None, [vp, vp]),
+        "orc_res_set_state": (C.c_int, [vp, vp]),
         "orc_per_create": (vp, [i64, f32, C.c_int, vp, u64]),
         "orc_per_destroy": (None, [vp]),
         "orc_per_update": (C.c_int, [vp, vp, vp, i64]),
@@ -70,6 +74,8 @@ def lib():
         "orc_per_head": (i64, [vp]),
         "orc_per_max_priority": (f32, [vp]),
         "orc_per_field": (vp, [vp, C.c_int]),
+        "orc_per_get_state": (None, [vp, vp]),
+        "orc_per_load_state": (C.c_int, [vp, vp, vp, i64, f32]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -146,6 +152,27 @@ class _Rows:
             return [np.empty(s, d) for s, d in zip(self.shapes, self.dtypes)]
         return [np.empty((n,) + s, d) for s, d in zip(self.shapes, self.dtypes)]
 
+    def _storage(self, field_fn, i):
+        """Writable view of field i's storage [capacity, *shape] inside the oracle."""
+        n = self.capacity * self.bytes[i]
+        raw = (C.c_ubyte * n).from_address(field_fn(self.h, i))
+        return np.frombuffer(raw, np.uint8).view(self.dtypes[i]).reshape((self.capacity,) + self.shapes[i])
+
+    def _load_rows(self, field_fn, fields):
+        for i, f in enumerate(fields):
+            a = np.asarray(f, dtype=self.dtypes[i])
+            self._storage(field_fn, i)[: a.shape[0]] = a.reshape((a.shape[0],) + self.shapes[i])
+
+    @staticmethod
+    def _counters(get_fn, h):
+        out = np.zeros(4, np.int64)
+        get_fn(h, out.ctypes.data)
+        return [int(v) for v in out]
+
+    @staticmethod
+    def _as_i64(values):
+        return np.array([int(v) - (1 << 64) if int(v) >= (1 << 63) else int(v) for v in values], np.int64)
+
 
 class OracleUniform(_Rows):
     """CPU twin of UniformReplayBuffer (mindspore_rl/core/uniform_replay_buffer.py:50-172)."""
@@ -190,6 +217,20 @@ class OracleUniform(_Rows):
 
     def reset(self):
         lib().orc_urb_reset(self.h)
+
+    def state_dict(self):
+        """Same layout as mindrl_amd.core.UniformReplayBuffer.state_dict() (numpy instead of torch)."""
+        count, head, seed, calls = self._counters(lib().orc_urb_get_state, self.h)
+        return {"kind": "uniform", "capacity": self.capacity, "count": count, "head": head,
+                "seed": seed & ((1 << 64) - 1), "calls": calls,
+                "fields": [self.field(i) for i in range(len(self.bytes))]}
+
+    def load_state_dict(self, state):
+        assert state["kind"] == "uniform" and state["capacity"] == self.capacity
+        self._load_rows(lib().orc_urb_field, [np.asarray(f) for f in state["fields"]])
+        c = self._as_i64([state["count"], state["head"], state["seed"], state["calls"]])
+        if lib().orc_urb_set_state(self.h, c.ctypes.data):
+            raise ValueError("orc_urb_set_state failed")
 
     @property
     def count(self):
@@ -240,6 +281,19 @@ class OracleReservoir(_Rows):
     def total(self):
         return lib().orc_res_total(self.h)
 
+    def state_dict(self):
+        size, total, seed, calls = self._counters(lib().orc_res_get_state, self.h)
+        return {"kind": "reservoir", "capacity": self.capacity, "size": size, "total": total,
+                "seed": seed & ((1 << 64) - 1), "calls": calls,
+                "fields": [self.field(i)[:size] for i in range(len(self.bytes))]}
+
+    def load_state_dict(self, state):
+        assert state["kind"] == "reservoir" and state["capacity"] == self.capacity
+        self._load_rows(lib().orc_res_field, [np.asarray(f) for f in state["fields"]])
+        c = self._as_i64([state["size"], state["total"], state["seed"], state["calls"]])
+        if lib().orc_res_set_state(self.h, c.ctypes.data):
+            raise ValueError("orc_res_set_state failed")
+
     def field(self, i):
         n = self.capacity * self.bytes[i]
         raw = (C.c_ubyte * n).from_address(lib().orc_res_field(self.h, i))
@@ -252,6 +306,7 @@ class OraclePER(_Rows):
     def __init__(self, alpha, capacity, shapes, dtypes, seed=0):
         super().__init__(shapes, dtypes)
         self.capacity = int(capacity)
+        self.alpha = float(alpha)
         self.h = lib().orc_per_create(self.capacity, float(alpha), len(self.bytes), self._fb, seed)
         if not self.h:
             raise ValueError("orc_per_create failed")
@@ -315,6 +370,23 @@ class OraclePER(_Rows):
     @property
     def max_priority(self):
         return lib().orc_per_max_priority(self.h)
+
+    def state_dict(self):
+        size, pushes, seed, calls = self._counters(lib().orc_per_get_state, self.h)
+        s, _ = self.export_tree()
+        return {"kind": "priority", "capacity": self.capacity, "alpha": self.alpha, "size": size, "pushes": pushes,
+                "seed": seed & ((1 << 64) - 1), "calls": calls, "max_priority": float(self.max_priority),
+                "leaves": s[self.leaves:self.leaves + size].copy(),
+                "fields": [self.field(i)[:size] for i in range(len(self.bytes))]}
+
+    def load_state_dict(self, state):
+        assert state["kind"] == "priority" and state["capacity"] == self.capacity
+        assert np.float32(state["alpha"]) == np.float32(self.alpha)
+        self._load_rows(lib().orc_per_field, [np.asarray(f) for f in state["fields"]])
+        leaves = np.ascontiguousarray(np.asarray(state["leaves"]), np.float32)
+        c = self._as_i64([state["size"], state["pushes"], state["seed"], state["calls"]])
+        if lib().orc_per_load_state(self.h, c.ctypes.data, leaves.ctypes.data, leaves.size, float(state["max_priority"])):
+            raise ValueError("orc_per_load_state failed")
 
     def field(self, i):
         n = self.capacity * self.bytes[i]

@@ -75,6 +75,79 @@ def test_uniform_ring_random_ops(mrb, orc, layout, cap):
     g.destroy()
 
 
+def test_config2_sac_shape_full_size(mrb, orc):
+    """BASELINE config 2 at its real size: capacity 1,000,000, rows f32[17] + f32[6] + f32[1] + f32[17] + bool
+    (165 B, mindspore_rl/algorithm/sac/config.py:95-100), filled by 1000 appends of 1000 rows
+    (mindspore_rl/core/uniform_replay_buffer.py:101-115), then batches of 256 gathered at seeded host-drawn
+    indices integers(0, count) (uniform_replay_buffer.py:130-139). Storage, count / head and every gathered
+    row are compared with the oracle."""
+    shapes, dtypes = URB_LAYOUTS[1]
+    cap, chunk, batch = 1_000_000, 1000, 256
+    rng = np.random.default_rng(1002)
+    g = mrb.URB(batch, cap, shapes, torch_types(dtypes), seed=1002)
+    c = orc.OracleUniform(cap, shapes, dtypes, seed=1002)
+    for i in range(cap // chunk + 3):  # three chunks past the capacity: the ring wraps
+        rows = [rng.normal(size=(chunk, 17)).astype(np.float32), rng.uniform(-1, 1, (chunk, 6)).astype(np.float32),
+                rng.normal(size=(chunk, 1)).astype(np.float32), rng.normal(size=(chunk, 17)).astype(np.float32),
+                rng.random((chunk, 1)) < 0.01]
+        g.insert(to_dev(rows))
+        c.append(rows, chunk)
+        if i in (0, 499, cap // chunk - 1, cap // chunk + 2):
+            assert (int(g.count), int(g.head)) == (c.count, c.head), i
+    assert (c.count, c.head) == (cap, 3 * chunk)
+    for f in range(len(shapes)):
+        assert np.array_equal(t2n(g.buffer[f]).view(np.uint8), c.field(f).view(np.uint8)), f
+    for call in range(20):
+        idx = rng.integers(0, c.count, batch)
+        for a, b in zip(g.sample(indices=torch.from_numpy(idx).cuda()), c.gather(idx)):
+            assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8)), call
+    gi, gf = g.sample_with_indices()  # the buffer's own generator on the full ring
+    ci, cf = c.sample(batch)
+    assert np.array_equal(t2n(gi), ci)
+    for a, b in zip(gf, cf):
+        assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+    for j in (0, -1, cap // 2):
+        for a, b in zip(g.get_item(j), c.get_item(j)):
+            assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+    g.check()
+    g.destroy()
+
+
+def test_options_belong_to_one_buffer(mrb, orc):
+    """Two prioritized buffers with the same contents, one forced onto the wide-row kernel with three
+    workgroups per row, the other onto the LDS-top kernel with 5 staged levels: interleaved calls give the
+    same bit-exact results, i.e. no option of one handle reaches the other."""
+    shapes, dtypes = [(300,), (1,)], [np.float32, np.int32]  # a 1200-byte field: wide rows
+    rng = np.random.default_rng(8)
+    cap, batch = 3000, 64
+    a, c = make_pair(mrb, orc, 0.6, cap, batch, seed=4, shapes=shapes, dtypes=dtypes)
+    b = mrb.PER(0.6, cap, batch, shapes, torch_types(dtypes), seed0=4)
+    a.set_option("sample_path", 1), a.set_option("row_split", 3)
+    b.set_option("sample_path", 2), b.set_option("lds_levels", 5)
+    with pytest.raises(ValueError):
+        a.set_option("no_such_option", 1)
+    with pytest.raises(ValueError):
+        a.set_option("row_split", 1000)
+    u = mrb.URB(8, 10, shapes, torch_types(dtypes))
+    with pytest.raises(ValueError):
+        u.set_option("sample_path", 1)  # an option of prioritized buffers
+    u.set_option("row_split", 2)
+    u.destroy()
+    rows = random_rows(rng, cap, shapes, dtypes)
+    a.insert(*to_dev(rows)), b.insert(*to_dev(rows)), c.push(rows, cap)
+    for step in range(6):
+        idx = rng.integers(0, cap, 500)
+        pr = (rng.pareto(1.5, 500) + 1e-6).astype(np.float32)
+        for buf in (a, b):
+            buf.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda())
+        c.update(idx, pr)
+        un = rng.random(batch).astype(np.float32)
+        want = c.sample(batch, 0.5, un)
+        assert_sample_equal(a.sample(0.5, uniforms=torch.from_numpy(un).cuda()), want, "wide step %d" % step)
+        assert_sample_equal(b.sample(0.5, uniforms=torch.from_numpy(un).cuda()), want, "lds step %d" % step)
+    a.destroy(), b.destroy()
+
+
 def test_uniform_primitive_attributes_used_by_reference_callers(mrb):
     """A subclass written like mindspore_rl/algorithm/mappo/mappo_replaybuffer.py:23-44 works unchanged,
     and buffer_sample.batch_size is readable (mindspore_rl/algorithm/gail/gail.py:163-164)."""
@@ -180,6 +253,125 @@ def test_state_dict_round_trip_continues_identically(mrb, tmp_path):
     for x, y in zip(r.sample(), q.sample()):
         assert torch.equal(x, y)
     r.destroy(), q.destroy()
+
+
+def test_state_dict_cross_loads_with_the_oracle(mrb, orc):
+    """The checkpoint path against the oracle, both ways: a state saved by the HIP buffer is loaded into
+    an oracle buffer, a state saved by an oracle buffer into a fresh HIP buffer; each pair then continues
+    with identical calls and must agree bit for bit (trees, running max, draws, rows, storage)."""
+    rng = np.random.default_rng(2024)
+    shapes, dtypes = [(5,), (1,), (40,)], [np.float32, np.int32, np.uint8]
+
+    def per_pair_continues(g, c, what):
+        for step in range(6):
+            assert_tree_equal(g, c, "%s step %d" % (what, step))
+            assert np.float32(g.max_priority) == np.float32(c.max_priority) and g.size() == c.size
+            u = rng.random(16).astype(np.float32)
+            out = g.sample(0.6, uniforms=torch.from_numpy(u).cuda())
+            assert_sample_equal(out, c.sample(16, 0.6, u), "%s step %d" % (what, step))
+            assert_sample_equal(g.sample(0.9), c.sample(16, 0.9), "%s step %d generator" % (what, step))
+            rows = random_rows(rng, 9, shapes, dtypes)
+            g.insert(*to_dev(rows)), c.push(rows, 9)
+            idx = rng.integers(0, c.size, 50)
+            pr = (rng.pareto(1.5, 50) + 1e-6).astype(np.float32)
+            g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda()), c.update(idx, pr)
+        for f, view in enumerate(g.storage()):
+            assert np.array_equal(t2n(view).view(np.uint8), c.field(f).view(np.uint8)), (what, f)
+
+    for cap in (300, 1000):  # 300: wrapped ring; 1000: partly filled
+        # HIP -> oracle
+        g = mrb.PER(0.6, cap, 16, shapes, torch_types(dtypes), seed0=5)
+        g.insert(*to_dev(random_rows(rng, 450, shapes, dtypes)))
+        g.update_priorities(torch.from_numpy(rng.integers(0, min(cap, 450), 200)).cuda(),
+                            torch.from_numpy(rng.pareto(1.5, 200).astype(np.float32) + 1e-6).cuda())
+        g.sample(0.4)  # advances the generator
+        c = orc.OraclePER(0.6, cap, shapes, dtypes, seed=12345)
+        c.load_state_dict(g.state_dict())
+        per_pair_continues(g, c, "hip->oracle cap %d" % cap)
+        g.destroy()
+        # oracle -> HIP
+        c = orc.OraclePER(0.6, cap, shapes, dtypes, seed=8)
+        c.push(random_rows(rng, 450, shapes, dtypes), 450)
+        c.update(rng.integers(0, min(cap, 450), 200), rng.pareto(1.5, 200).astype(np.float32) + 1e-6)
+        c.sample(16, 0.4)
+        g = mrb.PER(0.6, cap, 16, shapes, torch_types(dtypes), seed0=999)
+        g.load_state_dict(c.state_dict())
+        per_pair_continues(g, c, "oracle->hip cap %d" % cap)
+        with pytest.raises(ValueError):  # leaves are priorities ** alpha: another alpha must be refused
+            mrb.PER(0.5, cap, 16, shapes, torch_types(dtypes)).load_state_dict(c.state_dict())
+        g.destroy()
+
+    # uniform ring, wrapped, both ways
+    u = mrb.URB(8, 50, shapes, torch_types(dtypes), seed=3)
+    u.insert(to_dev(random_rows(rng, 70, shapes, dtypes)))
+    u.sample()
+    cu = orc.OracleUniform(50, shapes, dtypes, seed=77)
+    cu.load_state_dict(u.state_dict())
+    cw = orc.OracleUniform(50, shapes, dtypes, seed=4)
+    cw.append(random_rows(rng, 85, shapes, dtypes), 85)
+    cw.sample(8)
+    w = mrb.URB(8, 50, shapes, torch_types(dtypes), seed=5)
+    w.load_state_dict(cw.state_dict())
+    for gb, cb in ((u, cu), (w, cw)):
+        for step in range(4):
+            assert (int(gb.count), int(gb.head)) == (cb.count, cb.head)
+            gi, gf = gb.sample_with_indices()
+            ci, cf = cb.sample(8)
+            assert np.array_equal(t2n(gi), ci)
+            for a, b in zip(gf, cf):
+                assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+            rows = random_rows(rng, 13, shapes, dtypes)
+            gb.insert(to_dev(rows)), cb.append(rows, 13)
+            for a, b in zip(gb.get_item(-1), cb.get_item(-1)):
+                assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+        for f in range(len(shapes)):
+            assert np.array_equal(t2n(gb.buffer[f]).view(np.uint8), cb.field(f).view(np.uint8))
+        gb.destroy()
+
+    # reservoir past its capacity, both ways
+    r = mrb.RES(20, 8, shapes, torch_types(dtypes), seed1=6)
+    r.push(*to_dev(random_rows(rng, 90, shapes, dtypes)))
+    r.sample()
+    cr = orc.OracleReservoir(20, shapes, dtypes, seed=1)
+    cr.load_state_dict(r.state_dict())
+    cq = orc.OracleReservoir(20, shapes, dtypes, seed=9)
+    cq.push(random_rows(rng, 75, shapes, dtypes), 75)
+    cq.sample(8)
+    q = mrb.RES(20, 8, shapes, torch_types(dtypes), seed1=7)
+    q.load_state_dict(cq.state_dict())
+    for gb, cb in ((r, cr), (q, cq)):
+        for step in range(4):
+            rows = random_rows(rng, 40, shapes, dtypes)
+            gb.push(*to_dev(rows)), cb.push(rows, 40)
+            gi, gf = gb.sample(with_indices=True)
+            ci, cf = cb.sample(8)
+            assert np.array_equal(t2n(gi), ci)
+            for a, b in zip(gf, cf):
+                assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+        for f, view in enumerate(gb.storage()):
+            assert np.array_equal(t2n(view).view(np.uint8), cb.field(f).view(np.uint8))
+        gb.destroy()
+
+
+def test_zero_priority_gives_zero_weights_not_infinite_ones(mrb, orc):
+    """A leaf updated to priority 0 makes the tree minimum 0: (0 / total * size)^-beta is +inf as with
+    pow(), so every importance weight becomes 0 - on the oracle and on the GPU alike - and nothing is flagged."""
+    shapes, dtypes = [(2,)], [np.float32]
+    g, c = make_pair(mrb, orc, 0.6, 64, 8, seed=3, shapes=shapes, dtypes=dtypes)
+    rng = np.random.default_rng(5)
+    rows = random_rows(rng, 64, shapes, dtypes)
+    g.insert(*to_dev(rows)), c.push(rows, 64)
+    idx, pr = np.array([7, 30]), np.array([0.0, 2.5], np.float32)
+    g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda()), c.update(idx, pr)
+    u = rng.random(8).astype(np.float32)
+    for path in (1, 2):
+        g.set_option("sample_path", path)
+        gi, gw = g.sample(0.4, uniforms=torch.from_numpy(u).cuda())[:2]
+        ci, cw, _ = c.sample(8, 0.4, u)
+        assert np.array_equal(t2n(gi), ci) and 7 not in ci
+        assert np.array_equal(bits(t2n(gw)), bits(cw)) and np.all(cw == 0.0)
+    assert g.check() == 0
+    g.destroy()
 
 
 # --------------------------------------------------------- discounted return

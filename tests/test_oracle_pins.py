@@ -37,6 +37,12 @@ def test_powf_exact_cases(orc):
     assert orc.powf(2.0, -1.0) == 0.5
     assert orc.powf(1e30, 2.0) == np.inf
     assert orc.powf(1e-30, 2.0) == 0.0
+    # zero base, as libm pow(): 0^a is 0 for a > 0 and +inf for a < 0 (a zero minimum priority then
+    # gives importance weights r / inf = 0, not r / 0 = inf)
+    for a in (-0.4, -1.0, -2.5):
+        assert orc.powf(0.0, a) == np.inf
+    with np.errstate(divide="ignore"):
+        assert np.power(np.float64(0.0), -0.4) == np.inf  # what numpy's pow (libm) gives for the same case
     # monotone in x for a > 0
     x = np.linspace(0.001, 10, 5000).astype(np.float32)
     assert np.all(np.diff(orc.powf_array(x, 0.6)) >= 0)
@@ -215,6 +221,54 @@ def test_tree_equals_pairwise_rebuild_after_random_ops(orc, cap):
         assert np.array_equal(m[1:].view(np.int32), em[1:].view(np.int32))
         assert per.max_priority == maxp
         assert per.size == min(pushes, cap) and per.head == pushes % cap
+
+
+def test_load_state_rebuilds_the_same_tree_and_continues_identically(orc):
+    """orc_per_load_state (leaves in, every internal node recomputed bottom-up) against numpy's pairwise
+    reduction of the same leaves, and against the buffer the state came from, which then takes the same
+    calls; the same for the uniform ring and the reservoir."""
+    rng = np.random.default_rng(31)
+    for cap in (5, 64, 100):
+        a = new_per(orc, 0.6, cap)
+        a.push(rows_for(cap + 3, 0), cap + 3)
+        a.update(rng.integers(0, cap, 40), np.abs(rng.normal(size=40)).astype(np.float32) + np.float32(1e-6))
+        a.sample(4, 0.5)
+        state = a.state_dict()
+        b = new_per(orc, 0.6, cap)
+        b.load_state_dict(state)
+        leaves = a.leaves
+        leaf = np.zeros(leaves, np.float32)
+        leafmin = np.full(leaves, np.finfo(np.float32).max, np.float32)
+        leaf[:a.size] = leafmin[:a.size] = state["leaves"]
+        es, em = pairwise_levels(leaf, leafmin)
+        s, m = b.export_tree()
+        assert np.array_equal(s[1:].view(np.int32), es[1:].view(np.int32))
+        assert np.array_equal(m[1:].view(np.int32), em[1:].view(np.int32))
+        for step in range(5):
+            ia, wa, ra = a.sample(4, 0.7)
+            ib, wb, rb = b.sample(4, 0.7)
+            assert np.array_equal(ia, ib) and np.array_equal(wa.view(np.int32), wb.view(np.int32))
+            assert all(np.array_equal(x, y) for x, y in zip(ra, rb))
+            a.push(rows_for(3, 1000 + step), 3), b.push(rows_for(3, 1000 + step), 3)
+            a.update(ia, wa + np.float32(0.5)), b.update(ib, wb + np.float32(0.5))
+            assert a.max_priority == b.max_priority and (a.size, a.head) == (b.size, b.head)
+            assert np.array_equal(a.export_tree()[0][1:].view(np.int32), b.export_tree()[0][1:].view(np.int32))
+    shapes, dtypes = [(2,)], [np.int32]
+    u = orc.OracleUniform(7, shapes, dtypes, seed=3)
+    u.append([np.arange(24).reshape(12, 2)], 12)
+    u.sample(3)
+    w = orc.OracleUniform(7, shapes, dtypes, seed=99)
+    w.load_state_dict(u.state_dict())
+    assert (w.count, w.head) == (u.count, u.head) == (7, 5)
+    assert np.array_equal(u.sample(3)[0], w.sample(3)[0]) and np.array_equal(u.get_item(0)[0], w.get_item(0)[0])
+    r = orc.OracleReservoir(6, shapes, dtypes, seed=4)
+    r.push([np.arange(60).reshape(30, 2)], 30)
+    q = orc.OracleReservoir(6, shapes, dtypes, seed=5)
+    q.load_state_dict(r.state_dict())
+    more = [np.arange(100, 140).reshape(20, 2)]
+    r.push(more, 20), q.push(more, 20)
+    assert np.array_equal(r.field(0), q.field(0)) and (r.size, r.total) == (q.size, q.total) == (6, 50)
+    assert np.array_equal(r.sample(4)[0], q.sample(4)[0])
 
 
 def test_root_is_pairwise_not_sequential_sum(orc):
