@@ -1,28 +1,51 @@
-"""Builds buffers from the reference's `replay_buffer` config entry.
+"""Builds buffers from the `replay_buffer` entry of a MindRL algorithm config.
 
-Mirrors MSRL.__create_replay_buffer (mindspore_rl/core/msrl.py:270-300): the entry
-names the class under 'type', an optional 'number' of instances, either a 'params'
-dict or 'sample_size' / 'capacity', and the per-element 'data_shape' / 'data_type'
-that the algorithm's session fills in (mindspore_rl/algorithm/dqn/dqn_session.py:50-61).
+The entry's schema is the reference's (mindspore_rl/core/msrl.py:270-300, filled in by the
+algorithm's session, e.g. mindspore_rl/algorithm/dqn/dqn_session.py:50-61):
+
+    type         the buffer class (required)
+    number       how many instances to build (default 1; more than one returns a list)
+    params       constructor keywords, OR
+    sample_size  (default 1) and
+    capacity     when there is no `params`
+    data_shape   per-field shapes  -> constructor keyword `shapes`
+    data_type    per-field dtypes  -> constructor keyword `types`
 """
+
+_KNOWN_KEYS = frozenset(["type", "number", "params", "sample_size", "capacity", "data_shape", "data_type"])
+
+
+class ReplayBufferSpec:
+    """A validated `replay_buffer` config entry: which class to build, how often, with which keywords."""
+
+    def __init__(self, entry):
+        if not isinstance(entry, dict):
+            raise TypeError("a replay_buffer config entry is a dict, got %s" % type(entry).__name__)
+        unknown = sorted(set(entry) - _KNOWN_KEYS)
+        if unknown:
+            raise KeyError("unknown replay_buffer config keys: %s" % ", ".join(map(str, unknown)))
+        if "type" not in entry:
+            raise KeyError("the replay_buffer config entry names no 'type'")
+        if entry.get("data_shape") is None or entry.get("data_type") is None:
+            raise KeyError("the replay_buffer config entry needs 'data_shape' and 'data_type'")
+        self.cls = entry["type"]
+        self.count = int(entry.get("number", 1))
+        if self.count < 1:
+            raise ValueError("'number' must be at least 1, got %d" % self.count)
+        explicit = entry.get("params")
+        if explicit:
+            self.kwargs = dict(explicit)  # a copy: the caller's config is left as it is
+        else:
+            self.kwargs = {"sample_size": entry.get("sample_size", 1), "capacity": entry.get("capacity")}
+        self.kwargs.update(shapes=tuple(entry["data_shape"]), types=tuple(entry["data_type"]))
+
+    def build(self):
+        made = [self.cls(**self.kwargs) for _ in range(self.count)]
+        return made[0] if self.count == 1 else made
 
 
 def create_replay_buffer(replay_buffer_config):
-    """Returns one buffer, or a list of `number` buffers, for a config dict such as
+    """One buffer, or a list of `number` buffers, for an entry such as
     {'number': 1, 'type': UniformReplayBuffer, 'capacity': 100000, 'sample_size': 64,
      'data_shape': [(4,), (1,), (1,), (4,)], 'data_type': [float32, int32, float32, float32]}."""
-    num_replay_buffer = replay_buffer_config.get("number", 1)
-    replay_buffer_type = replay_buffer_config["type"]
-    params = replay_buffer_config.get("params", None)
-    if not params:
-        params = {
-            "sample_size": replay_buffer_config.get("sample_size", 1),
-            "capacity": replay_buffer_config.get("capacity"),
-        }
-    else:
-        params = dict(params)
-    params["shapes"] = tuple(replay_buffer_config.get("data_shape"))
-    params["types"] = tuple(replay_buffer_config.get("data_type"))
-    if num_replay_buffer == 1:
-        return replay_buffer_type(**params)
-    return [replay_buffer_type(**params) for _ in range(num_replay_buffer)]
+    return ReplayBufferSpec(replay_buffer_config).build()

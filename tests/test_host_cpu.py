@@ -129,6 +129,16 @@ def test_create_replay_buffer_follows_the_reference_config_entry():
     assert with_params.args == (2, 5, ((1,),), ("float32",))
     default_size = create_replay_buffer({"type": Fake, "capacity": 7, "data_shape": [(1,)], "data_type": ["int32"]})
     assert default_size.args[0] == 1
+    params = {"sample_size": 2, "capacity": 5}
+    create_replay_buffer({"type": Fake, "params": params, "data_shape": [(1,)], "data_type": ["float32"]})
+    assert params == {"sample_size": 2, "capacity": 5}  # the caller's dict is not written to
+    for bad in ({"capacity": 7, "data_shape": [(1,)], "data_type": ["int32"]},               # no type
+                {"type": Fake, "capacity": 7, "data_type": ["int32"]},                        # no data_shape
+                {"type": Fake, "capacity": 7, "data_shape": [(1,)], "data_type": ["int32"], "sampel_size": 3}):
+        with pytest.raises(KeyError):
+            create_replay_buffer(bad)
+    with pytest.raises(ValueError):
+        create_replay_buffer(dict(cfg, number=0))
 
 
 def test_bench_refuses_more_than_one_gpu():
