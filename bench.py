@@ -1,20 +1,23 @@
 #!/usr/bin/env python3
 """Replay-buffer hot-path benchmark on one MI355X.
 
-A step is one pass of the hot path over one batch: PriorityReplayBuffer.sample
-(stratified sum-tree descent + importance weights + row gather) on the
-Atari-shaped buffer of capacity 1,000,000 (28,241 stored bytes per row, batch
-512). Inputs are synthetic and resident in HBM before the timed region; the
-sampling uniforms are drawn on the host beforehand, one set per step.
+A step is one pass of the hot path over one batch. The default workload is BASELINE config 3:
+PriorityReplayBuffer.sample (stratified sum-tree descent + importance weights + row gather) on the
+Atari-shaped buffer of capacity 1,000,000 (28,241 stored bytes per row, batch 512), one C-ABI call
+per step on one stream, every call ordered after the one before it. Inputs are synthetic and resident
+in HBM before the timed region; the sampling uniforms are drawn on the host beforehand, one set per step.
 
-Prints ONE JSON line. `roofline` prices the sample kernel's algorithmic bytes
-against the HBM peak; `cpu_baseline` is the CPU oracle timed on this machine's
-host cores on a bounded sample of the same workload (rank 0, N = 1 only).
+Prints ONE JSON line. `roofline` prices the dominant kernel's algorithmic bytes against the HBM peak with
+the launch duration measured by HIP events over the timed region; `cpu_baseline` is the CPU oracle
+(a sequential C restatement of the reference path) timed on this machine's host cores on a bounded
+sample of the same workload. Other workloads: c1 (DQN-PER loop), c2 (uniform buffer gather), c4, c5
+(prioritized, narrow rows), res (reservoir), dr (discounted return).
 """
 import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,8 +29,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-WORKLOADS = {
+PER_WORKLOADS = {
     # name: (capacity, batch, shapes, numpy dtypes, update n, insert n, description)
+    "c1": (10_000, 64, [(4,), (1,), (1,), (4,), (1,)], ["float32", "int32", "float32", "float32", "bool"], 64, 1,
+           "config 1: DQN-PER CartPole-shaped PriorityReplayBuffer, capacity 10,000, 41 B rows; step = sample 64 + "
+           "update_priorities 64 + insert 1"),
     "c3": (1_000_000, 512, [(84, 84, 4), (1,), (1,), (1,), (1,)], ["uint8", "int64", "int32", "float32", "bool"],
            512, 4, "config 3: Atari-shaped PriorityReplayBuffer, capacity 1,000,000, 28,241 B stored rows "
                    "(obs u8[84,84,4] + next_idx i64 + action i32 + reward f32 + done bool), batch 512"),
@@ -36,6 +42,12 @@ WORKLOADS = {
     "c5": (1 << 24, 65536, [(1,), (1,)], ["int32", "float32"], 65536, 4096,
            "config 5: tree-descent stress, capacity 16,777,216, 8 B rows, batch 65,536"),
 }
+WORKLOAD_CAP = {k: v[0] for k, v in PER_WORKLOADS.items()}
+# the rocprofv3 summary that holds the tracked figures of a workload's dominant kernel
+PROFILE_OF = {
+    "c3": "k_per_sample_wide_config3_atari_cap1M_batch512.md",
+    "c5": "k_per_sample_lds_and_tree_update_config5_2pow24_batch65536.md",
+}
 
 
 def parse():
@@ -43,18 +55,50 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=2000)
     p.add_argument("--warmup", type=int, default=200)
-    p.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c2", "res", "dr"])
+    p.add_argument("--workload", default="c3", choices=sorted(PER_WORKLOADS) + ["c2", "res", "dr"])
     p.add_argument("--capacity", type=int, default=0, help="override the workload's capacity (for quick trials)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--graph", action="store_true", help="replay the timed steps as one captured HIP graph")
     p.add_argument("--row-split", type=int, default=0, help="workgroups per sampled row (0 = library default)")
     p.add_argument("--sample-path", type=int, default=0, help="0 auto, 1 wide-row kernel, 2 LDS-top kernel")
-    p.add_argument("--extras", action="store_true", help="also time update_priorities, insert and the full loop")
+    p.add_argument("--no-extras", action="store_true",
+                   help="skip the untimed side figures (update, insert, loop, graph replay, several streams)")
     return p.parse_args()
 
 
-def fill_per(buf, torch, capacity, shapes, np_dtypes, seed):
-    """Prefill to capacity in chunks (rows generated on the device), then set lognormal priorities."""
+def profile_figures(workload):
+    """Figures of the committed rocprofv3 summary of this workload's dominant kernel (lines `key: number`
+    in its "figures" block), or {} if the summary is not there."""
+    name = PROFILE_OF.get(workload)
+    path = os.path.join(ROOT, "profiles", name) if name else None
+    if not path or not os.path.exists(path):
+        return {}, name
+    out = {}
+    for key, val in re.findall(r"^\s*(rocprof_avg_ns|traffic_bytes_per_launch):\s*([0-9.eE+]+)\s*$",
+                               open(path).read(), re.M):
+        out[key] = float(val)
+    return out, name
+
+
+def roofline(kernel, algo_bytes, kern_s, wall_s_per_step, workload, formula, defaults=True):
+    """achieved = algorithmic bytes per launch / average launch duration (HIP events over the timed
+    region); frac_wall prices the same bytes with the host's wall clock per step. The rocprofv3 average
+    and the counter-measured HBM traffic cannot be measured inside this process: they are read from the
+    committed summary of this very command, and left out (null) when the run is not the default one."""
+    fig, name = profile_figures(workload) if defaults else ({}, PROFILE_OF.get(workload))
+    achieved = algo_bytes / kern_s / 1e9
+    r = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+         "traffic": fig.get("traffic_bytes_per_launch"), "kernel": kernel, "algorithmic_bytes_per_launch": algo_bytes,
+         "algorithmic_bytes": formula, "avg_launch_us": kern_s * 1e6,
+         "frac_wall": algo_bytes / wall_s_per_step / 1e9 / HBM_PEAK_GBS, "profile": name}
+    if "rocprof_avg_ns" in fig:
+        r["rocprof_avg_us"] = fig["rocprof_avg_ns"] * 1e-3
+        r["frac_kernel_rocprof"] = algo_bytes / (fig["rocprof_avg_ns"] * 1e-9) / 1e9 / HBM_PEAK_GBS
+    return r
+
+
+def fill_per(buf, torch, capacity, shapes, np_dtypes, seed, lognormal=True):
+    """Prefill to capacity in chunks (rows generated on the device), then set the priorities."""
     gen = torch.Generator(device="cuda").manual_seed(seed)
     row_bytes = sum(int(np.prod(s)) * np.dtype(d).itemsize for s, d in zip(shapes, np_dtypes))
     chunk = max(1, min(capacity, (256 << 20) // row_bytes))
@@ -76,21 +120,24 @@ def fill_per(buf, torch, capacity, shapes, np_dtypes, seed):
                 fields.append(torch.randint(0, 18, (n,) + tuple(s), dtype=torch.int32, device="cuda", generator=gen))
         buf.insert(*fields)
         done += n
-    rng = np.random.default_rng(seed)
-    pr = rng.lognormal(0.0, 1.0, capacity).astype(np.float32)
-    buf.update_priorities(torch.arange(capacity, device="cuda"), torch.from_numpy(pr).cuda())
+    if lognormal:
+        rng = np.random.default_rng(seed)
+        pr = rng.lognormal(0.0, 1.0, capacity).astype(np.float32)
+        buf.update_priorities(torch.arange(capacity, device="cuda"), torch.from_numpy(pr).cuda())
     torch.cuda.synchronize()
-    return pr
 
 
-def cpu_baseline(workload, shapes, np_dtypes, batch, seed):
-    """The CPU oracle (sequential C restatement of the reference path) on this host:
-    same row shape and batch, capacity cut to 131,072 rows to bound memory and time."""
+def oracle_per(workload, shapes, np_dtypes, seed, lognormal=True):
+    """The CPU oracle filled like the GPU buffer. Config 3 is cut to 131,072 rows: its 10^6 rows of
+    28 KB would be 28 GB of host memory and minutes of filling; the tree then has 17 levels instead of
+    20, which favours the CPU. The other workloads run at their full capacity."""
     from oracle import orc
-    cap = min(WORKLOADS[workload][0], 1 << 17)
+    cap = WORKLOAD_CAP[workload]
+    if workload == "c3":
+        cap = min(cap, 1 << 17)
     rng = np.random.default_rng(seed)
     per = orc.OraclePER(0.6, cap, shapes, np_dtypes, seed=seed)
-    chunk = 2048
+    chunk = min(cap, 2048)
     rows = []
     for s, d in zip(shapes, np_dtypes):
         d = np.dtype(d)
@@ -101,8 +148,20 @@ def cpu_baseline(workload, shapes, np_dtypes, batch, seed):
         else:
             rows.append(rng.integers(0, 3, (chunk,) + tuple(s)).astype(d))
     for start in range(0, cap, chunk):
-        per.push(rows, min(chunk, cap - start))
-    per.update(np.arange(cap), rng.lognormal(0, 1, cap).astype(np.float32))
+        n = min(chunk, cap - start)
+        per.push([r[:n] for r in rows], n)
+    if lognormal:
+        for start in range(0, cap, 1 << 20):
+            n = min(1 << 20, cap - start)
+            per.update(np.arange(start, start + n), rng.lognormal(0, 1, n).astype(np.float32))
+    return per, cap, rows
+
+
+def cpu_baseline_sample(workload, shapes, np_dtypes, batch, seed):
+    """orc_per_sample (descent + weights + row copies) on one thread, and with the row copies on all cores."""
+    from oracle import orc
+    per, cap, _ = oracle_per(workload, shapes, np_dtypes, seed)
+    rng = np.random.default_rng(seed + 7)
     L = orc.lib()
     idx = np.empty(batch, np.int64)
     w = np.empty(batch, np.float32)
@@ -121,19 +180,274 @@ def cpu_baseline(workload, shapes, np_dtypes, batch, seed):
         return calls, time.perf_counter() - t0
 
     calls, dt = timed(10.0)
-    # all host cores: the tree walk stays sequential, the row copies are shared out with OpenMP
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     cores = max(1, min(cores, 16))
     orc.set_threads(cores)
     calls_mt, dt_mt = timed(4.0)
     orc.set_threads(1)
+    cut = " (cut from %d: 28 GB of host rows)" % WORKLOAD_CAP[workload] if cap != WORKLOAD_CAP[workload] else ""
     return {
         "value": calls * batch / dt, "unit": "transitions/s", "cores": 1, "kind": "port",
-        "sample": "%d sample calls (batch %d, same row shape) in %.1f s on a capacity-%d buffer, 1 thread" % (
-            calls, batch, dt, cap),
+        "sample": "%d sample calls (batch %d, same row shape) in %.1f s on a capacity-%d buffer%s, 1 thread" % (
+            calls, batch, dt, cap, cut),
         "all_cores": {"value": calls_mt * batch / dt_mt, "cores": cores,
                       "sample": "%d calls in %.1f s, row copies on %d OpenMP threads" % (calls_mt, dt_mt, cores)},
     }
+
+
+def cpu_baseline_loop(workload, shapes, np_dtypes, batch, upd_n, ins_n, seed):
+    """The same sample + update_priorities + insert loop on the oracle, one thread."""
+    from oracle import orc
+    per, cap, rows = oracle_per(workload, shapes, np_dtypes, seed, lognormal=False)
+    rng = np.random.default_rng(seed + 7)
+    L = orc.lib()
+    idx = np.empty(batch, np.int64)
+    w = np.empty(batch, np.float32)
+    dst = per._dst(batch)
+    dptr = orc._ptr_array(dst)
+    u_all = rng.random((64, batch)).astype(np.float32)
+    upd = min(upd_n, batch)
+    pr_all = (np.abs(rng.normal(size=(64, upd_n))) + 1e-6).astype(np.float32)
+    src = [np.ascontiguousarray(r[:ins_n]) for r in rows]
+    sptr = orc._ptr_array(src)
+    steps, t_end = 0, time.perf_counter() + 10.0
+    t0 = time.perf_counter()
+    while time.perf_counter() < t_end:
+        for _ in range(64):
+            i = steps % 64
+            L.orc_per_sample(per.h, batch, 0.4, u_all[i].ctypes.data, idx.ctypes.data, w.ctypes.data, dptr)
+            L.orc_per_update(per.h, idx.ctypes.data, pr_all[i].ctypes.data, upd)
+            L.orc_per_push(per.h, sptr, ins_n, None)
+            steps += 1
+    dt = time.perf_counter() - t0
+    return {"value": steps / dt, "unit": "steps/s", "cores": 1, "kind": "port",
+            "sample": "%d steps of sample %d + update %d + insert %d in %.1f s on a capacity-%d buffer, 1 thread" % (
+                steps, batch, upd, ins_n, dt, cap)}
+
+
+def events(torch):
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+class PerRun:
+    """One prioritized buffer filled for a workload, with the C-ABI calls of its step bound to device buffers."""
+
+    def __init__(self, a, torch):
+        from mindrl_amd import _lib
+        from mindrl_amd.core import PriorityReplayBuffer
+        from mindrl_amd.core._rows import pointers
+
+        self.torch, self._lib, self.pointers = torch, _lib, pointers
+        self.capacity, self.batch, self.shapes, self.np_dtypes, self.upd_n, self.ins_n, self.desc = PER_WORKLOADS[a.workload]
+        if a.capacity:
+            self.capacity = a.capacity
+            self.desc += " [capacity overridden to %d]" % a.capacity
+        self.loop_step = a.workload == "c1"  # config 1's step is the whole loop, the others time sample()
+        self.seed = 1000 + int(a.workload[1])
+        self.buf = PriorityReplayBuffer(0.6, self.capacity, self.batch, self.shapes,
+                                        [getattr(torch, d) for d in self.np_dtypes], seed0=self.seed)
+        self.buf.set_option("row_split", a.row_split)
+        self.buf.set_option("sample_path", a.sample_path)
+        t0 = time.perf_counter()
+        fill_per(self.buf, torch, self.capacity, self.shapes, self.np_dtypes, self.seed, lognormal=not self.loop_step)
+        self.fill_s = time.perf_counter() - t0
+        self.K, self.W = a.steps, a.warmup
+        n, batch = self.K + self.W, self.batch
+        self.rng = np.random.default_rng(self.seed + 1)
+        self.uniforms = torch.from_numpy(self.rng.random((n, batch)).astype(np.float32)).cuda()
+        self.betas = (np.linspace(0.4, 1.0, n) if a.workload == "c3" else np.full(n, 0.4)).astype(np.float32)
+        self.idx = torch.empty(batch, dtype=torch.int64, device="cuda")
+        self.wts = torch.empty(batch, dtype=torch.float32, device="cuda")
+        self.fields = self.buf._layout.empty(batch, self.buf._dev)
+        self.fptr = pointers(self.fields)
+        self.L = _lib.lib()
+        self.stream = torch.cuda.current_stream()
+        self.sp = C.c_void_p(self.stream.cuda_stream)
+        self.h = self.buf._h
+        self.upd = min(self.upd_n, batch)
+        self.upr = torch.from_numpy((np.abs(self.rng.normal(size=(64, self.upd_n))) + 1e-6).astype(np.float32)).cuda()
+        ins_n = self.ins_n
+        self.src = [f[:ins_n].contiguous() if f.shape[0] >= ins_n else
+                    f.repeat((ins_n + f.shape[0] - 1) // f.shape[0], *([1] * (f.dim() - 1)))[:ins_n].contiguous()
+                    for f in self.fields]
+        self.sptr = pointers(self.src)
+        # config 4 inserts its rows at actor-side priorities |N(0,1)| + eps; the others at the running max
+        self.ins_prio = (torch.randn(ins_n, device="cuda").abs() + 1e-6) if a.workload == "c4" else None
+        self.ins_pr = self.ins_prio.data_ptr() if self.ins_prio is not None else None
+
+    def sample(self, i, sp=None, out=None):
+        ip, wp, fptr = out if out else (self.idx.data_ptr(), self.wts.data_ptr(), self.fptr)
+        rc = self.L.mrb_per_sample(self.h, self.batch, float(self.betas[i]), self.uniforms.data_ptr() + i * self.batch * 4,
+                                   ip, wp, fptr, sp or self.sp)
+        if rc:
+            self._lib.check(rc)
+
+    def loop(self, i, sp=None):
+        self.sample(i, sp)
+        self.L.mrb_per_update(self.h, self.idx.data_ptr(), self.upr[i % 64].data_ptr(), self.upd, sp or self.sp)
+        self.L.mrb_per_push(self.h, self.sptr, self.ins_n, self.ins_pr, sp or self.sp)
+
+
+def bench_per(a):
+    """Configs 1, 3, 4, 5 (prioritized buffers)."""
+    import torch
+
+    r = PerRun(a, torch)
+    K, W, batch = r.K, r.W, r.batch
+    defaults = not (a.capacity or a.row_split or a.sample_path or a.graph)
+    step = r.loop if r.loop_step else r.sample
+    for i in range(W):
+        step(i)
+    torch.cuda.synchronize()
+
+    ev0, ev1 = events(torch)
+    graph = None
+    if a.graph:
+        if r.loop_step:
+            raise SystemExit("bench.py: --graph captures sample() steps; the config-1 loop advances host-side counters")
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            sp_side = C.c_void_p(side.cuda_stream)
+            graph.capture_begin()
+            for i in range(W, W + K):
+                r.sample(i, sp_side)
+            graph.capture_end()
+        torch.cuda.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record(r.stream)
+    if graph is not None:
+        graph.replay()
+    else:
+        for i in range(W, W + K):
+            step(i)
+    ev1.record(r.stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_s = ev0.elapsed_time(ev1) * 1e-3
+    flags = r.buf.check()
+
+    row_bytes = sum(r.buf._layout.bytes)
+    levels = max(1, (r.capacity - 1).bit_length())
+    # the library's own choice (mrb_per_sample): the LDS-top kernel for many narrow rows, else the wide-row kernel
+    lds_path = a.sample_path == 2 or (a.sample_path == 0 and batch >= 8192 and max(r.buf._layout.bytes) <= 256)
+    kernel_name = "k_per_sample_lds" if lds_path else "k_per_sample_wide"
+    if a.workload == "c3":
+        # rows read + rows written + index (8) + weight (4): the gather-bound headline figure
+        algo_bytes, formula = batch * (2 * row_bytes + 12), "batch * (2 * row_bytes + 12)"
+    else:
+        # narrow rows: the descent's own bytes count too (one left-child sum per level and the leaf)
+        algo_bytes = batch * (2 * row_bytes + 12 + 4 * levels + 4)
+        formula = "batch * (2 * row_bytes + 12 + 4 * levels + 4), levels = %d" % levels
+    if r.loop_step:
+        metric, value, unit = "config-1 loop steps/sec (sample 64 + update_priorities 64 + insert 1)", K / wall, "steps/s"
+    else:
+        metric = ("sampled transitions/sec (sample+IS+gather) at cap 1M; HBM GB/s vs peak" if a.workload == "c3" else
+                  "sampled transitions/sec (sample+IS+gather), %s" % r.desc.split(":")[0])
+        value, unit = K * batch / wall, "transitions/s"
+    out = {
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": wall * 1e3 / K, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": r.desc, "capacity": r.capacity, "batch": batch, "row_bytes": row_bytes, "alpha": 0.6,
+                   "beta": "0.4->1.0" if a.workload == "c3" else "0.4",
+                   "launch": "hip graph replay" if a.graph else "eager C-ABI calls, one stream, in order",
+                   "prefill_s": round(r.fill_s, 2), "device_flags": flags},
+    }
+    if r.loop_step:
+        # the sample kernel's share of a loop step is timed on its own; the loop itself is launch-bound
+        for i in range(20):
+            r.sample(i)
+        torch.cuda.synchronize()
+        e0, e1 = events(torch)
+        e0.record(r.stream)
+        for i in range(K):
+            r.sample(W + i)
+        e1.record(r.stream)
+        torch.cuda.synchronize()
+        out["roofline"] = roofline(kernel_name, algo_bytes, e0.elapsed_time(e1) * 1e-3 / K, wall / K, a.workload, formula, defaults)
+        out["roofline"]["note"] = ("the loop is bound by kernel launches, not by bytes: frac is the sample kernel alone, "
+                                   "frac_wall prices the sample's bytes against a whole loop step")
+    else:
+        out["roofline"] = roofline(kernel_name, algo_bytes, dev_s / K, wall / K, a.workload, formula, defaults)
+    if not a.no_extras:
+        out["extras"] = per_extras(a, torch, r)
+    if a.no_cpu_baseline:
+        out["cpu_baseline"] = None
+    elif r.loop_step:
+        out["cpu_baseline"] = cpu_baseline_loop(a.workload, r.shapes, r.np_dtypes, batch, r.upd_n, r.ins_n, r.seed)
+    else:
+        out["cpu_baseline"] = cpu_baseline_sample(a.workload, r.shapes, r.np_dtypes, batch, r.seed)
+    r.buf.destroy()
+    print(json.dumps(out))
+    return 0
+
+
+def per_extras(a, torch, r):
+    """Untimed side figures: the other operations of the config's step, the same sample steps replayed from
+    a HIP graph, and issued round robin on several streams (independent calls, one output set per stream)."""
+    L, h, sp, K, W, batch = r.L, r.h, r.sp, r.K, r.W, r.batch
+    extras = {}
+    n_it = max(20, min(300, K))
+
+    def timed(fn, n=n_it):
+        for i in range(10):
+            fn(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    uidx = torch.from_numpy(r.rng.integers(0, r.capacity, (64, r.upd_n))).cuda()
+    extras["updates_per_s"] = r.upd_n / timed(
+        lambda i: L.mrb_per_update(h, uidx[i % 64].data_ptr(), r.upr[i % 64].data_ptr(), r.upd_n, sp))
+    extras["inserts_per_s"] = r.ins_n / timed(lambda i: L.mrb_per_push(h, r.sptr, r.ins_n, r.ins_pr, sp))
+    extras["loop_steps_per_s"] = 1.0 / timed(lambda i: r.loop(W + i % K))
+    if not r.loop_step:
+        extras["sample_us_per_call"] = timed(lambda i: r.sample(W + i % K)) * 1e6
+        # the same calls replayed from one captured HIP graph (a chain: every call ordered after the one before)
+        n_g = min(K, 200)
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            sps = C.c_void_p(side.cuda_stream)
+            graph.capture_begin()
+            for i in range(n_g):
+                r.sample(W + i, sps)
+            graph.capture_end()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        extras["graph_replay_us_per_call"] = (time.perf_counter() - t0) / (5 * n_g) * 1e6
+        del graph
+        # independent sample calls issued round robin on several streams, each stream with its own outputs:
+        # what a prefetching caller sustains when calls need not wait for one another
+        sets = []
+        for _ in range(4):
+            st = torch.cuda.Stream()
+            f = r.buf._layout.empty(batch, r.buf._dev)
+            sets.append((C.c_void_p(st.cuda_stream), (torch.empty(batch, dtype=torch.int64, device="cuda"),
+                                                      torch.empty(batch, dtype=torch.float32, device="cuda"), f), st))
+        torch.cuda.synchronize()
+        pipelined = {}
+        for ns in (2, 4):
+            def rr(i):
+                s_, (i_, w_, f_), _ = sets[i % ns]
+                r.sample(W + i % K, s_, (i_.data_ptr(), w_.data_ptr(), r.pointers(f_)))
+            pipelined[str(ns)] = timed(rr, max(n_it, 200)) * 1e6
+        extras["streams_round_robin_us_per_call"] = pipelined
+        row_bytes = sum(r.buf._layout.bytes)
+        extras["streams_round_robin_frac_of_peak"] = (batch * (2 * row_bytes + 12) / (min(pipelined.values()) * 1e-6)
+                                                      / 1e9 / HBM_PEAK_GBS)
+    r.buf.check()
+    return extras
 
 
 def bench_uniform(a):
@@ -170,7 +484,7 @@ def bench_uniform(a):
     for i in range(W):
         _lib.check(L.mrb_urb_gather(buf._h, ibase + i * batch * 8, batch, optr, sp))
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0, ev1 = events(torch)
     t0 = time.perf_counter()
     ev0.record()
     for i in range(W, W + K):
@@ -188,9 +502,7 @@ def bench_uniform(a):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "config 2: SAC-shaped UniformReplayBuffer, capacity %d, 165 B rows, batch 256, "
                                "host-drawn indices" % capacity, "row_bytes": row_bytes},
-        "roofline": {"bound": "hbm", "achieved": algo / kern_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "k_rows_gather",
-                     "algorithmic_bytes_per_launch": algo, "avg_launch_us": kern_s * 1e6},
+        "roofline": roofline("k_rows_gather", algo, kern_s, wall / K, "c2", "batch * (2 * row_bytes + 8)"),
         "extras": {"inserts_per_s": capacity / ins_s, "insert_chunk": chunk},
         "cpu_baseline": None,
     }
@@ -250,7 +562,7 @@ def bench_reservoir(a):
     for _ in range(W):
         _lib.check(L.mrb_res_sample(buf._h, batch, None, optr, sp))
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0, ev1 = events(torch)
     t0 = time.perf_counter()
     ev0.record()
     for _ in range(K):
@@ -267,9 +579,7 @@ def bench_reservoir(a):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "ReservoirReplayBuffer, capacity %d, 92 B rows, push 4096 per call past capacity, "
                                "sample 256 per call" % capacity, "row_bytes": row_bytes},
-        "roofline": {"bound": "hbm", "achieved": algo / kern_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "k_rows_gather",
-                     "algorithmic_bytes_per_launch": algo, "avg_launch_us": kern_s * 1e6},
+        "roofline": roofline("k_rows_gather", algo, kern_s, wall / K, "res", "batch * 2 * row_bytes"),
         "extras": {"pushes_per_s": n_push * chunk / push_s, "push_chunk": chunk},
         "cpu_baseline": None,
     }
@@ -324,7 +634,7 @@ def bench_discounted_return(a):
     for _ in range(W):
         step()
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0, ev1 = events(torch)
     t0 = time.perf_counter()
     ev0.record()
     for _ in range(K):
@@ -339,10 +649,8 @@ def bench_discounted_return(a):
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": wall * 1e3 / K, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "DiscountedReturn, reward [1000, %d, 1] f32, gamma 0.99, 1 %% dones" % b},
-        "roofline": {"bound": "hbm", "achieved": algo / kern_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "k_discounted_return_tiled" if b * inner <= 16384 else "k_discounted_return",
-                     "algorithmic_bytes_per_launch": algo, "avg_launch_us": kern_s * 1e6},
+        "roofline": roofline("k_discounted_return_tiled" if b * inner <= 16384 else "k_discounted_return", algo, kern_s,
+                             wall / K, "dr", "T * B * (4 read + 4 written) + T * B done flags"),
         "cpu_baseline": None,
     }
     if not a.no_cpu_baseline:
@@ -368,10 +676,6 @@ def main():
         return 2
     import torch
 
-    from mindrl_amd import _lib
-    from mindrl_amd.core import PriorityReplayBuffer
-    from mindrl_amd.core._rows import pointers
-
     assert torch.cuda.is_available(), "bench.py needs a HIP device"
     torch.cuda.set_device(0)
     if a.workload == "c2":
@@ -380,175 +684,7 @@ def main():
         return bench_reservoir(a)
     if a.workload == "dr":
         return bench_discounted_return(a)
-    capacity, batch, shapes, np_dtypes, upd_n, ins_n, desc = WORKLOADS[a.workload]
-    if a.capacity:
-        capacity = a.capacity
-        desc += " [capacity overridden to %d]" % capacity
-    seed = 1000 + int(a.workload[1])
-    t_types = [getattr(torch, d) for d in np_dtypes]
-    buf = PriorityReplayBuffer(0.6, capacity, batch, shapes, t_types, seed0=seed)
-    buf.set_option("row_split", a.row_split)
-    buf.set_option("sample_path", a.sample_path)
-    t0 = time.perf_counter()
-    fill_per(buf, torch, capacity, shapes, np_dtypes, seed)
-    fill_s = time.perf_counter() - t0
-
-    K, W = a.steps, a.warmup
-    rng = np.random.default_rng(seed + 1)
-    uniforms = torch.from_numpy(rng.random((K + W, batch)).astype(np.float32)).cuda()
-    betas = np.linspace(0.4, 1.0, K + W).astype(np.float32)
-    idx = torch.empty(batch, dtype=torch.int64, device="cuda")
-    wts = torch.empty(batch, dtype=torch.float32, device="cuda")
-    fields = buf._layout.empty(batch, buf._dev)
-    fptr = pointers(fields)
-    L = _lib.lib()
-    stream = torch.cuda.current_stream()
-    sp = C.c_void_p(stream.cuda_stream)
-    h = buf._h
-    ubase, ustride = uniforms.data_ptr(), batch * 4
-    ip, wp = idx.data_ptr(), wts.data_ptr()
-
-    def step(i):
-        rc = L.mrb_per_sample(h, batch, float(betas[i]), ubase + i * ustride, ip, wp, fptr, sp)
-        if rc:
-            _lib.check(rc)
-
-    for i in range(W):
-        step(i)
-    torch.cuda.synchronize()
-
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    graph = None
-    if a.graph:
-        graph = torch.cuda.CUDAGraph()
-        side = torch.cuda.Stream()
-        with torch.cuda.stream(side):
-            sp_side = C.c_void_p(side.cuda_stream)
-            graph.capture_begin()
-            for i in range(W, W + K):
-                rc = L.mrb_per_sample(h, batch, float(betas[i]), ubase + i * ustride, ip, wp, fptr, sp_side)
-                if rc:
-                    _lib.check(rc)
-            graph.capture_end()
-        torch.cuda.synchronize()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ev0.record(stream)
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(W, W + K):
-            step(i)
-    ev1.record(stream)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    dev_ms = ev0.elapsed_time(ev1)
-    flags = buf.check()
-
-    # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this very command, scaled by what the
-    # same counters read for the ring-append copy kernel; only valid for
-    # the default workload and library defaults.
-    traffic = 33.6e6 if (a.workload == "c3" and not a.capacity and not a.row_split and not a.sample_path) else None
-    row_bytes = sum(buf._layout.bytes)
-    algo_bytes = batch * (2 * row_bytes + 12)  # rows read + rows written + index (8) + weight (4)
-    kern_s = dev_ms * 1e-3 / K
-    achieved = algo_bytes / kern_s / 1e9
-    # the library's own choice (mrb_per_sample): the LDS-top kernel for many narrow rows, else the wide-row kernel
-    lds_path = a.sample_path == 2 or (a.sample_path == 0 and batch >= 8192 and max(buf._layout.bytes) <= 256)
-    kernel_name = "k_per_sample_lds" if lds_path else "k_per_sample_wide"
-    out = {
-        "metric": "sampled transitions/sec (sample+IS+gather) at cap 1M; HBM GB/s vs peak",
-        "value": K * batch / wall,
-        "unit": "transitions/s",
-        "n_gpus": 1,
-        "steps": K,
-        "warmup": W,
-        "ms_per_step": wall * 1e3 / K,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "u8",
-        "data": "synthetic",
-        "config": {"workload": desc, "capacity": capacity, "batch": batch, "row_bytes": row_bytes,
-                   "alpha": 0.6, "beta": "0.4->1.0", "launch": "hip graph replay" if a.graph else "eager C-ABI calls",
-                   "prefill_s": round(fill_s, 2), "device_flags": flags},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": kernel_name, "algorithmic_bytes_per_launch": algo_bytes,
-                     "avg_launch_us": kern_s * 1e6},
-    }
-
-    if a.extras:
-        extras = {}
-        uidx = torch.from_numpy(rng.integers(0, capacity, (64, upd_n))).cuda()
-        upr = torch.from_numpy((np.abs(rng.normal(size=(64, upd_n))) + 1e-6).astype(np.float32)).cuda()
-        n_it = 300
-        for i in range(20):
-            L.mrb_per_update(h, uidx[i % 64].data_ptr(), upr[i % 64].data_ptr(), upd_n, sp)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(n_it):
-            L.mrb_per_update(h, uidx[i % 64].data_ptr(), upr[i % 64].data_ptr(), upd_n, sp)
-        torch.cuda.synchronize()
-        extras["updates_per_s"] = n_it * upd_n / (time.perf_counter() - t0)
-        src = [f[:ins_n].contiguous() if f.shape[0] >= ins_n else f.repeat((ins_n + f.shape[0] - 1) // f.shape[0],
-               *([1] * (f.dim() - 1)))[:ins_n].contiguous() for f in fields]
-        sptr = pointers(src)
-        # config 4 inserts its rows at actor-side priorities |N(0,1)| + eps; the others at the running max
-        ins_prio = (torch.randn(ins_n, device="cuda").abs() + 1e-6) if a.workload == "c4" else None
-        ins_pr = ins_prio.data_ptr() if ins_prio is not None else None
-        for i in range(20):
-            L.mrb_per_push(h, sptr, ins_n, ins_pr, sp)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(n_it):
-            L.mrb_per_push(h, sptr, ins_n, ins_pr, sp)
-        torch.cuda.synchronize()
-        extras["inserts_per_s"] = n_it * ins_n / (time.perf_counter() - t0)
-        t0 = time.perf_counter()
-        for i in range(n_it):
-            step(W + (i % K))
-            L.mrb_per_update(h, ip, upr[i % 64].data_ptr(), min(upd_n, batch), sp)
-            L.mrb_per_push(h, sptr, ins_n, ins_pr, sp)
-        torch.cuda.synchronize()
-        extras["loop_steps_per_s"] = n_it / (time.perf_counter() - t0)
-        # Reference points for the sample kernel on the same storage and output buffers: what a copy of the same
-        # number of bytes costs per launch, with and without the random row addresses, and without any tree work.
-        big = max(range(len(fields)), key=lambda i: fields[i].numel() * fields[i].element_size())
-        store = buf.storage()[big]
-        dst = fields[big]
-        n_it = 500
-
-        def per_launch(fn):
-            for _ in range(20):
-                fn()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(n_it):
-                fn()
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) * 1e3 / n_it
-
-        step(W)
-        torch.cuda.synchronize()
-        sampled = idx.clone()  # a real set of sampled slots
-        extras["ceiling_contiguous_copy_us"] = per_launch(lambda: dst.copy_(store[:batch]))
-        extras["ceiling_index_select_us"] = per_launch(lambda: torch.index_select(store, 0, sampled, out=dst))
-        extras["ceiling_bytes"] = 2 * dst.numel() * dst.element_size()
-        # the library's own gather at given slots (no tree work): the optional next_obs dereference of config 3
-        L.mrb_per_gather(h, sampled.data_ptr(), batch, fptr, sp)
-        extras["gather_at_given_slots_us"] = per_launch(lambda: L.mrb_per_gather(h, sampled.data_ptr(), batch, fptr, sp))
-        out["extras"] = extras
-
-    if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(a.workload, shapes, np_dtypes, batch, seed)
-    else:
-        out["cpu_baseline"] = None
-    buf.destroy()
-    print(json.dumps(out))
-    return 0
+    return bench_per(a)
 
 
 if __name__ == "__main__":
