@@ -21,10 +21,16 @@
  *     uniforms, outputs) are DEVICE pointers; the caller owns them and keeps
  *     them alive until the work enqueued on `stream` has completed.
  *   - `stream` is a hipStream_t (NULL = the null stream). All device work is
- *     enqueued on it in program order; only create/destroy/state/check/
- *     export_tree synchronise. Calls on one handle must be serialised by the
- *     caller (the reference orders them with side_effect_io,
- *     priority_replay_buffer.py:67-76); different handles are independent.
+ *     enqueued on it in program order. Only *_create, *_destroy, mrb_per_state
+ *     (when the running max is asked for), *_check and mrb_per_export_tree wait
+ *     for the device; only *_create allocates device memory, with one exception:
+ *     an mrb_per_update of more entries than the buffer has rows and than any
+ *     earlier call had enlarges its scratch (hipMalloc; nothing is freed before
+ *     *_destroy). Calls that change one handle must be serialised by the caller
+ *     (the reference orders them with side_effect_io,
+ *     priority_replay_buffer.py:67-76); sample / gather calls on one handle may
+ *     run at the same time on different streams as long as no call that changes
+ *     the handle is in flight; different handles are independent.
  *   - storage is structure-of-arrays: field i is one [capacity, field_bytes[i]]
  *     byte matrix (reference layout: uniform_replay_buffer.py:26-47).
  */

@@ -905,11 +905,12 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, 
         rc = sample_wide(b->rows, a, t, s);
         if (rc) return rc;
     } else {
-        int levels = b->lds_levels > 0 ? (int)b->lds_levels : 12;
+        int levels = b->lds_levels > 0 ? (int)b->lds_levels : 9;
         if (levels > b->depth) levels = b->depth;
         const uint32_t ntop = (2u << levels) < 4 ? 4 : (2u << levels);
         const size_t lds = ntop * sizeof(float) + kWG * sizeof(int64_t);
-        hipLaunchKernelGGL(k_per_sample_lds, dim3((uint32_t)((batch + kWG - 1) / kWG)), dim3(kWG), lds, s, a, t, levels);
+        hipLaunchKernelGGL(k_per_sample_lds, dim3((uint32_t)((batch + kWG - 1) / kWG)), dim3(kLdsWG), lds, s, a.sum, a.uniforms,
+                           a.mn, a.depth, levels, (int)batch, beta, a.seed, a.calls, a, t);
         LAUNCH_CHECK("k_per_sample_lds");
     }
     if (!uniforms) b->calls += 1;
@@ -1127,8 +1128,8 @@ int mrb_per_load_leaves(int64_t h, const float* leaves, int64_t n, float max_pri
     fill_zero(b->sum, nodes * sizeof(float), s);
     hipLaunchKernelGGL(k_fill_f32, dim3(grid_for(nodes)), dim3(kWG), 0, s, b->mn, FLT_MAX, (uint64_t)nodes);
     LAUNCH_CHECK("k_fill_f32");
-    HIP_TRY(hipMemcpyAsync(b->maxp, &max_priority, sizeof(float), hipMemcpyHostToDevice, s));
-    HIP_TRY(hipStreamSynchronize(s));  // max_priority lives on this stack frame
+    hipLaunchKernelGGL(k_fill_f32, dim3(1), dim3(kWG), 0, s, b->maxp, max_priority, (uint64_t)1);
+    LAUNCH_CHECK("k_fill_f32");
     if (n == 0) return MRB_OK;
     int rc = next_epoch(*b, s);
     if (rc) return rc;

@@ -280,6 +280,19 @@ __device__ __forceinline__ uint32_t walk16(f32x16 v, float& mass, float& picked)
     return p;
 }
 
+// Five levels in one thread: `lo`, `hi` hold the 32 descendants five levels below a node (one
+// aligned 128-byte line); the first step compares with the pairwise sum of the lower sixteen, the
+// rest is walk16 on the half entered.
+__device__ __forceinline__ uint32_t walk32(f32x16 lo, f32x16 hi, float& mass, float& picked) {
+    const f32x8 q8 = __builtin_shufflevector(lo, lo, 0, 2, 4, 6, 8, 10, 12, 14) +
+                     __builtin_shufflevector(lo, lo, 1, 3, 5, 7, 9, 11, 13, 15);
+    const f32x4 q4 = __builtin_shufflevector(q8, q8, 0, 2, 4, 6) + __builtin_shufflevector(q8, q8, 1, 3, 5, 7);
+    const float left = (q4.x + q4.y) + (q4.z + q4.w);
+    const bool r = !(mass <= left);
+    mass = r ? mass - left : mass;
+    return (r ? 16u : 0u) + walk16(r ? hi : lo, mass, picked);
+}
+
 // Number of round trips and the levels taken by each for a tree of `depth` levels.
 __device__ __forceinline__ int group_count(int depth) { return (depth + kGroupMaxLevels - 1) / kGroupMaxLevels; }
 __device__ __forceinline__ int group_levels(int depth, int count, int i) {

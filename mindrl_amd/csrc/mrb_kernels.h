@@ -10,7 +10,17 @@
 
 namespace mrb {
 
+#ifdef MRB_PROBE
+__device__ uint64_t g_probe[16384 * 16];
+#define MRB_TS(var) const uint64_t var = wall_clock64()
+#define MRB_TS_OUT(slot, var) do { if ((threadIdx.x & 63) == 0 && (threadIdx.x < 64 || (slot) >= 0)) g_probe[(blockIdx.x * 16 + (slot)) & (16384 * 16 - 1)] = (var); } while (0)
+#else
+#define MRB_TS(var) do { } while (0)
+#define MRB_TS_OUT(slot, var) do { } while (0)
+#endif
+
 constexpr int kWG = 256;          // threads per workgroup of the row and sample kernels
+constexpr int kLdsWG = kWG + 64;  // the LDS-top sample kernel: kWG strata and a helper wave
 constexpr int kRoundLevels = 8;   // most tree levels rebuilt by one round of k_tree_update
 constexpr int kBlockNodes = 256;  // nodes per wave tile in k_tree_update (float4 per lane)
 constexpr int kTopMaxDepth = 12;  // deepest level k_tree_top normally starts from (4096 nodes)
@@ -64,6 +74,35 @@ __device__ __forceinline__ void copy_granule(gbyte* dst, const gbyte* src, uint3
 }
 
 using granule_t = __attribute__((ext_vector_type(4))) uint32_t;  // one 16-byte copy granule
+
+// One granule of 1 << vl bytes held between its load and its store. vl is wave-uniform; every size
+// has its own member so that no value of one load is merged with another's (a merge would make the
+// compiler wait for the load right away).
+struct AnyGranule {
+    granule_t q;
+    uint64_t d;
+    uint32_t w;
+    uint16_t h;
+    uint8_t b;
+    __device__ __forceinline__ void load(const gbyte* src, uint32_t vl) {
+        switch (vl) {
+            case 4: q = *(const __attribute__((address_space(1))) granule_t*)src; break;
+            case 3: d = *(const __attribute__((address_space(1))) uint64_t*)src; break;
+            case 2: w = *(const __attribute__((address_space(1))) uint32_t*)src; break;
+            case 1: h = *(const __attribute__((address_space(1))) uint16_t*)src; break;
+            default: b = *src; break;
+        }
+    }
+    __device__ __forceinline__ void store(gbyte* dst, uint32_t vl) const {
+        switch (vl) {
+            case 4: *(__attribute__((address_space(1))) granule_t*)dst = q; break;
+            case 3: *(__attribute__((address_space(1))) uint64_t*)dst = d; break;
+            case 2: *(__attribute__((address_space(1))) uint32_t*)dst = w; break;
+            case 1: *(__attribute__((address_space(1))) uint16_t*)dst = h; break;
+            default: *dst = b; break;
+        }
+    }
+};
 
 __device__ __forceinline__ int field_of(const IoTable& t, uint64_t w) {
     int f = 0;
@@ -299,15 +338,6 @@ struct SampleTail {
     int64_t size;
     float beta;
 };
-
-#ifdef MRB_PROBE
-__device__ uint64_t g_probe[16384 * 16];
-#define MRB_TS(var) const uint64_t var = wall_clock64()
-#define MRB_TS_OUT(slot, var) do { if ((threadIdx.x & 63) == 0) g_probe[(blockIdx.x * 16 + (slot)) & (16384 * 16 - 1)] = (var); } while (0)
-#else
-#define MRB_TS(var) do { } while (0)
-#define MRB_TS_OUT(slot, var) do { } while (0)
-#endif
 
 constexpr int kCopyWaves = 4;
 constexpr int kCopyThreads = 64 * kCopyWaves;
@@ -720,22 +750,46 @@ __global__ __launch_bounds__(kWideWG) void k_rows_gather_wide(const int64_t* __r
 // the levels below; then the workgroup gathers its 256 rows with coalesced
 // writes. Same outputs, bit for bit, as k_per_sample_wide.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kWG) void k_per_sample_lds(SampleArgs a, IoTable t, int lds_levels) {
+// sum .. calls repeat members of `a` as plain leading parameters: those are preloaded into scalar
+// registers, so the staging loads go out when the wave starts instead of a round trip to the
+// kernel-argument segment later.
+__global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restrict__ sum, const float* __restrict__ uniforms,
+                                                        const float* __restrict__ mn, int depth, int lds_levels,
+                                                        int batch, float beta, uint64_t seed, uint64_t calls,
+                                                        SampleArgs a, IoTable t) {
     extern __shared__ float s_top[];  // [2 << lds_levels] floats, then kWG int64 slots
+    __shared__ float s_max_w;
     const uint32_t ntop = 2u << lds_levels;
     int64_t* s_slot = reinterpret_cast<int64_t*>(s_top + (ntop < 4 ? 4 : ntop));
-    if (ntop >= 4) {
-        for (uint32_t i = threadIdx.x * 4; i < ntop; i += kWG * 4)
-            *reinterpret_cast<float4*>(s_top + i) = *reinterpret_cast<const float4*>(a.sum + i);
-    } else if (threadIdx.x < ntop) {
-        s_top[threadIdx.x] = a.sum[threadIdx.x];
-    }
-    __syncthreads();
+    MRB_TS(ts0);
     const int64_t k0 = (int64_t)blockIdx.x * kWG;
     const int64_t k = k0 + threadIdx.x;
-    if (k < a.batch) {
+    if (threadIdx.x >= kWG) {
+        // The helper wave: the weights' common denominator (pmin / total * size)^-beta, once per
+        // workgroup, off the strata's path (two loads and a power: as long as staging the top).
+        __syncthreads();
+        if (threadIdx.x == kWG) s_max_w = powf_det(mn[1] / sum[1] * (float)a.size, -beta);
+        __syncthreads();
+        return;
+    }
+    // the stratum's draw is requested together with the top of the tree
+    float u = 0.0f;
+    if (k < batch && uniforms) u = uniforms[k];
+    if (ntop >= 4) {
+        for (uint32_t i = threadIdx.x * 4; i < ntop; i += kWG * 4)
+            *reinterpret_cast<float4*>(s_top + i) = *reinterpret_cast<const float4*>(sum + i);
+    } else if (threadIdx.x < ntop) {
+        s_top[threadIdx.x] = sum[threadIdx.x];
+    }
+    __syncthreads();
+    MRB_TS(ts1);
+    constexpr int kOwn = 4;  // leading fields whose row is one granule: every thread copies its own stratum's
+    AnyGranule own[kOwn];
+    float weight = 0.0f;
+    if (k < batch) {
         const float total = s_top[1];
-        float mass = stratum_mass(a, total, k);
+        if (!uniforms) u = rng_uniform(seed, calls, (uint64_t)k);
+        float mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
         uint32_t node = 1;
         int d = 0;
         for (; d < lds_levels; ++d) {
@@ -747,65 +801,133 @@ __global__ __launch_bounds__(kWG) void k_per_sample_lds(SampleArgs a, IoTable t,
                 node = 2 * node + 1;
             }
         }
-        // Below the staged levels every dependent load brings several levels at once: the 16
-        // (or 8) descendants of `node` four (three) levels down are 64 (32) contiguous, aligned
-        // bytes; the levels between are rebuilt with the additions the tree was built with.
-        float picked = a.depth <= lds_levels ? s_top[node] : 0.0f;
-        for (; d + 4 <= a.depth; d += 4) {
-            const f32x4* src = reinterpret_cast<const f32x4*>(a.sum + ((uint64_t)node << 4));
-            const f32x4 t0 = src[0], t1 = src[1], t2 = src[2], t3 = src[3];
-            const f32x16 v = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
-                                                     __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2,
-                                                     3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
-            node = (node << 4) + walk16(v, mass, picked);
-        }
-        for (; d + 3 <= a.depth; d += 3) {
-            const float4* src = reinterpret_cast<const float4*>(a.sum + ((uint64_t)node << 3));
-            const float4 lo = src[0], hi = src[1];
-            const float a0 = lo.x + lo.y, a1 = lo.z + lo.w, a2 = hi.x + hi.y;
-            const float b0 = a0 + a1;
-            uint32_t p = 0;
-            if (!(mass <= b0)) {
-                mass -= b0;
-                p = 4;
-            }
-            const float left1 = p ? a2 : a0;
-            if (!(mass <= left1)) {
-                mass -= left1;
-                p += 2;
-            }
-            const float n0 = p == 0 ? lo.x : p == 2 ? lo.z : p == 4 ? hi.x : hi.z;
-            const float n1 = p == 0 ? lo.y : p == 2 ? lo.w : p == 4 ? hi.y : hi.w;
-            if (!(mass <= n0)) {
-                mass -= n0;
-                p += 1;
-                picked = n1;
+        // Below the staged levels every dependent load brings up to five levels at once: the 32 (16, 8,
+        // 4, 2) descendants of `node` five (four, ... one) levels down are 128 (64, ... 8) contiguous,
+        // aligned bytes - a whole cache line in the first case; the levels between are rebuilt with
+        // the additions the tree was built with. The remaining levels are taken five at a time, except
+        // that seven are split 4 + 3 (5 + 1 + 1 would be a load more).
+        float picked = depth <= lds_levels ? s_top[node] : 0.0f;
+#ifdef MRB_PROBE
+        asm volatile("" ::"v"(node), "v"(mass));
+#endif
+        MRB_TS(ts2);
+        while (d < depth) {  // wave-uniform
+            const int rest = depth - d;
+            const int g = rest >= 5 ? (rest == 7 ? 4 : 5) : rest;
+            if (g == 5) {
+                const f32x4* src = reinterpret_cast<const f32x4*>(sum + ((uint64_t)node << 5));
+                const f32x4 t0 = src[0], t1 = src[1], t2 = src[2], t3 = src[3], t4 = src[4], t5 = src[5], t6 = src[6], t7 = src[7];
+                const f32x16 lo = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
+                                                          __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
+                                                          2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+                const f32x16 hi = __builtin_shufflevector(__builtin_shufflevector(t4, t5, 0, 1, 2, 3, 4, 5, 6, 7),
+                                                          __builtin_shufflevector(t6, t7, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
+                                                          2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+                node = (node << 5) + walk32(lo, hi, mass, picked);
+            } else if (g == 4) {
+                const f32x4* src = reinterpret_cast<const f32x4*>(sum + ((uint64_t)node << 4));
+                const f32x4 t0 = src[0], t1 = src[1], t2 = src[2], t3 = src[3];
+                const f32x16 v = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
+                                                         __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
+                                                         2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+                node = (node << 4) + walk16(v, mass, picked);
+            } else if (g == 3) {
+                const float4* src = reinterpret_cast<const float4*>(sum + ((uint64_t)node << 3));
+                const float4 lo = src[0], hi = src[1];
+                const float a0 = lo.x + lo.y, a1 = lo.z + lo.w, a2 = hi.x + hi.y;
+                const float b0 = a0 + a1;
+                uint32_t p = 0;
+                if (!(mass <= b0)) {
+                    mass -= b0;
+                    p = 4;
+                }
+                const float left1 = p ? a2 : a0;
+                if (!(mass <= left1)) {
+                    mass -= left1;
+                    p += 2;
+                }
+                const float n0 = p == 0 ? lo.x : p == 2 ? lo.z : p == 4 ? hi.x : hi.z;
+                const float n1 = p == 0 ? lo.y : p == 2 ? lo.w : p == 4 ? hi.y : hi.w;
+                if (!(mass <= n0)) {
+                    mass -= n0;
+                    p += 1;
+                    picked = n1;
+                } else {
+                    picked = n0;
+                }
+                node = (node << 3) + p;
+            } else if (g == 2) {
+                const float4 v = *reinterpret_cast<const float4*>(sum + ((uint64_t)node << 2));
+                const float left = v.x + v.y;
+                uint32_t p = 0;
+                if (!(mass <= left)) {
+                    mass -= left;
+                    p = 2;
+                }
+                const float n0 = p ? v.z : v.x, n1 = p ? v.w : v.y;
+                if (!(mass <= n0)) {
+                    mass -= n0;
+                    p += 1;
+                    picked = n1;
+                } else {
+                    picked = n0;
+                }
+                node = (node << 2) + p;
             } else {
-                picked = n0;
+                const float2 pair = *reinterpret_cast<const float2*>(sum + 2 * (uint64_t)node);
+                if (mass <= pair.x) {
+                    node = 2 * node;
+                    picked = pair.x;
+                } else {
+                    mass -= pair.x;
+                    node = 2 * node + 1;
+                    picked = pair.y;
+                }
             }
-            node = (node << 3) + p;
+            d += g;
         }
-        for (; d < a.depth; ++d) {
-            const float2 pair = *reinterpret_cast<const float2*>(a.sum + 2 * (uint64_t)node);
-            if (mass <= pair.x) {
-                node = 2 * node;
-                picked = pair.x;
-            } else {
-                mass -= pair.x;
-                node = 2 * node + 1;
-                picked = pair.y;
-            }
-        }
-        const int64_t idx = (int64_t)node - a.leaves;
+#ifdef MRB_PROBE
+        asm volatile("" ::"v"(node), "v"(mass));
+#endif
+        MRB_TS(ts3);
+        MRB_TS_OUT(0, ts0);
+        MRB_TS_OUT(1, ts1);
+        MRB_TS_OUT(2, ts2);
+        MRB_TS_OUT(3, ts3);
+        const int64_t idx = (int64_t)node - ((int64_t)1 << depth);
+        const int64_t slot = idx < a.capacity ? idx : a.capacity - 1;
+        // the row's scalar fields are requested now, before the weight's arithmetic and the barrier
+#pragma unroll
+        for (int f = 0; f < kOwn; ++f)
+            if (f < t.nfields && t.units[f] == 1)
+                own[f].load(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f], t.vec_log2[f]);
         a.out_idx[k] = idx;
-        a.out_w[k] = is_weight(picked, total, a.mn[1], (float)a.size, a.beta);
+        weight = powf_det(picked / total * (float)a.size, -beta);
         sample_flags(a, total, idx);
-        s_slot[threadIdx.x] = idx < a.capacity ? idx : a.capacity - 1;
+        s_slot[threadIdx.x] = slot;
     }
+    MRB_TS(ts4);
     __syncthreads();
-    const uint32_t rows = (uint32_t)((a.batch - k0) < kWG ? (a.batch - k0) : kWG);
+    MRB_TS(ts5);
+    MRB_TS_OUT(4, ts4);
+    MRB_TS_OUT(5, ts5);
+    const uint32_t rows = (uint32_t)((batch - k0) < kWG ? (batch - k0) : kWG);
+#ifdef MRB_PROBE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+    MRB_TS(ts6);
+    MRB_TS_OUT(6, ts6);
+    if (k < batch) {
+        a.out_w[k] = weight / s_max_w;
+#pragma unroll
+        for (int f = 0; f < kOwn; ++f)
+            if (f < t.nfields && t.units[f] == 1)
+                own[f].store(as_global(t.io[f]) + (uint64_t)k * t.row_bytes[f], t.vec_log2[f]);
+    }
+    // fields of several granules per row (and fields past the first kOwn): coalesced over the workgroup's rows
     for (int f = 0; f < t.nfields; ++f) {
         const uint32_t units = t.units[f];
+        if (f < kOwn && units == 1) continue;
         const uint32_t vl = t.vec_log2[f];
         const uint64_t work = (uint64_t)rows * units;
         for (uint64_t w = threadIdx.x; w < work; w += kWG) {
@@ -817,6 +939,8 @@ __global__ __launch_bounds__(kWG) void k_per_sample_lds(SampleArgs a, IoTable t,
                          as_global(t.store[f]) + (uint64_t)s_slot[r] * t.row_bytes[f] + off, vl);
         }
     }
+    MRB_TS(ts7);
+    MRB_TS_OUT(7, ts7);
 }
 
 // ---------------------------------------------------------------------------

@@ -110,6 +110,35 @@ def test_kernels_use_no_scratch_memory(tmp_path):
             assert lds == 4096, (name, lds)
 
 
+def test_only_the_documented_entry_points_wait_or_allocate():
+    """include/mrb.h promises that only create / destroy / state / check / export_tree wait for the device and
+    that only create allocates (mrb_per_update may enlarge its scratch, never free it). Checked on the source:
+    the body of every other extern "C" function, and of the helpers they share, names no such call."""
+    src = open(os.path.join(ROOT, "mindrl_amd", "csrc", "mrb.hip")).read()
+    bodies = {}
+    for m in re.finditer(r"^(?:static )?(?:int|void|uint32_t|int64_t|const char\*) (\w+)\([^;{]*\)\s*\{\n(.*?)^\}", src, re.M | re.S):
+        bodies[m.group(1)] = m.group(2)
+    one_liners = {"mrb_last_error", "mrb_backend", "mrb_version"}  # return a constant
+    assert {n for n in bodies if n.startswith("mrb_")} == set(declared_symbols()) - one_liners, sorted(bodies)
+    waits = re.compile(r"hipDeviceSynchronize|hipStreamSynchronize|hipEventSynchronize|hipMemcpy\(")
+    allocs = re.compile(r"hipMalloc|hipFree|hipHostMalloc")
+    may_wait = {"mrb_urb_create", "mrb_per_create", "mrb_res_create", "mrb_urb_destroy", "mrb_per_destroy",
+                "mrb_res_destroy", "mrb_per_state", "mrb_per_export_tree", "read_and_clear_flags", "rows_alloc"}
+    may_alloc = {"mrb_urb_create", "mrb_per_create", "mrb_res_create", "rows_alloc", "mrb_per_update"}
+    for name, body in bodies.items():
+        if name not in may_wait:
+            assert not waits.search(body), "%s waits for the device" % name
+        if name not in may_alloc:
+            assert not allocs.search(body), "%s allocates or frees device memory" % name
+    assert "hipFree" not in bodies["mrb_per_update"]
+    # the check functions wait through this helper and nothing else does
+    users = [n for n, b in bodies.items() if "read_and_clear_flags(" in b]
+    assert sorted(users) == ["mrb_per_check", "mrb_urb_check"]
+    # the allocation-free entry point and the core it shares with mrb_per_update
+    for name in ("mrb_per_update_noalloc", "per_update", "tree_rebuild", "next_epoch", "static_scratch"):
+        assert not allocs.search(bodies[name]) and not waits.search(bodies[name]), name
+
+
 def test_create_replay_buffer_follows_the_reference_config_entry():
     """mindspore_rl/core/msrl.py:270-300: type / number / params-or-(sample_size, capacity) + data_shape / data_type."""
     from mindrl_amd.core import create_replay_buffer
