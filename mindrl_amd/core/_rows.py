@@ -112,6 +112,14 @@ class FieldLayout:
         return list(out)
 
 
+def flat_on_device(x, dtype, dev):
+    """1-D contiguous device tensor of `dtype` holding x; x itself when it already is one (the common case
+    on the training path: no conversion, no copy)."""
+    if isinstance(x, torch.Tensor) and x.dtype == dtype and x.device == dev and x.is_contiguous():
+        return x if x.dim() == 1 else x.reshape(-1)
+    return torch.as_tensor(x).to(device=dev, dtype=dtype).contiguous().reshape(-1)
+
+
 def pointers(tensors):
     return _lib.ptr_array([t.data_ptr() for t in tensors])
 

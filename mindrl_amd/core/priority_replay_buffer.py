@@ -7,8 +7,8 @@ import numpy as np
 import torch
 
 from .. import _lib
-from ._rows import (FieldLayout, device, get_counters, load_fields, pointers, save_fields, set_counters, stream_ptr,
-                    view_of)
+from ._rows import (FieldLayout, device, flat_on_device, get_counters, load_fields, pointers, save_fields,
+                    set_counters, stream_ptr, view_of)
 
 
 class PriorityReplayBuffer:
@@ -24,9 +24,13 @@ class PriorityReplayBuffer:
         sample_size (int): rows returned by sample().
         shapes, types: shape / element type of each tensor of an element.
         seed0, seed1 (int): generator seed; seed1 if non-zero, else seed0, else entropy.
+        output_ring (int): sample() hands out its result tensors from this many preallocated sets in
+            turn (default 4), so a call allocates nothing; a returned batch is overwritten by the
+            `output_ring`-th sample() call after it - clone() what must live longer. 0: fresh tensors
+            on every call.
     """
 
-    def __init__(self, alpha, capacity, sample_size, shapes, types, seed0=0, seed1=0):
+    def __init__(self, alpha, capacity, sample_size, shapes, types, seed0=0, seed1=0, output_ring=4):
         self._dev = device()
         self._layout = FieldLayout(shapes, types)
         self._capacity = int(capacity)
@@ -39,6 +43,21 @@ class PriorityReplayBuffer:
         self._h = h.value
         self._handle = torch.tensor([self._h], dtype=torch.int64)
         self._keep = None
+        self._ring_size = int(output_ring)
+        self._ring, self._ring_at = None, 0  # output sets, built by the first sample()
+
+    def _next_outputs(self):
+        """The next preallocated (indices, weights, fields, field pointer array) set."""
+        if self._ring is None:
+            n = self._sample_size
+            self._ring = []
+            for _ in range(self._ring_size):
+                fields = self._layout.empty(n, self._dev)
+                self._ring.append((torch.empty(n, dtype=torch.int64, device=self._dev),
+                                   torch.empty(n, dtype=torch.float32, device=self._dev), fields, pointers(fields)))
+        out = self._ring[self._ring_at]
+        self._ring_at = (self._ring_at + 1) % self._ring_size
+        return out
 
     # -- reference methods ---------------------------------------------------
     def insert(self, *transition, priorities=None):
@@ -53,7 +72,7 @@ class PriorityReplayBuffer:
         src = self._layout.to_device(transition, self._dev)
         pr = None
         if priorities is not None:
-            pr = torch.as_tensor(priorities).to(device=self._dev, dtype=torch.float32).contiguous().reshape(-1)
+            pr = flat_on_device(priorities, torch.float32, self._dev)
             if pr.numel() != n:
                 raise ValueError("priorities must hold one value per pushed row")
         _lib.check(_lib.lib().mrb_per_push(self._h, pointers(src), n, pr.data_ptr() if pr is not None else None,
@@ -70,30 +89,36 @@ class PriorityReplayBuffer:
 
         Returns (indices int64[B], weights f32[B], *transitions [B, *shape_i]).
         `uniforms` (f32[B] in [0,1)) replaces the buffer's generator, stratum k
-        using uniforms[k]. `out` = (indices, weights, [fields]) reuses output tensors."""
+        using uniforms[k]. `out` = (indices, weights, [fields]) writes into the caller's tensors.
+        Without `out` the result comes from the buffer's ring of preallocated output sets (see
+        `output_ring`): it stays valid until `output_ring` further sample() calls have been made."""
         n = self._sample_size
         u = None
         if uniforms is not None:
-            u = torch.as_tensor(uniforms).to(device=self._dev, dtype=torch.float32).contiguous().reshape(-1)
+            u = flat_on_device(uniforms, torch.float32, self._dev)
             if u.numel() != n:
                 raise ValueError("uniforms must hold sample_size = %d values" % n)
         if out is not None:
             idx, w, fields = out
             fields = self._layout.check_out(fields, n, self._dev)
+            fptr = pointers(fields)
+        elif self._ring_size > 0:
+            idx, w, fields, fptr = self._next_outputs()
         else:
             idx = torch.empty(n, dtype=torch.int64, device=self._dev)
             w = torch.empty(n, dtype=torch.float32, device=self._dev)
             fields = self._layout.empty(n, self._dev)
+            fptr = pointers(fields)
         _lib.check(_lib.lib().mrb_per_sample(self._h, n, float(beta), u.data_ptr() if u is not None else None,
-                                             idx.data_ptr(), w.data_ptr(), pointers(fields), stream_ptr()))
+                                             idx.data_ptr(), w.data_ptr(), fptr, stream_ptr()))
         self._keep = u
         return (idx, w) + tuple(fields)
 
     def update_priorities(self, indices, priorities):
         """leaf[indices[j]] = priorities[j] ** alpha in order, last write wins
         (priority_replay_buffer.py:108-120). Returns the handle tensor."""
-        idx = torch.as_tensor(indices).to(device=self._dev, dtype=torch.int64).contiguous().reshape(-1)
-        pr = torch.as_tensor(priorities).to(device=self._dev, dtype=torch.float32).contiguous().reshape(-1)
+        idx = flat_on_device(indices, torch.int64, self._dev)
+        pr = flat_on_device(priorities, torch.float32, self._dev)
         if idx.numel() != pr.numel():
             raise ValueError("indices and priorities differ in length")
         _lib.check(_lib.lib().mrb_per_update(self._h, idx.data_ptr(), pr.data_ptr(), idx.numel(), stream_ptr()))
@@ -104,7 +129,7 @@ class PriorityReplayBuffer:
         """Rows at the given slots (int64, each in [0, size)): one [n, *shape_i] tensor per field.
         For transitions that store the slot of their successor instead of a copy of it, e.g.
         `next_rows = buf.gather(sampled_next_idx)`."""
-        idx = torch.as_tensor(indices).to(device=self._dev, dtype=torch.int64).contiguous().reshape(-1)
+        idx = flat_on_device(indices, torch.int64, self._dev)
         n = idx.numel()
         dst = self._layout.check_out(out, n, self._dev) if out is not None else self._layout.empty(n, self._dev)
         _lib.check(_lib.lib().mrb_per_gather(self._h, idx.data_ptr(), n, pointers(dst), stream_ptr()))
@@ -123,6 +148,7 @@ class PriorityReplayBuffer:
         """Releases the native buffer (priority_replay_buffer.py:130-138)."""
         if self._h:
             h, self._h = self._h, 0
+            self._ring = None
             _lib.check(_lib.lib().mrb_per_destroy(h))
         return self._handle
 

@@ -113,6 +113,38 @@ def test_config2_sac_shape_full_size(mrb, orc):
     g.destroy()
 
 
+def test_sample_output_ring(mrb, orc):
+    """sample() hands out preallocated output sets in turn: `output_ring` calls return distinct tensors, the
+    next call reuses the first set; output_ring=0 allocates fresh tensors; an explicit out= is written in
+    place. The results are the oracle's in every mode."""
+    shapes, dtypes = [(6,), (1,)], [np.float32, np.int32]
+    rng = np.random.default_rng(12)
+    cap, batch = 500, 16
+    rows = random_rows(rng, cap, shapes, dtypes)
+    for ring in (3, 0):
+        g = mrb.PER(0.6, cap, batch, shapes, torch_types(dtypes), seed0=6, output_ring=ring)
+        c = orc.OraclePER(0.6, cap, shapes, dtypes, seed=6)
+        g.insert(*to_dev(rows)), c.push(rows, cap)
+        outs = []
+        for call in range(4):
+            out = g.sample(0.5)
+            assert_sample_equal(out, c.sample(batch, 0.5), "ring %d call %d" % (ring, call))
+            outs.append(out)
+        ptrs = [o[2].data_ptr() for o in outs]
+        if ring:
+            assert len(set(ptrs[:3])) == 3 and ptrs[3] == ptrs[0]  # the fourth call overwrote the first batch
+            assert torch.equal(outs[3][0], outs[0][0])
+        else:
+            assert len(set(ptrs)) == 4
+        mine = (torch.empty(batch, dtype=torch.int64, device="cuda"), torch.empty(batch, device="cuda"),
+                [torch.empty((batch,) + s, dtype=t, device="cuda") for s, t in zip(shapes, torch_types(dtypes))])
+        u = rng.random(batch).astype(np.float32)
+        back = g.sample(0.5, uniforms=torch.from_numpy(u).cuda(), out=mine)
+        assert back[0].data_ptr() == mine[0].data_ptr() and back[2].data_ptr() == mine[2][0].data_ptr()
+        assert_sample_equal(back, c.sample(batch, 0.5, u), "out=")
+        g.destroy()
+
+
 def test_options_belong_to_one_buffer(mrb, orc):
     """Two prioritized buffers with the same contents, one forced onto the wide-row kernel with three
     workgroups per row, the other onto the LDS-top kernel with 5 staged levels: interleaved calls give the
