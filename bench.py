@@ -446,6 +446,36 @@ def per_extras(a, torch, r):
         row_bytes = sum(r.buf._layout.bytes)
         extras["streams_round_robin_frac_of_peak"] = (batch * (2 * row_bytes + 12) / (min(pipelined.values()) * 1e-6)
                                                       / 1e9 / HBM_PEAK_GBS)
+        # several batches per launch (mrb_per_sample_many): the launch and the descent are paid once for
+        # all of them, which is what a learner that prefetches batches between priority updates can use
+        many = {}
+        for nb in (4, 16):
+            if nb > K + W or nb * batch * row_bytes > (8 << 30):
+                continue
+            fo = r.buf._layout.empty(nb * batch, r.buf._dev)
+            io = torch.empty(nb * batch, dtype=torch.int64, device="cuda")
+            wo = torch.empty(nb * batch, dtype=torch.float32, device="cuda")
+            fp = r.pointers(fo)
+            # every call takes other draws, so no call finds the rows of the one before in the caches
+            nset = (K + W) // nb
+            call = lambda i: L.mrb_per_sample_many(h, nb, batch, float(r.betas[W]),
+                                                   r.uniforms.data_ptr() + (i % nset) * nb * batch * 4,
+                                                   io.data_ptr(), wo.data_ptr(), fp, sp)
+            for i in range(5):
+                call(i)
+            torch.cuda.synchronize()
+            e0, e1 = events(torch)
+            reps = max(10, 200 // nb)
+            e0.record(r.stream)
+            for i in range(reps):
+                call(i)
+            e1.record(r.stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / (reps * nb)
+            many[str(nb)] = {"us_per_batch": us,
+                             "frac_of_peak": batch * (2 * row_bytes + 12) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+            del fo, io, wo
+        extras["sample_many_batches_per_launch"] = many
     r.buf.check()
     return extras
 

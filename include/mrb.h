@@ -136,6 +136,13 @@ int mrb_per_push(int64_t h, const void *const *src_fields, int64_t nrows, const 
  * out_fields[i] = [batch, field_bytes[i]]. */
 int mrb_per_sample(int64_t h, int64_t batch, float beta, const float *uniforms, int64_t *out_indices,
                    float *out_weights, void *const *out_fields, void *stream);
+/* `nbatch` stratified batches in one call: exactly what nbatch successive mrb_per_sample calls with the
+ * same beta would return on an unchanged buffer (batch i uses uniforms[i * batch .. (i + 1) * batch), or
+ * the generator's next call counter), written batch after batch into outputs of nbatch * batch rows.
+ * No counterpart among the reference's primitives: it is for learners that draw several batches per
+ * update of the priorities (prefetching); one launch then amortises the launch and the tree descent. */
+int mrb_per_sample_many(int64_t h, int64_t nbatch, int64_t batch, float beta, const float *uniforms,
+                        int64_t *out_indices, float *out_weights, void *const *out_fields, void *stream);
 /* Replaces PriorityReplayBufferUpdate (priority_replay_buffer.py:71-73,120):
  * leaf[indices[j]] = priorities[j]^alpha for j in order (last write wins on
  * duplicates), every ancestor of a touched leaf recomputed from its final

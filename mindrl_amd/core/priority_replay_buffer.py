@@ -114,6 +114,26 @@ class PriorityReplayBuffer:
         self._keep = u
         return (idx, w) + tuple(fields)
 
+    def sample_many(self, nbatch, beta, uniforms=None):
+        """`nbatch` batches in one launch: what `nbatch` successive sample(beta) calls would return on an
+        unchanged buffer, stacked: (indices int64[nbatch, B], weights f32[nbatch, B], *transitions
+        [nbatch, B, *shape_i]). For learners that draw several batches between priority updates; one launch
+        amortises the launch and the tree descent. `uniforms`: f32[nbatch, B] or None (generator)."""
+        nbatch, n = int(nbatch), self._sample_size
+        u = None
+        if uniforms is not None:
+            u = flat_on_device(uniforms, torch.float32, self._dev)
+            if u.numel() != nbatch * n:
+                raise ValueError("uniforms must hold nbatch * sample_size = %d values" % (nbatch * n))
+        idx = torch.empty((nbatch, n), dtype=torch.int64, device=self._dev)
+        w = torch.empty((nbatch, n), dtype=torch.float32, device=self._dev)
+        fields = [torch.empty((nbatch, n) + s, dtype=d, device=self._dev)
+                  for s, d in zip(self._layout.shapes, self._layout.dtypes)]
+        _lib.check(_lib.lib().mrb_per_sample_many(self._h, nbatch, n, float(beta), u.data_ptr() if u is not None else None,
+                                                  idx.data_ptr(), w.data_ptr(), pointers(fields), stream_ptr()))
+        self._keep = u
+        return (idx, w) + tuple(fields)
+
     def update_priorities(self, indices, priorities):
         """leaf[indices[j]] = priorities[j] ** alpha in order, last write wins
         (priority_replay_buffer.py:108-120). Returns the handle tensor."""

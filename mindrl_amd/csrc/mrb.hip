@@ -147,7 +147,9 @@ int64_t widest_field(const RowStore& r) {
 // kMaxInFlight * kCopyThreads (2048) wide granules, or the buffer's "row_split" option asks for more.
 // Returns the number of granules a copy thread holds (2 or 8) or 0 on error.
 int wide_plan(const RowStore& r, const IoTable& t, int64_t n, WidePlan& plan, dim3& grid) {
+    const uint32_t nbatch = plan.nbatch;
     plan = WidePlan{};
+    plan.nbatch = nbatch;
     for (int i = 0; i < r.nfields; ++i) plan.nwide += r.vec_log2[i] == 4;
     plan.nnarrow = r.nfields - plan.nwide;
     int w = 0, m = plan.nwide;
@@ -189,7 +191,8 @@ template <int kInF, bool kTen, bool kOneWide>
 void launch_sample_wide(dim3 grid, const SampleArgs& a, const WidePlan& plan, hipStream_t s) {
     const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
     hipLaunchKernelGGL((k_per_sample_wide<kInF, kTen, kOneWide>), grid, dim3(kWideWG), 0, s, a.sum, a.uniforms, a.depth,
-                       pack_groups(a.depth), (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, tail, plan);
+                       pack_groups(a.depth) | ((plan.nbatch - 1) << 20), (int)a.batch, (uint32_t)a.capacity, a.seed,
+                       a.calls, tail, plan);
 }
 
 template <int kInF>
@@ -200,10 +203,11 @@ void launch_sample_wide_as(dim3 grid, const SampleArgs& a, const WidePlan& plan,
     else one ? launch_sample_wide<kInF, false, true>(grid, a, plan, s) : launch_sample_wide<kInF, false, false>(grid, a, plan, s);
 }
 
-int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, hipStream_t s) {
+int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, int64_t nbatch, hipStream_t s) {
     WidePlan plan;
     dim3 grid;
-    switch (wide_plan(r, t, a.batch, plan, grid)) {
+    plan.nbatch = (uint32_t)nbatch;
+    switch (wide_plan(r, t, nbatch * a.batch, plan, grid)) {
         case 0: return MRB_EINVAL;
         case 2: launch_sample_wide_as<2>(grid, a, plan, s); break;
         default: launch_sample_wide_as<8>(grid, a, plan, s); break;
@@ -236,6 +240,7 @@ int gather_rows(const RowStore& r, const int64_t* indices, int64_t fixed_slot, i
         const int mode = fixed_slot >= 0 ? kFromFixedSlot : (indices ? kFromIndices : kFromGenerator);
         WidePlan plan;
         dim3 grid;
+        plan.nbatch = 1;
         switch (wide_plan(r, t, n, plan, grid)) {
             case 0: return MRB_EINVAL;
             case 2: launch_gather_wide<2>(grid, indices, mode, count, fixed_slot, seed, calls, out_indices, err, plan, s); break;
@@ -431,6 +436,7 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
             tiles = (uint32_t)((a.first_slot + a.n - 1) / kBlockNodes) - tile_base + 1;
         }
         const PutArgs& put = (r == 0 && ride) ? *ride : none;
+        if (r == 0 && a.inline_election) tiles = (uint32_t)a.n;  // a wave per entry (see k_tree_update)
         hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4 + put.blocks), dim3(kWG), 0, s, a, r, tile_base, put);
         LAUNCH_CHECK("k_tree_update");
     }
@@ -873,15 +879,18 @@ int mrb_per_update_noalloc(int64_t h, const int64_t* indices, const float* prior
     return per_update(*b, indices, priorities, n, powered, static_cast<hipStream_t>(stream));
 }
 
-int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, int64_t* out_indices,
-                   float* out_weights, void* const* out_fields, void* stream) {
-    GET_PER(b, h);
+// `nbatch` batches of `batch` stratified samples each, as nbatch successive mrb_per_sample calls on
+// an unchanged tree would draw them. Outputs hold nbatch * batch rows, batch after batch.
+static int per_sample_impl(Per* b, int64_t nbatch, int64_t batch, float beta, const float* uniforms,
+                           int64_t* out_indices, float* out_weights, void* const* out_fields, hipStream_t s) {
     if (batch <= 0 || batch > (1ll << 24)) return fail(MRB_EINVAL, "batch %lld outside [1, 2^24]", (long long)batch);
+    if (nbatch <= 0 || nbatch > 4096 || nbatch * batch > (1ll << 24))
+        return fail(MRB_EINVAL, "%lld batches of %lld rows exceed one call (at most 4096 batches, 2^24 rows)",
+                    (long long)nbatch, (long long)batch);
     if (!out_indices || !out_weights) return fail(MRB_EINVAL, "out_indices or out_weights is NULL");
     if (b->size <= 0) return fail(MRB_ESTATE, "sample from an empty buffer");
-    hipStream_t s = static_cast<hipStream_t>(stream);
     IoTable t;
-    int rc = make_table(b->rows, out_fields, batch, t);
+    int rc = make_table(b->rows, out_fields, nbatch * batch, t);
     if (rc) return rc;
     SampleArgs a{};
     a.sum = b->sum;
@@ -902,19 +911,43 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, 
     int path = (int)b->sample_path;
     if (path == 0) path = (batch >= 8192 && max_bytes <= 256) ? 2 : 1;
     if (path == 1) {
-        rc = sample_wide(b->rows, a, t, s);
+        rc = sample_wide(b->rows, a, t, nbatch, s);
         if (rc) return rc;
     } else {
+        // the LDS-top kernel takes one batch per launch (its batches are large enough to fill the chip)
         int levels = b->lds_levels > 0 ? (int)b->lds_levels : 9;
         if (levels > b->depth) levels = b->depth;
         const uint32_t ntop = (2u << levels) < 4 ? 4 : (2u << levels);
         const size_t lds = ntop * sizeof(float) + kWG * sizeof(int64_t);
-        hipLaunchKernelGGL(k_per_sample_lds, dim3((uint32_t)((batch + kWG - 1) / kWG)), dim3(kLdsWG), lds, s, a.sum, a.uniforms,
-                           a.mn, a.depth, levels, (int)batch, beta, a.seed, a.calls, a, t);
-        LAUNCH_CHECK("k_per_sample_lds");
+        for (int64_t i = 0; i < nbatch; ++i) {
+            SampleArgs ai = a;
+            IoTable ti = t;
+            ai.uniforms = uniforms ? uniforms + i * batch : nullptr;
+            ai.calls = a.calls + (uint64_t)i;
+            ai.out_idx = out_indices + i * batch;
+            ai.out_w = out_weights + i * batch;
+            for (int f = 0; f < t.nfields; ++f) ti.io[f] = t.io[f] + (uint64_t)i * batch * t.row_bytes[f];
+            hipLaunchKernelGGL(k_per_sample_lds, dim3((uint32_t)((batch + kWG - 1) / kWG)), dim3(kLdsWG), lds, s, ai.sum,
+                               ai.uniforms, ai.mn, ai.depth, levels, (int)batch, beta, ai.seed, ai.calls, ai, ti);
+            LAUNCH_CHECK("k_per_sample_lds");
+        }
     }
-    if (!uniforms) b->calls += 1;
+    if (!uniforms) b->calls += (uint64_t)nbatch;
     return MRB_OK;
+}
+
+int mrb_per_sample(int64_t h, int64_t batch, float beta, const float* uniforms, int64_t* out_indices,
+                   float* out_weights, void* const* out_fields, void* stream) {
+    GET_PER(b, h);
+    return per_sample_impl(b.get(), 1, batch, beta, uniforms, out_indices, out_weights, out_fields,
+                           static_cast<hipStream_t>(stream));
+}
+
+int mrb_per_sample_many(int64_t h, int64_t nbatch, int64_t batch, float beta, const float* uniforms,
+                        int64_t* out_indices, float* out_weights, void* const* out_fields, void* stream) {
+    GET_PER(b, h);
+    return per_sample_impl(b.get(), nbatch, batch, beta, uniforms, out_indices, out_weights, out_fields,
+                           static_cast<hipStream_t>(stream));
 }
 
 int mrb_per_gather(int64_t h, const int64_t* indices, int64_t n, void* const* dst_fields, void* stream) {

@@ -325,7 +325,8 @@ struct WidePlan {
     uint32_t wide_items;    // wide granules per row
     uint32_t narrow_items;  // bytes of narrow fields per row
     int nwide, nnarrow;     // fields of each kind
-    uint32_t pad[2];
+    uint32_t nbatch;        // host side only: batches in the launch
+    uint32_t pad;
     WideField f[MRB_MAX_FIELDS];  // the wide fields first, then the narrow ones
 };
 
@@ -523,7 +524,7 @@ struct CopyWork {
 // Replaces PriorityReplayBufferSample (mindspore_rl/core/priority_replay_buffer.py:70,92-106).
 // sum .. calls are the arguments the tree walk needs; they are preloaded into scalar registers.
 // `groups` packs the descent plan: bits 0-3 the number of node groups, then 5 bits per group
-// with the levels it takes. kTen: every group takes 10 levels (trees of 10, 20 or 30 levels); the
+// with the levels it takes; bits 20-31 hold the number of batches in the launch minus one. kTen: every group takes 10 levels (trees of 10, 20 or 30 levels); the
 // walk is then compiled for that size, which shortens it by a third.
 template <int kInF, bool kTen, bool kOneWide>
 __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __restrict__ sum, const float* __restrict__ uniforms,
@@ -533,8 +534,15 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
     __shared__ float s_picked, s_total, s_pmin;
     __shared__ float s_tot[4];
     __shared__ SampleTail s_tail;
-    const int64_t k = blockIdx.x;      // row
+    const int64_t k = blockIdx.x;      // output row
     const uint32_t part = blockIdx.y;  // which of the row's workgroups
+    // Several batches in one launch (groups >> 20 = their number - 1): output row k is stratum `stratum`
+    // of batch `nth`; each batch is stratified on its own and takes the generator's next call counter.
+    uint32_t stratum = (uint32_t)k, nth = 0;
+    if (groups >> 20) {
+        nth = (uint32_t)k / (uint32_t)batch;
+        stratum = (uint32_t)k - nth * (uint32_t)batch;
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const bool walker = wave == 0;
     const bool deep = depth == 21 || depth == 22;
@@ -556,7 +564,7 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
         if (mine) {
             group_request(sum, (1u << share) + w, kGroupMaxLevels, lane, r0, r1, r2, r3);
             total = sum[1];
-            u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
+            u = uniforms ? uniforms[k] : rng_uniform(seed, calls + nth, (uint64_t)stratum);
             __builtin_amdgcn_sched_barrier(0);
             v = group_finish(kGroupMaxLevels, lane, r0, r1, r2, r3);
             const float t = group_total(v);
@@ -564,7 +572,7 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
         }
         __syncthreads();
         if (mine) {
-            float mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
+            float mass = (u + (float)stratum) * (total / (float)batch);  // each operation rounded once
             uint32_t q = 0;
             if (share == 2) {
                 const float left = s_tot[0] + s_tot[1];  // the node at depth 1
@@ -596,7 +604,7 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
         // the walk is a chain of dependent instructions: it goes ahead of the copy waves' address
         // arithmetic on the SIMD they share
         __builtin_amdgcn_s_setprio(3);
-        const int ngroups = (int)(groups & 15u);
+        const int ngroups = (int)(groups & 15u);  // (bits 4-18: the groups' sizes, bits 20-31: batches - 1)
         uint32_t node = 1;
         float picked, mass = 0.0f, total;
         if (depth >= 2) {
@@ -604,15 +612,15 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
             // together with the total and the draw (read from a valid address also when the generator
             // supplies the draw: no branch sits between the requests); the scheduling barrier keeps
             // every request ahead of the first use and of the generator's arithmetic.
-            uint32_t packed = groups >> 4;
+            uint32_t packed = (groups >> 4) & 0x7fffu;
             int g = kTen ? kGroupMaxLevels : (int)(packed & 31u);
             f32x4 r0, r1, r2, r3;
             group_request(sum, 1u, g, lane, r0, r1, r2, r3);
             total = sum[1];
             const float u_given = *(uniforms ? uniforms + k : sum + 1);
             __builtin_amdgcn_sched_barrier(0);
-            const float u = uniforms ? u_given : rng_uniform(seed, calls, (uint64_t)k);
-            mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
+            const float u = uniforms ? u_given : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+            mass = (u + (float)stratum) * (total / (float)batch);  // each operation rounded once
             node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
 #pragma nounroll
             for (int i = 1; i < ngroups; ++i) {
@@ -625,8 +633,8 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
         } else {
             // one or two leaves
             total = sum[1];
-            const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls, (uint64_t)k);
-            mass = (u + (float)k) * (total / (float)batch);
+            const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+            mass = (u + (float)stratum) * (total / (float)batch);
             picked = total;
             node = (1u << depth) + (depth ? group_walk(group_load_tiny(sum, 1u, depth, lane), depth, lane, mass, picked) : 0u);
         }
@@ -1117,13 +1125,21 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
         win[4 * lane + 2] = -1;
         win[4 * lane + 3] = -1;
         __builtin_amdgcn_wave_barrier();
-        for (int64_t base = 0; base < a.n; base += 64) {
-            const int64_t j = base + lane;
-            if (j < a.n) {
-                const int64_t idx = a.indices[j];
-                if (idx >= 0 && idx < a.capacity && valid_priority(a.priorities[j]) &&
-                    (uint32_t)((uint64_t)idx / kBlockNodes) == tile)
-                    atomicMax(&win[idx % kBlockNodes], (int)j);
+        // four entries per lane and trip: their loads go out together, then the election
+        for (int64_t base = 0; base < a.n; base += 64 * 4) {
+            int64_t idx[4];
+            float pr[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int64_t j = base + 64 * q + lane;
+                idx[q] = j < a.n ? a.indices[j] : -1;
+                pr[q] = j < a.n ? a.priorities[j] : -1.0f;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (idx[q] >= 0 && idx[q] < a.capacity && valid_priority(pr[q]) &&
+                    (uint32_t)((uint64_t)idx[q] / kBlockNodes) == tile)
+                    atomicMax(&win[idx[q] % kBlockNodes], (int)(base + 64 * q + lane));
             }
         }
         __threadfence_block();  // LDS operations of a wave complete in order; this also stops the compiler
@@ -1321,12 +1337,23 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
     }
     const uint32_t lane = threadIdx.x & 63;
     const int lo = a.lo[round], g = a.g[round];
-    const uint32_t tile = tile_base + blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
+    uint32_t tile = tile_base + blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
     const uint32_t ntiles = (1u << lo) / kBlockNodes;
     const bool last_round = round + 1 == a.nrounds;
-    if (tile >= ntiles) return;
     const bool elect = round == 0 && a.inline_election;
-    if (elect) entry_duty(a, tile, ntiles, lane);
+    if (elect) {
+        // Small update: a wave per ENTRY, not per tile of the level. Wave j rebuilds the tile that entry j
+        // falls into, with every entry of the call that falls into it; entries sharing a tile make
+        // their waves write the same values to the same nodes. (4096 tiles scanned for 512 entries
+        // cost three times as much as the rebuild itself.)
+        const uint32_t j = tile;  // tile_base is 0 here
+        if ((int64_t)j >= a.n) return;
+        entry_duty(a, j, (uint32_t)a.n, lane);
+        const int64_t idx = a.indices[j];
+        if (idx < 0 || idx >= a.capacity || !valid_priority(a.priorities[j])) return;
+        tile = (uint32_t)((uint64_t)idx / kBlockNodes);
+    }
+    if (tile >= ntiles) return;
     tile_round(a, lo, g, tile, true, (elect || (round == 0 && !a.indices)) ? nullptr : a.dirty[round],
                last_round ? nullptr : a.dirty[round + 1], last_round ? 0 : a.g[round + 1], lane,
                s_win[threadIdx.x >> 6]);

@@ -113,6 +113,41 @@ def test_config2_sac_shape_full_size(mrb, orc):
     g.destroy()
 
 
+@pytest.mark.parametrize("shape", ["wide", "deep", "narrow"])
+def test_sample_many_equals_successive_samples(mrb, orc, shape):
+    """mrb_per_sample_many against the oracle's successive sample() calls: with given draws and with the
+    generator (whose call counter then advances by the number of batches), on wide rows (one launch), on
+    a 21-level tree (shared top group) and through the LDS-top kernel (one launch per batch)."""
+    rng = np.random.default_rng(99)
+    if shape == "wide":
+        shapes, dtypes, cap, batch, path = [(300,), (1,), (3,)], [np.float32, np.int32, np.uint8], 3000, 48, 1
+    elif shape == "deep":
+        shapes, dtypes, cap, batch, path = [(2,)], [np.float32], (1 << 20) + 5, 40, 1
+    else:
+        shapes, dtypes, cap, batch, path = [(1,), (1,)], [np.int32, np.float32], 5000, 64, 2
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=21, shapes=shapes, dtypes=dtypes)
+    g.set_option("sample_path", path)
+    fill = min(cap, 6000)
+    rows = random_rows(rng, fill, shapes, dtypes)
+    g.insert(*to_dev(rows)), c.push(rows, fill)
+    idx = rng.integers(0, fill, 900)
+    pr = (rng.pareto(1.5, 900) + 1e-6).astype(np.float32)
+    g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda()), c.update(idx, pr)
+    for nb in (1, 3, 7):
+        u = rng.random((nb, batch)).astype(np.float32)
+        got = g.sample_many(nb, 0.6, uniforms=torch.from_numpy(u).cuda())
+        gen = g.sample_many(nb, 0.6)
+        for i in range(nb):
+            assert_sample_equal([x[i] for x in got], c.sample(batch, 0.6, u[i]), "%s nb %d batch %d" % (shape, nb, i))
+        for i in range(nb):
+            assert_sample_equal([x[i] for x in gen], c.sample(batch, 0.6), "%s generator nb %d batch %d" % (shape, nb, i))
+    assert_sample_equal(g.sample(0.6), c.sample(batch, 0.6), "generator position after sample_many")
+    with pytest.raises(ValueError):
+        g.sample_many(0, 0.5)
+    g.check()
+    g.destroy()
+
+
 def test_sample_output_ring(mrb, orc):
     """sample() hands out preallocated output sets in turn: `output_ring` calls return distinct tensors, the
     next call reuses the first set; output_ring=0 allocates fresh tensors; an explicit out= is written in
