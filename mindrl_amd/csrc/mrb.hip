@@ -344,6 +344,7 @@ struct Per {
     int device = 0;           // the HIP device the buffer lives on
     int64_t sample_path = 0;  // option "sample_path": 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
     int64_t lds_levels = 0;   // option "lds_levels": tree levels staged in LDS by the LDS-top kernel (0 = auto)
+    int64_t fused = 1;        // option "fused_rebuild": small updates and pushes rebuild the tree in one launch
     ~Per() {
         if (sum) (void)hipFree(sum);
         if (mn) (void)hipFree(mn);
@@ -427,6 +428,24 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
         a.nrounds = 0;
         a.top_depth = a.depth;
     }
+    // One round below the top and at most 16 waves of work (an update: a wave per entry; a push that does
+    // not wrap: a wave per leaf tile under its slots): one launch of one workgroup that goes on to the top.
+    if (a.nrounds == 1 && b.fused) {
+        uint32_t units = 0, tile_base = 0;
+        if (a.inline_election) {
+            units = (uint32_t)a.n;
+        } else if (!a.indices && a.first_slot + a.n <= a.capacity) {
+            tile_base = (uint32_t)(a.first_slot / kBlockNodes);
+            units = (uint32_t)((a.first_slot + a.n - 1) / kBlockNodes) - tile_base + 1;
+        }
+        if (units > 0 && units <= kFusedWG / 64) {
+            PutArgs put = ride ? *ride : none;
+            put.blocks = (put.blocks + 3) / 4;  // the ride-along copy was sized for workgroups a quarter as large
+            hipLaunchKernelGGL(k_tree_fused, dim3(1 + put.blocks), dim3(kFusedWG), 0, s, a, tile_base, units, put);
+            LAUNCH_CHECK("k_tree_fused");
+            return MRB_OK;
+        }
+    }
     for (int r = 0; r < a.nrounds; ++r) {
         uint32_t tiles = (1u << a.lo[r]) / kBlockNodes;
         uint32_t tile_base = 0;
@@ -443,7 +462,6 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
     const PutArgs& put = (a.nrounds == 0 && ride) ? *ride : none;
     hipLaunchKernelGGL(k_tree_top, dim3(1 + put.blocks), dim3(kTopWG), 0, s, a, put);
     LAUNCH_CHECK("k_tree_top");
-    (void)b;
     return MRB_OK;
 }
 
@@ -567,6 +585,10 @@ int mrb_set_option(int64_t h, const char* name, int64_t value) {
         if (!per) return fail(MRB_EINVAL, "lds_levels is an option of prioritized buffers");
         if (value < 0 || value > 12) return fail(MRB_EINVAL, "lds_levels must be in [0, 12]");
         per->lds_levels = value;
+    } else if (!strcmp(name, "fused_rebuild")) {
+        if (!per) return fail(MRB_EINVAL, "fused_rebuild is an option of prioritized buffers");
+        if (value < 0 || value > 1) return fail(MRB_EINVAL, "fused_rebuild must be 0 or 1");
+        per->fused = value;
     } else {
         return fail(MRB_EINVAL, "unknown option '%s'", name);
     }

@@ -1084,6 +1084,35 @@ __device__ __forceinline__ bool range_meets(const UpdateArgs& a, int64_t lo, int
 //              and the blocks holding a winner are the dirty ones
 // Lanes of clean blocks neither load nor store; the shuffles of a dirty block only mix
 // lanes of that block.
+// The g levels above a tile whose nodes (four per lane, vs / vm) are final: parents by in-lane
+// operations and wave shuffles, stored by the lanes of dirty blocks (`active`). `first`: heap index
+// of the tile's first node.
+__device__ __forceinline__ void tile_parents(const UpdateArgs& a, int g, uint32_t first, uint32_t lane, bool active,
+                                             const float4& vs, const float4& vm) {
+    // one level up: two nodes per lane; two levels up: one node per lane
+    const float s0 = vs.x + vs.y, s1 = vs.z + vs.w;
+    const float m0 = fminf(vm.x, vm.y), m1 = fminf(vm.z, vm.w);
+    float cs = s0 + s1, cm = fminf(m0, m1);
+    if (active && g >= 1) {
+        *reinterpret_cast<float2*>(a.sum + (first >> 1) + 2 * lane) = make_float2(s0, s1);
+        *reinterpret_cast<float2*>(a.mn + (first >> 1) + 2 * lane) = make_float2(m0, m1);
+    }
+    if (active && g >= 2) {
+        a.sum[(first >> 2) + lane] = cs;
+        a.mn[(first >> 2) + lane] = cm;
+    }
+    // three to eight levels up: 32, 16, 8, 4, 2, 1 nodes per full tile
+#pragma unroll
+    for (int s = 0; s < 6; ++s) {
+        cs = cs + __shfl_xor(cs, 1 << s);
+        cm = fminf(cm, __shfl_xor(cm, 1 << s));
+        if (active && g >= 3 + s && (lane & ((2u << s) - 1)) == 0) {
+            a.sum[(first >> (3 + s)) + (lane >> (s + 1))] = cs;
+            a.mn[(first >> (3 + s)) + (lane >> (s + 1))] = cm;
+        }
+    }
+}
+
 __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, uint32_t tile, bool sparse,
                                            const uint32_t* __restrict__ dirty_in, uint32_t* __restrict__ dirty_out,
                                            int g_next, uint32_t lane, int* win = nullptr) {
@@ -1186,28 +1215,7 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
         }
         if (dirty_out && ((off & ((1u << g) - 1)) == 0)) dirty_out[(off >> g) >> g_next] = a.epoch;
     }
-    // level lo-1: two nodes per lane; level lo-2: one node per lane
-    const float s0 = vs.x + vs.y, s1 = vs.z + vs.w;
-    const float m0 = fminf(vm.x, vm.y), m1 = fminf(vm.z, vm.w);
-    float cs = s0 + s1, cm = fminf(m0, m1);
-    if (active && g >= 1) {
-        *reinterpret_cast<float2*>(a.sum + (first >> 1) + 2 * lane) = make_float2(s0, s1);
-        *reinterpret_cast<float2*>(a.mn + (first >> 1) + 2 * lane) = make_float2(m0, m1);
-    }
-    if (active && g >= 2) {
-        a.sum[(first >> 2) + lane] = cs;
-        a.mn[(first >> 2) + lane] = cm;
-    }
-    // levels lo-3 .. lo-8: 32, 16, 8, 4, 2, 1 nodes per full tile
-#pragma unroll
-    for (int s = 0; s < 6; ++s) {
-        cs = cs + __shfl_xor(cs, 1 << s);
-        cm = fminf(cm, __shfl_xor(cm, 1 << s));
-        if (active && g >= 3 + s && (lane & ((2u << s) - 1)) == 0) {
-            a.sum[(first >> (3 + s)) + (lane >> (s + 1))] = cs;
-            a.mn[(first >> (3 + s)) + (lane >> (s + 1))] = cm;
-        }
-    }
+    tile_parents(a, g, first, lane, active, vs, vm);
 }
 
 // ---------------------------------------------------------------------------
@@ -1306,6 +1314,73 @@ __device__ __forceinline__ void entry_duty(const UpdateArgs& a, uint32_t wave_id
     }
 }
 
+// A small update's wave: rebuilds the 256-leaf tile that entry j falls into, with every entry of
+// the call that falls into it (the last one aimed at a leaf wins, elected by an LDS integer max over
+// a scan of the call's entries), and the g levels above it. Entries that share a tile make their
+// waves write the same values to the same nodes. The loads are kept apart from what they do not
+// depend on: the entry, the first entries of the scan and then the tile are requested before the
+// election runs.
+// dirty_out: the next round's words, marked for every block rebuilt here (NULL when the top comes next).
+__device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t j, uint32_t lane, int* win,
+                                           uint32_t* __restrict__ dirty_out, int g_next) {
+    constexpr int kPer = 4;  // entries per lane and trip of the scan
+    int64_t idx[kPer];
+    float pr[kPer];
+    const int64_t idx_j = a.indices[j];
+    const float p_j = a.priorities[j];
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        const int64_t e = 64 * q + lane;
+        idx[q] = e < a.n ? a.indices[e] : -1;
+        pr[q] = e < a.n ? a.priorities[e] : -1.0f;
+    }
+    win[4 * lane + 0] = -1;
+    win[4 * lane + 1] = -1;
+    win[4 * lane + 2] = -1;
+    win[4 * lane + 3] = -1;
+    if (idx_j < 0 || idx_j >= a.capacity || !valid_priority(p_j)) return;  // wave-uniform: an entry that is skipped
+    const uint32_t tile = (uint32_t)((uint64_t)idx_j / kBlockNodes);
+    const uint32_t first = (1u << a.depth) + tile * kBlockNodes;
+    float4 vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * lane);
+    float4 vm = *reinterpret_cast<const float4*>(a.mn + first + 4 * lane);
+    __builtin_amdgcn_wave_barrier();
+    for (int64_t base = 0; base < a.n; base += 64 * kPer) {
+        if (base > 0) {
+#pragma unroll
+            for (int q = 0; q < kPer; ++q) {
+                const int64_t e = base + 64 * q + lane;
+                idx[q] = e < a.n ? a.indices[e] : -1;
+                pr[q] = e < a.n ? a.priorities[e] : -1.0f;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            if (idx[q] >= 0 && idx[q] < a.capacity && valid_priority(pr[q]) &&
+                (uint32_t)((uint64_t)idx[q] / kBlockNodes) == tile)
+                atomicMax(&win[idx[q] % kBlockNodes], (int)(base + 64 * q + lane));  // the last entry wins
+        }
+    }
+    __threadfence_block();  // LDS operations of a wave complete in order; this also stops the compiler
+    __builtin_amdgcn_wave_barrier();
+    const int jw0 = win[4 * lane + 0], jw1 = win[4 * lane + 1], jw2 = win[4 * lane + 2], jw3 = win[4 * lane + 3];
+    const unsigned long long hit = __ballot(jw0 >= 0 || jw1 >= 0 || jw2 >= 0 || jw3 >= 0);
+    const uint32_t lanes_per_block = g >= 8 ? 64u : (1u << g) / 4u;
+    const unsigned long long block_lanes =
+        lanes_per_block >= 64 ? ~0ull : ((1ull << lanes_per_block) - 1) << (lane & ~(lanes_per_block - 1));
+    const bool active = (hit & block_lanes) != 0;  // this lane's block of 2^g leaves holds a winner
+    if (jw0 >= 0) vs.x = vm.x = powf_det(a.priorities[jw0], a.alpha);
+    if (jw1 >= 0) vs.y = vm.y = powf_det(a.priorities[jw1], a.alpha);
+    if (jw2 >= 0) vs.z = vm.z = powf_det(a.priorities[jw2], a.alpha);
+    if (jw3 >= 0) vs.w = vm.w = powf_det(a.priorities[jw3], a.alpha);
+    if (jw0 >= 0 || jw1 >= 0 || jw2 >= 0 || jw3 >= 0) {
+        *reinterpret_cast<float4*>(a.sum + first + 4 * lane) = vs;
+        *reinterpret_cast<float4*>(a.mn + first + 4 * lane) = vm;
+    }
+    const uint32_t off = tile * kBlockNodes + 4 * lane;  // this lane's first leaf
+    if (active && dirty_out && (off & ((1u << g) - 1)) == 0) dirty_out[(off >> g) >> g_next] = a.epoch;
+    tile_parents(a, g, first, lane, active, vs, vm);
+}
+
 // Rebuilds everything above depth `top` (<= 16) with one workgroup: first up to 8 levels over
 // the tiles of that depth (shared out among the waves), then the rest in one tile. When `top`
 // is the leaf level, clean tiles are skipped like in a round. `win`: 256 ints of LDS per wave
@@ -1348,10 +1423,10 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
         // cost three times as much as the rebuild itself.)
         const uint32_t j = tile;  // tile_base is 0 here
         if ((int64_t)j >= a.n) return;
+        entry_tile(a, g, j, lane, s_win[threadIdx.x >> 6], last_round ? nullptr : a.dirty[round + 1],
+                   last_round ? 0 : a.g[round + 1]);
         entry_duty(a, j, (uint32_t)a.n, lane);
-        const int64_t idx = a.indices[j];
-        if (idx < 0 || idx >= a.capacity || !valid_priority(a.priorities[j])) return;
-        tile = (uint32_t)((uint64_t)idx / kBlockNodes);
+        return;
     }
     if (tile >= ntiles) return;
     tile_round(a, lo, g, tile, true, (elect || (round == 0 && !a.indices)) ? nullptr : a.dirty[round],
@@ -1380,6 +1455,54 @@ __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) 
         // with an invalid priority take it), so it is raised only now.
         float q = 0.0f;
         for (int64_t j = threadIdx.x; j < a.n; j += kTopWG) {
+            const float p = a.priorities[j];
+            if (valid_priority(p)) {
+                q = fmaxf(q, powf_det(p, a.alpha));
+            } else {
+                atomicOr(a.err, MRB_DERR_PRIORITY);
+            }
+        }
+        for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+        if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// A push of few rows, or an update of at most 16 entries, on a tree with one round below the top,
+// in ONE launch: the tile work fits the 16 waves of one workgroup (a wave per leaf tile of a push,
+// or per entry of an update), and the same workgroup goes on to the top after a barrier. Within one
+// workgroup that needs no fence: its waves share a compute unit, and the nodes the top reads were
+// never in that unit's cache before they were written. (Handing the tiles of SEVERAL workgroups to a
+// last one through agent-scope stores, a counter and agent-scope loads was measured too: the three
+// trips through memory cost 2.9 us, more than the second launch they save.)
+//   units      waves with work: entries (update) or leaf tiles from tile_base on (push), at most 16
+// ---------------------------------------------------------------------------
+constexpr int kFusedWG = 1024;
+
+__global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t tile_base, uint32_t units, PutArgs put) {
+    __shared__ int s_win[kFusedWG / 64][kBlockNodes];
+    if (blockIdx.x >= 1) {
+        rows_put_part(put, blockIdx.x - 1, put.blocks);
+        return;
+    }
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (wave < units) {
+        if (a.inline_election) {
+            entry_tile(a, a.g[0], wave, lane, s_win[wave], nullptr, 0);
+            entry_duty(a, wave, units, lane);
+        } else {
+            tile_round(a, a.lo[0], a.g[0], tile_base + wave, true, nullptr, nullptr, 0, lane);
+        }
+    }
+    __threadfence_block();  // the tiles' highest nodes, written by other waves of this workgroup, are read below
+    __syncthreads();
+    top_rebuild(a, a.top_depth, &s_win[0][0]);
+    if (a.fold_max) {
+        // the tiles read the running max as it was before the call (fresh slots with an invalid
+        // priority take it); every workgroup has arrived, so it can be raised now
+        __syncthreads();
+        float q = 0.0f;
+        for (int64_t j = threadIdx.x; j < a.n; j += kFusedWG) {
             const float p = a.priorities[j];
             if (valid_priority(p)) {
                 q = fmaxf(q, powf_det(p, a.alpha));

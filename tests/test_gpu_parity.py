@@ -620,9 +620,10 @@ def make_pair(mrb, orc, alpha, cap, batch, seed=9, shapes=PER_SHAPES, dtypes=PER
     return g, c
 
 
+@pytest.mark.parametrize("fused", [1, 0])
 @pytest.mark.parametrize("path", [1, 2])
-@pytest.mark.parametrize("cap", [1, 2, 5, 100, 200, 4096, 5000, 10000, 70000])
-def test_per_random_ops_bit_exact(mrb, orc, cap, path):
+@pytest.mark.parametrize("cap", [1, 2, 5, 100, 200, 4096, 5000, 10000, 70000, 300000])
+def test_per_random_ops_bit_exact(mrb, orc, cap, path, fused):
     """Random pushes (plain / with priorities / larger than capacity), updates with
     duplicates and samples; after every step both trees, indices, rows, size, head and
     running max are compared. Capacities cover tree depths 0..17, i.e. the top kernel
@@ -631,9 +632,12 @@ def test_per_random_ops_bit_exact(mrb, orc, cap, path):
     batch = 32
     g, c = make_pair(mrb, orc, 0.6, cap, batch)
     g.set_option("sample_path", path)
+    g.set_option("fused_rebuild", fused)  # small updates and pushes in one launch, or a launch per round
     serial, exact_w = 0, 0
     for step in range(12):
         n = int(rng.integers(1, min(2 * cap + 3, 3000)))
+        if step % 4 == 1:
+            n = int(rng.integers(1, 40))  # a push of a few rows
         rows = id_rows(n, serial)
         serial += n
         if step % 3 == 2:
@@ -644,7 +648,12 @@ def test_per_random_ops_bit_exact(mrb, orc, cap, path):
             g.insert(*to_dev(rows))
             c.push(rows, n)
         k = int(rng.integers(1, min(2 * cap + 2, 2500)))
+        if step % 2 == 0:
+            k = int(rng.integers(1, 1025))  # few enough entries for the launch driven by entries
         idx = rng.integers(0, cap, k)
+        if step % 3 == 0:
+            idx[: k // 2] = idx[0] // 256 * 256 + rng.integers(0, 256, k // 2)  # many entries in one leaf tile
+            idx = np.minimum(idx, cap - 1)
         pr = rng.pareto(1.5, k).astype(np.float32) + np.float32(1e-6)
         g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda())
         c.update(idx, pr)
