@@ -499,6 +499,7 @@ UpdateArgs update_args(Per& b) {
     a.sum = b.sum;
     a.mn = b.mn;
     a.maxp = b.maxp;
+    a.maxp_next = b.maxp + 1;
     a.err = b.err;
     a.nrounds = b.nrounds;
     for (int r = 0; r < kMaxRounds; ++r) {
@@ -769,6 +770,10 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
         rest = 2;
         b->top_depth -= 1;
     }
+    if (rest == kRoundLevels + 1) {  // 21 levels: a top one level deeper (32 tiles) saves a whole round, i.e. a launch
+        rest = kRoundLevels;
+        b->top_depth += 1;
+    }
     b->nrounds = (rest + kRoundLevels - 1) / kRoundLevels;
     for (int r = 0, lo = b->depth; r < b->nrounds; ++r) {
         b->lo[r] = lo;
@@ -814,8 +819,8 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     }
     hipLaunchKernelGGL(k_fill_f32, dim3(grid_for(nodes)), dim3(kWG), 0, nullptr, b->mn, FLT_MAX, (uint64_t)nodes);
     LAUNCH_CHECK("k_fill_f32");
-    const float one = 1.0f;
-    HIP_TRY(hipMemcpy(b->maxp, &one, sizeof(one), hipMemcpyHostToDevice));
+    const float one_then_zero[4] = {1.0f, 0.0f, 0.0f, 0.0f};  // the running max; the max a push in progress has seen
+    HIP_TRY(hipMemcpy(b->maxp, one_then_zero, sizeof(one_then_zero), hipMemcpyHostToDevice));
     HIP_TRY(hipDeviceSynchronize());
     std::lock_guard<std::mutex> lk(g_mu);
     *out_handle = g_next++;
@@ -845,11 +850,14 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     if (rc) return rc;
     UpdateArgs a = update_args(*b);
     // push-then-update: the running max sees every priority of the call, surviving or not, and is
-    // raised only after the tree work (a fresh slot with an invalid priority keeps the old running max)
-    const bool fold = opt_priorities && skip == 0 && nrows <= 1024;  // few enough for the top workgroup
+    // raised only after the tree work (a fresh slot with an invalid priority keeps the old running max).
+    // Few rows: the top workgroup scans the priorities itself. More: the leaf-level waves, which compute
+    // every p^alpha anyway, collect their max beside the running max and the top workgroup folds it in.
+    // Only a call that overwrites rows of its own (more rows than capacity) needs a pass over all priorities.
+    const int fold = !opt_priorities ? 0 : (skip == 0 && nrows <= 1024) ? 1 : (skip == 0 && a.nrounds > 0) ? 2 : 0;
     if (opt_priorities) {
         a.priorities = opt_priorities + skip;
-        a.fold_max = fold ? 1 : 0;
+        a.fold_max = fold;
     }
     a.first_slot = first;
     a.n = n;

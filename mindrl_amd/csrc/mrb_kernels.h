@@ -994,6 +994,7 @@ struct UpdateArgs {
     float* mn;
     float* powered;  // [n] priorities^alpha of this call's entries (update_priorities only)
     float* maxp;  // running max priority (device scalar)
+    float* maxp_next;  // a push with priorities in progress: the largest p^alpha its leaf-level waves have seen
     uint32_t* err;
     // rebuild plan: round r starts at depth lo[r] and rebuilds g[r] levels; the top starts at top_depth
     int nrounds;
@@ -1001,7 +1002,8 @@ struct UpdateArgs {
     int g[kMaxRounds];
     int top_depth;
     uint32_t* dirty[kMaxRounds];  // per round: one epoch word per block of 1 << g[r] nodes at depth lo[r]
-    int fold_max;                // push with priorities: k_tree_top also folds them into the running max
+    int fold_max;                // push with priorities: the top workgroup also raises the running max, 1 = from a
+                                 // scan of the priorities, 2 = from maxp_next, where the leaf-level waves left it
     int inline_election;         // small update_priorities: no stamp pass, the leaf-level waves scan the entries
     // sparse updates of very large trees: the lowest sparse_g0 levels are rebuilt per entry
     // (k_tree_sparse) instead of per tile
@@ -1058,7 +1060,9 @@ __device__ __forceinline__ bool leaf_value(const UpdateArgs& a, int64_t leaf, fl
     if (j >= a.n) return false;
     if (a.priorities) {
         const float p = a.priorities[j];
-        q = valid_priority(p) ? powf_det(p, a.alpha) : *a.maxp;
+        const bool ok = valid_priority(p);
+        q = ok ? powf_det(p, a.alpha) : *a.maxp;
+        if (a.fold_max == 2 && !ok) atomicOr(a.err, MRB_DERR_PRIORITY);
     } else {
         q = *a.maxp;
     }
@@ -1215,6 +1219,14 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
         }
         if (dirty_out && ((off & ((1u << g) - 1)) == 0)) dirty_out[(off >> g) >> g_next] = a.epoch;
     }
+    if (leaf_level && a.fold_max == 2) {
+        // the largest leaf of the tile bounds every p^alpha written here from above, and is itself a p^alpha or
+        // a value no larger than the running max: folding it in raises the running max to exactly what a pass
+        // over the call's priorities would
+        float q = active ? fmaxf(fmaxf(vs.x, vs.y), fmaxf(vs.z, vs.w)) : 0.0f;
+        for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+        if (lane == 0 && q > 0.0f) raise_max(a.maxp_next, q);
+    }
     tile_parents(a, g, first, lane, active, vs, vm);
 }
 
@@ -1312,6 +1324,33 @@ __device__ __forceinline__ void entry_duty(const UpdateArgs& a, uint32_t wave_id
         for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
         if (lane == 0 && q > 0.0f) raise_max(a.maxp, q);
     }
+}
+
+// A push with priorities raises the running max to the largest p^alpha of the call, after the tree
+// work: the leaves read the running max as it was before the call (a fresh slot with an invalid
+// priority takes it), so every wave of the top workgroup passes the barrier before any raises it.
+__device__ __forceinline__ void fold_push_max(const UpdateArgs& a) {
+    __syncthreads();
+    if (a.fold_max == 2) {
+        // collected by the leaf-level waves, in this launch or the ones before it
+        if (threadIdx.x == 0) {
+            // taken and set back to zero in one atomic, where the waves' atomic maxima were performed
+            const float q = __uint_as_float(atomicExch(reinterpret_cast<unsigned int*>(a.maxp_next), 0u));
+            if (q > 0.0f) raise_max(a.maxp, q);
+        }
+        return;
+    }
+    float q = 0.0f;
+    for (int64_t j = threadIdx.x; j < a.n; j += blockDim.x) {
+        const float p = a.priorities[j];
+        if (valid_priority(p)) {
+            q = fmaxf(q, powf_det(p, a.alpha));
+        } else {
+            atomicOr(a.err, MRB_DERR_PRIORITY);
+        }
+    }
+    for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+    if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
 }
 
 // A small update's wave: rebuilds the 256-leaf tile that entry j falls into, with every entry of
@@ -1447,24 +1486,7 @@ __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) 
         return;
     }
     top_rebuild(a, a.top_depth, &s_win[0][0]);
-    if (a.fold_max) {
-        // every wave has finished reading the running max (a fresh slot with an invalid priority takes
-        // its value from before the call) before any wave raises it
-        __syncthreads();
-        // The rounds before this launch read the running max as it was before the call (fresh slots
-        // with an invalid priority take it), so it is raised only now.
-        float q = 0.0f;
-        for (int64_t j = threadIdx.x; j < a.n; j += kTopWG) {
-            const float p = a.priorities[j];
-            if (valid_priority(p)) {
-                q = fmaxf(q, powf_det(p, a.alpha));
-            } else {
-                atomicOr(a.err, MRB_DERR_PRIORITY);
-            }
-        }
-        for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
-        if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
-    }
+    if (a.fold_max) fold_push_max(a);
 }
 
 // ---------------------------------------------------------------------------
@@ -1497,22 +1519,7 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
     __threadfence_block();  // the tiles' highest nodes, written by other waves of this workgroup, are read below
     __syncthreads();
     top_rebuild(a, a.top_depth, &s_win[0][0]);
-    if (a.fold_max) {
-        // the tiles read the running max as it was before the call (fresh slots with an invalid
-        // priority take it); every workgroup has arrived, so it can be raised now
-        __syncthreads();
-        float q = 0.0f;
-        for (int64_t j = threadIdx.x; j < a.n; j += kFusedWG) {
-            const float p = a.priorities[j];
-            if (valid_priority(p)) {
-                q = fmaxf(q, powf_det(p, a.alpha));
-            } else {
-                atomicOr(a.err, MRB_DERR_PRIORITY);
-            }
-        }
-        for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
-        if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
-    }
+    if (a.fold_max) fold_push_max(a);
 }
 
 // ---------------------------------------------------------------------------
