@@ -31,6 +31,13 @@
  *     priority_replay_buffer.py:67-76); sample / gather calls on one handle may
  *     run at the same time on different streams as long as no call that changes
  *     the handle is in flight; different handles are independent.
+ *   - calls that neither wait nor allocate may be recorded into a HIP graph. A replay repeats the call
+ *     as it was recorded: the ring position, the row count and the generator's call counter are host-side
+ *     state that becomes kernel arguments, so a replayed push writes the slots it wrote when recorded and
+ *     a replayed sample without `uniforms` draws the numbers it drew then. mrb_per_gather and an
+ *     mrb_per_update of at most 1024 entries replay correctly against whatever the buffer holds at replay
+ *     time; so does mrb_per_sample with `uniforms` while the number of stored rows is what it was when
+ *     recorded (a full buffer).
  *   - storage is structure-of-arrays: field i is one [capacity, field_bytes[i]]
  *     byte matrix (reference layout: uniform_replay_buffer.py:26-47).
  */
