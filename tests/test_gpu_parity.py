@@ -148,6 +148,53 @@ def test_sample_many_equals_successive_samples(mrb, orc, shape):
     g.destroy()
 
 
+@pytest.mark.parametrize("path", [1, 2])
+def test_hip_graph_replays_update_and_sample(mrb, orc, path):
+    """update_priorities (<= 1024 entries) + sample with given draws, recorded once into a HIP graph and
+    replayed five times on new inputs, with eager calls and synchronisations between the replays: every
+    replay equals the oracle's update + sample, and so does the eager work in between."""
+    rng = np.random.default_rng(31 + path)
+    shapes, dtypes = ([(300,), (1,)], [np.float32, np.int32]) if path == 1 else ([(1,), (2,)], [np.int32, np.float32])
+    cap, batch, nupd = 3000, 64, 200
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=5, shapes=shapes, dtypes=dtypes)
+    g.set_option("sample_path", path)
+    rows = random_rows(rng, cap, shapes, dtypes)  # a full buffer: the number of stored rows stays what was recorded
+    g.insert(*to_dev(rows)), c.push(rows, cap)
+    u_dev = torch.zeros(batch, dtype=torch.float32, device="cuda")
+    idx_dev = torch.zeros(nupd, dtype=torch.int64, device="cuda")
+    pr_dev = torch.ones(nupd, dtype=torch.float32, device="cuda")
+    out = (torch.empty(batch, dtype=torch.int64, device="cuda"), torch.empty(batch, dtype=torch.float32, device="cuda"),
+           g._layout.empty(batch, g._dev))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        g.update_priorities(idx_dev, pr_dev)
+        g.sample(0.7, uniforms=u_dev, out=out)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for rep in range(5):
+        idx = rng.integers(0, cap, nupd)
+        idx[:20] = idx[0]  # duplicates: the last entry wins
+        pr = (rng.pareto(1.5, nupd) + 1e-6).astype(np.float32)
+        u = rng.random(batch).astype(np.float32)
+        idx_dev.copy_(torch.from_numpy(idx)), pr_dev.copy_(torch.from_numpy(pr)), u_dev.copy_(torch.from_numpy(u))
+        graph.replay()
+        torch.cuda.synchronize()
+        c.update(idx, pr)
+        assert_sample_equal((out[0], out[1]) + tuple(out[2]), c.sample(batch, 0.7, u), "path %d replay %d" % (path, rep))
+        assert_tree_equal(g, c, "path %d replay %d" % (path, rep))
+        # eager work between the replays
+        e_idx = rng.integers(0, cap, 50)
+        e_pr = (rng.pareto(1.5, 50) + 1e-6).astype(np.float32)
+        g.update_priorities(torch.from_numpy(e_idx).cuda(), torch.from_numpy(e_pr).cuda()), c.update(e_idx, e_pr)
+        u2 = rng.random(batch).astype(np.float32)
+        assert_sample_equal(g.sample(0.4, uniforms=torch.from_numpy(u2).cuda()), c.sample(batch, 0.4, u2), "eager %d" % rep)
+    del graph
+    g.destroy()
+
+
 def test_sample_output_ring(mrb, orc):
     """sample() hands out preallocated output sets in turn: `output_ring` calls return distinct tensors, the
     next call reuses the first set; output_ring=0 allocates fresh tensors; an explicit out= is written in
