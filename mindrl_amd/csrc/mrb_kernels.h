@@ -1543,7 +1543,7 @@ __global__ __launch_bounds__(kWG) void k_discounted_return(const float* __restri
     int64_t t = timesteps - 1;
     for (; t >= UNROLL - 1; t -= UNROLL) {
         float r[UNROLL];
-        uint8_t d[UNROLL];
+        uint32_t d[UNROLL];  // 32-bit: byte-sized register arrays make the compiler pack and unpack them
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             r[u] = __builtin_nontemporal_load(reward + (t - u) * cols + c);
@@ -1564,91 +1564,157 @@ __global__ __launch_bounds__(kWG) void k_discounted_return(const float* __restri
 }
 
 // The same recurrence for inputs with few columns, where a thread per column leaves the memory
-// system idle: a workgroup takes 64 columns and walks the time axis in chunks of kDrChunk steps.
-// All sixteen waves load a chunk's rewards and done flags into LDS (independent, fully coalesced
-// loads), wave 0 runs the recurrence over the chunk out of LDS (lane = column), all waves store
-// the results. The arithmetic and its order are those of k_discounted_return.
-constexpr int kDrChunk = 256;
+// system idle: a workgroup takes 64 columns and walks the time axis backwards in chunks of
+// kDrChunk steps through three LDS buffers, as a pipeline whose stages run at the same time on
+// consecutive chunks:
+//   request  waves 1..15 (the movers) request chunk s+1's rewards and done flags into registers
+//            (independent, coalesced loads); they arrive during the stage ...
+//   deposit  ... the movers put chunk s, requested a stage ago, into its LDS buffer ...
+//   recur    ... wave 0 runs the recurrence over chunk s-1 out of LDS (lane = column) ...
+//   drain    ... and the movers write chunk s-2's results from LDS to memory.
+// One barrier per stage; no wave waits for a load it has just issued. The memory system so sees
+// loads and stores all the time, instead of a load phase, a phase without traffic and a store
+// phase per chunk. The arithmetic and its order are those of k_discounted_return.
+// A workgroup barrier for data handed over in LDS only: it waits for the wave's LDS operations, not for
+// its global loads and stores, which __syncthreads() would also wait for - here those are the next
+// chunk's requests and the last chunk's results, meant to stay in flight across the barrier.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+constexpr int kDrChunk = 128;
 constexpr int kDrCols = 64;
-constexpr int kDrWG = 1024;  // 16 waves: each thread moves 16 rows of a chunk, all 16 loads in flight at once
+constexpr int kDrWG = 1024;
+constexpr int kDrMovers = kDrWG - 64;                         // threads of waves 1..15
+constexpr int kDrSweep = kDrMovers / kDrCols;                 // rows the movers cover at once
+constexpr int kDrPer = (kDrChunk + kDrSweep - 1) / kDrSweep;  // elements a mover carries per chunk
 __global__ __launch_bounds__(kDrWG) void k_discounted_return_tiled(const float* __restrict__ reward,
                                                                  const uint8_t* __restrict__ done,
                                                                  const float* __restrict__ last_value,
                                                                  float* __restrict__ out, int64_t timesteps,
                                                                  int64_t batch, int64_t inner, float gamma) {
-    __shared__ float s_val[kDrChunk * kDrCols];    // rewards in, returns out
-    __shared__ uint8_t s_done[kDrChunk * kDrCols];
+    __shared__ float s_val[3][kDrChunk * kDrCols];    // rewards in, returns out
+    __shared__ uint8_t s_done[3][kDrChunk * kDrCols];
     const int64_t cols = batch * inner;
     const int64_t c0 = (int64_t)blockIdx.x * kDrCols;
     const int ncols = (int)(cols - c0 < kDrCols ? cols - c0 : kDrCols);
     const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const bool mover = wave != 0;
+    // a mover's elements of a chunk: column m % 64 of the rows m / 64, m / 64 + 15, ... (960 movers = 15 rows
+    // of 64 columns per sweep), so its addresses differ by a constant from one element to the next
+    const int m = (int)threadIdx.x - 64;
+    const int mrow = m / kDrCols;
+    const bool mcol_ok = m % kDrCols < ncols;
+    const int mcol = mcol_ok ? m % kDrCols : 0;  // a column past the end reads column 0 and stores nothing
+    const int64_t mb = (c0 + mcol) / inner;      // the column's batch entry (done flags)
+    const int nchunks = (int)((timesteps + kDrChunk - 1) / kDrChunk);
+    // chunk c covers the steps [lo, lo + steps), counted from the end of the time axis
+    auto chunk_lo = [&](int c) -> int64_t {
+        const int64_t hi = timesteps - (int64_t)c * kDrChunk;
+        return hi > kDrChunk ? hi - kDrChunk : 0;
+    };
+    auto chunk_steps = [&](int c) -> int {
+        const int64_t hi = timesteps - (int64_t)c * kDrChunk;
+        return (int)(hi > kDrChunk ? kDrChunk : hi);
+    };
+    // (done flags travel as 32-bit values: byte-sized register arrays make the compiler pack and unpack them)
+    auto request = [&](int c, float (&r)[kDrPer], uint32_t (&d)[kDrPer]) {
+        if (c >= nchunks) return;
+        const int64_t lo = chunk_lo(c);
+        const int steps = chunk_steps(c);
+        const float* rp = reward + (lo + mrow) * cols + c0 + mcol;
+        const uint8_t* dp = done + (lo + mrow) * batch + mb;
+        const int64_t rstep = kDrSweep * cols, dstep = kDrSweep * batch;  // wave-uniform
+#pragma unroll
+        for (int u = 0; u < kDrPer; ++u) {
+            if (mrow + u * kDrSweep < steps) {
+                r[u] = __builtin_nontemporal_load(rp);
+                d[u] = *dp;
+            }
+            rp += rstep;
+            dp += dstep;
+        }
+    };
+    auto deposit = [&](int c, const float (&r)[kDrPer], const uint32_t (&d)[kDrPer]) {
+        if (c >= nchunks) return;
+        const int steps = chunk_steps(c);
+        float* dv = s_val[c % 3] + m;
+        uint8_t* dd = s_done[c % 3] + m;
+#pragma unroll
+        for (int u = 0; u < kDrPer; ++u) {
+            if (mrow + u * kDrSweep < steps) {
+                dv[u * kDrMovers] = r[u];
+                dd[u * kDrMovers] = (uint8_t)d[u];
+            }
+        }
+    };
+    auto drain = [&](int c) {
+        if (c < 0 || c >= nchunks || !mcol_ok) return;
+        const int64_t lo = chunk_lo(c);
+        const int steps = chunk_steps(c);
+        const float* src = s_val[c % 3] + m;
+        float* op = out + (lo + mrow) * cols + c0 + mcol;
+        const int64_t ostep = kDrSweep * cols;  // wave-uniform
+#pragma unroll
+        for (int u = 0; u < kDrPer; ++u) {
+            if (mrow + u * kDrSweep < steps) __builtin_nontemporal_store(src[u * kDrMovers], op);
+            op += ostep;
+        }
+    };
     float last = 0.0f;
-    if (threadIdx.x < ncols) last = last_value[c0 + threadIdx.x];
-    for (int64_t hi = timesteps; hi > 0; hi -= kDrChunk) {
-        const int64_t t0 = hi > kDrChunk ? hi - kDrChunk : 0;
-        const int steps = (int)(hi - t0);
-        // thread -> column cc, time rows tr, tr + 16, ...: 16 loads are issued before the first LDS write
-        {
-            constexpr int BATCH = 16, ROWS = kDrWG / kDrCols;
-            const int cc = threadIdx.x % kDrCols, tr = threadIdx.x / kDrCols;
-            const int64_t c = c0 + (cc < ncols ? cc : 0);
-            const int64_t b = c / inner;
-            for (int base = tr; base < steps; base += ROWS * BATCH) {
-                float r[BATCH];
-                uint8_t d[BATCH];
+    if (wave == 0 && lane < ncols) last = last_value[c0 + lane];
+    // (1 - done) * gamma has two values; computing both once leaves a select, a multiply and an add per step
+    const float scaled_live = (1.0f - 0.0f) * gamma, scaled_done = (1.0f - 1.0f) * gamma;
+    auto recur = [&](int c) {
+        if (c < 0 || c >= nchunks || lane >= ncols) return;
+        const int steps = chunk_steps(c);
+        float* val = s_val[c % 3];
+        const uint8_t* dn = s_done[c % 3];
+        // 16 steps at a time through registers, so that the LDS reads are not serialised behind the
+        // recurrence's stores
+        constexpr int STEP = 16;
+        int tt = steps - 1;
+        for (; tt >= STEP - 1; tt -= STEP) {
+            float r[STEP];
+            uint32_t d[STEP];
 #pragma unroll
-                for (int u = 0; u < BATCH; ++u) {
-                    const int tt = base + u * ROWS < steps ? base + u * ROWS : tr;  // clamped: always a valid row
-                    r[u] = __builtin_nontemporal_load(reward + (t0 + tt) * cols + c);
-                    d[u] = done[(t0 + tt) * batch + b];
-                }
-#pragma unroll
-                for (int u = 0; u < BATCH; ++u) {
-                    const int tt = base + u * ROWS;
-                    if (tt < steps) {
-                        s_val[tt * kDrCols + cc] = r[u];
-                        s_done[tt * kDrCols + cc] = d[u];
-                    }
-                }
+            for (int u = 0; u < STEP; ++u) {
+                r[u] = val[(tt - u) * kDrCols + lane];
+                d[u] = dn[(tt - u) * kDrCols + lane];
             }
-        }
-        __syncthreads();
-        if (threadIdx.x < 64 && lane < ncols) {
-            // 32 steps at a time through registers, so that the LDS reads are not serialised
-            // behind the recurrence's stores
-            constexpr int STEP = 32;
-            int tt = steps - 1;
-            for (; tt >= STEP - 1; tt -= STEP) {
-                float r[STEP];
-                uint8_t d[STEP];
 #pragma unroll
-                for (int u = 0; u < STEP; ++u) {
-                    r[u] = s_val[(tt - u) * kDrCols + lane];
-                    d[u] = s_done[(tt - u) * kDrCols + lane];
-                }
-#pragma unroll
-                for (int u = 0; u < STEP; ++u) {
-                    const float scaled = (1.0f - (d[u] ? 1.0f : 0.0f)) * gamma;
-                    last = r[u] + scaled * last;
-                    r[u] = last;
-                }
-#pragma unroll
-                for (int u = 0; u < STEP; ++u) s_val[(tt - u) * kDrCols + lane] = r[u];
+            for (int u = 0; u < STEP; ++u) {
+                last = r[u] + (d[u] ? scaled_done : scaled_live) * last;
+                r[u] = last;
             }
-            for (; tt >= 0; --tt) {
-                const float scaled = (1.0f - (s_done[tt * kDrCols + lane] ? 1.0f : 0.0f)) * gamma;
-                last = s_val[tt * kDrCols + lane] + scaled * last;
-                s_val[tt * kDrCols + lane] = last;
-            }
+#pragma unroll
+            for (int u = 0; u < STEP; ++u) val[(tt - u) * kDrCols + lane] = r[u];
         }
-        __syncthreads();
-        {
-            const int cc = threadIdx.x % kDrCols, tr = threadIdx.x / kDrCols;
-            if (cc < ncols)
-                for (int tt = tr; tt < steps; tt += kDrWG / kDrCols)
-                    __builtin_nontemporal_store(s_val[tt * kDrCols + cc], out + (t0 + tt) * cols + c0 + cc);
+        for (; tt >= 0; --tt) {
+            last = val[tt * kDrCols + lane] + (dn[tt * kDrCols + lane] ? scaled_done : scaled_live) * last;
+            val[tt * kDrCols + lane] = last;
         }
-        __syncthreads();
+    };
+    // two register sets take turns: the chunk requested in one stage is deposited in the next
+    float ra[kDrPer], rb[kDrPer];
+    uint32_t da[kDrPer], db[kDrPer];
+    if (mover) request(0, ra, da);
+    for (int s = 0; s < nchunks + 2; s += 2) {
+        if (mover) {
+            request(s + 1, rb, db);
+            drain(s - 2);
+            deposit(s, ra, da);
+        } else if (wave == 0) {
+            recur(s - 1);
+        }
+        lds_barrier();
+        if (mover) {
+            request(s + 2, ra, da);
+            drain(s - 1);
+            deposit(s + 1, rb, db);
+        } else if (wave == 0) {
+            recur(s);
+        }
+        lds_barrier();
     }
 }
 
