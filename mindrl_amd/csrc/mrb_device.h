@@ -70,6 +70,12 @@ __device__ __forceinline__ float powf_det(float x, float a) {
     return (float)(q * scale);
 }
 
+// The same function as one shared copy, for kernels that take powers in many places (the tree kernels
+// inline their tile code several times over, each with several powers): the call keeps their code half
+// as large, and launches that are bound by latency, instruction fetch included, notice. The kernel with a
+// power per thread on its critical path (the LDS-top sample kernel) keeps the inlined one.
+__device__ __attribute__((noinline)) float powf_det_call(float x, float a) { return powf_det(x, a); }
+
 // Counter-based generator: one 64-bit mix of (seed, call counter, draw number).
 __device__ __forceinline__ uint64_t rng_u64(uint64_t seed, uint64_t counter, uint64_t k) {
     uint64_t z = seed + 0x9E3779B97F4A7C15ULL * ((counter << 32) + k + 1ULL);

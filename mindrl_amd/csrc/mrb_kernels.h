@@ -694,7 +694,7 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
     const float fsize = (float)s_tail.size;
     const float x = lane == 0 ? s_picked : s_pmin;
     float r = 0.0f;
-    if (lane < 2) r = powf_det(x / total * fsize, -s_tail.beta);
+    if (lane < 2) r = powf_det_call(x / total * fsize, -s_tail.beta);
     const float max_w = __shfl(r, 1);
     if (lane == 0) {
         s_tail.out_idx[k] = idx;
@@ -1029,7 +1029,7 @@ __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
         if (!idx_ok) atomicOr(a.err, MRB_DERR_INDEX);
         if (!valid_priority(p)) atomicOr(a.err, MRB_DERR_PRIORITY);
         if (idx_ok && valid_priority(p)) {
-            q = powf_det(p, a.alpha);
+            q = powf_det_call(p, a.alpha);
             if (a.indices) {
                 a.powered[j] = q;
                 atomicMax(&a.stamp[idx], ((unsigned long long)a.epoch << 32) | (unsigned long long)j);
@@ -1061,7 +1061,7 @@ __device__ __forceinline__ bool leaf_value(const UpdateArgs& a, int64_t leaf, fl
     if (a.priorities) {
         const float p = a.priorities[j];
         const bool ok = valid_priority(p);
-        q = ok ? powf_det(p, a.alpha) : *a.maxp;
+        q = ok ? powf_det_call(p, a.alpha) : *a.maxp;
         if (a.fold_max == 2 && !ok) atomicOr(a.err, MRB_DERR_PRIORITY);
     } else {
         q = *a.maxp;
@@ -1202,10 +1202,10 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
             float q;
             bool wrote = false;
             if (elect) {
-                if (jw0 >= 0) { vs.x = vm.x = powf_det(a.priorities[jw0], a.alpha); wrote = true; }
-                if (jw1 >= 0) { vs.y = vm.y = powf_det(a.priorities[jw1], a.alpha); wrote = true; }
-                if (jw2 >= 0) { vs.z = vm.z = powf_det(a.priorities[jw2], a.alpha); wrote = true; }
-                if (jw3 >= 0) { vs.w = vm.w = powf_det(a.priorities[jw3], a.alpha); wrote = true; }
+                if (jw0 >= 0) { vs.x = vm.x = powf_det_call(a.priorities[jw0], a.alpha); wrote = true; }
+                if (jw1 >= 0) { vs.y = vm.y = powf_det_call(a.priorities[jw1], a.alpha); wrote = true; }
+                if (jw2 >= 0) { vs.z = vm.z = powf_det_call(a.priorities[jw2], a.alpha); wrote = true; }
+                if (jw3 >= 0) { vs.w = vm.w = powf_det_call(a.priorities[jw3], a.alpha); wrote = true; }
             } else {
                 if (leaf_value(a, off + 0, q)) { vs.x = vm.x = q; wrote = true; }
                 if (leaf_value(a, off + 1, q)) { vs.y = vm.y = q; wrote = true; }
@@ -1319,7 +1319,7 @@ __device__ __forceinline__ void entry_duty(const UpdateArgs& a, uint32_t wave_id
             const bool idx_ok = idx >= 0 && idx < a.capacity;
             if (!idx_ok) atomicOr(a.err, MRB_DERR_INDEX);
             if (!valid_priority(p)) atomicOr(a.err, MRB_DERR_PRIORITY);
-            if (idx_ok && valid_priority(p)) q = powf_det(p, a.alpha);
+            if (idx_ok && valid_priority(p)) q = powf_det_call(p, a.alpha);
         }
         for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
         if (lane == 0 && q > 0.0f) raise_max(a.maxp, q);
@@ -1344,7 +1344,7 @@ __device__ __forceinline__ void fold_push_max(const UpdateArgs& a) {
     for (int64_t j = threadIdx.x; j < a.n; j += blockDim.x) {
         const float p = a.priorities[j];
         if (valid_priority(p)) {
-            q = fmaxf(q, powf_det(p, a.alpha));
+            q = fmaxf(q, powf_det_call(p, a.alpha));
         } else {
             atomicOr(a.err, MRB_DERR_PRIORITY);
         }
@@ -1407,10 +1407,10 @@ __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t 
     const unsigned long long block_lanes =
         lanes_per_block >= 64 ? ~0ull : ((1ull << lanes_per_block) - 1) << (lane & ~(lanes_per_block - 1));
     const bool active = (hit & block_lanes) != 0;  // this lane's block of 2^g leaves holds a winner
-    if (jw0 >= 0) vs.x = vm.x = powf_det(a.priorities[jw0], a.alpha);
-    if (jw1 >= 0) vs.y = vm.y = powf_det(a.priorities[jw1], a.alpha);
-    if (jw2 >= 0) vs.z = vm.z = powf_det(a.priorities[jw2], a.alpha);
-    if (jw3 >= 0) vs.w = vm.w = powf_det(a.priorities[jw3], a.alpha);
+    if (jw0 >= 0) vs.x = vm.x = powf_det_call(a.priorities[jw0], a.alpha);
+    if (jw1 >= 0) vs.y = vm.y = powf_det_call(a.priorities[jw1], a.alpha);
+    if (jw2 >= 0) vs.z = vm.z = powf_det_call(a.priorities[jw2], a.alpha);
+    if (jw3 >= 0) vs.w = vm.w = powf_det_call(a.priorities[jw3], a.alpha);
     if (jw0 >= 0 || jw1 >= 0 || jw2 >= 0 || jw3 >= 0) {
         *reinterpret_cast<float4*>(a.sum + first + 4 * lane) = vs;
         *reinterpret_cast<float4*>(a.mn + first + 4 * lane) = vm;
