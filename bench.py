@@ -408,6 +408,31 @@ def per_extras(a, torch, r):
     extras["loop_steps_per_s"] = 1.0 / timed(lambda i: r.loop(W + i % K))
     if not r.loop_step:
         extras["sample_us_per_call"] = timed(lambda i: r.sample(W + i % K)) * 1e6
+        # spread over the run: an event after every 10 calls (an event after every call would add its own ~3 us),
+        # 40 groups of 10 back-to-back calls
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(41)]
+        torch.cuda.synchronize()
+        evs[0].record(r.stream)
+        for g in range(40):
+            for i in range(10):
+                r.sample(W + (10 * g + i) % K)
+            evs[g + 1].record(r.stream)
+        torch.cuda.synchronize()
+        per_call = np.sort(np.array([evs[g].elapsed_time(evs[g + 1]) * 100.0 for g in range(40)]))
+        extras["sample_us_p10_p50_p90_of_10_call_groups"] = [float(per_call[4]), float(per_call[20]), float(per_call[36])]
+        if a.workload == "c3":
+            # the frame-shared next observation: rows at the sampled transitions' next_idx, through mrb_per_gather
+            # (whole rows, 2 * 28,241 B each: 28.9 MB per call on top of the sample's)
+            nxt = r.fields[1].reshape(-1)
+            gfields = r.buf._layout.empty(batch, r.buf._dev)
+            gptr = r.pointers(gfields)
+            r.sample(W)
+            extras["next_obs_gather_same_slots_us_per_call"] = timed(
+                lambda i: L.mrb_per_gather(h, nxt.data_ptr(), batch, gptr, sp)) * 1e6
+            # sample, then gather at the slots that very sample returned: other rows every call
+            extras["sample_plus_next_obs_us"] = timed(
+                lambda i: (r.sample(W + i % K), L.mrb_per_gather(h, nxt.data_ptr(), batch, gptr, sp))) * 1e6
+            del gfields
         # the same calls replayed from one captured HIP graph (a chain: every call ordered after the one before)
         n_g = min(K, 200)
         graph = torch.cuda.CUDAGraph()
