@@ -108,8 +108,12 @@ def set_option(handle, name, value):
     check(lib().mrb_set_option(int(handle), name.encode(), int(value)))
 
 
+_PTR_ARRAYS = {}
+
+
 def ptr_array(pointers):
-    arr = (C.c_void_p * len(pointers))()
-    for i, p in enumerate(pointers):
-        arr[i] = p
-    return arr
+    n = len(pointers)
+    kind = _PTR_ARRAYS.get(n)
+    if kind is None:
+        kind = _PTR_ARRAYS[n] = C.c_void_p * n
+    return kind(*pointers)

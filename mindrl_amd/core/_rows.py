@@ -85,6 +85,21 @@ class FieldLayout:
                 raise ValueError("fields disagree on the number of rows (%d vs %d)" % (n, rows))
         return n
 
+    def rows_if_ready(self, fields, dev):
+        """Number of rows when `fields` already are contiguous device tensors of the declared dtypes holding
+        whole elements (the training path: nothing to convert, one pass), else None."""
+        if len(fields) != len(self.numel):
+            return None
+        n = -1
+        for f, d, numel in zip(fields, self.dtypes, self.numel):
+            if not (isinstance(f, torch.Tensor) and f.dtype == d and f.device == dev and f.is_contiguous()):
+                return None
+            rows, rest = divmod(f.numel(), numel)
+            if rest or (n >= 0 and rows != n):
+                return None
+            n = rows
+        return n
+
     def to_device(self, fields, dev):
         """Contiguous device tensors of the declared dtypes (copies host data if needed)."""
         out = []

@@ -68,8 +68,12 @@ class PriorityReplayBuffer:
         tensor int64[1]."""
         if len(transition) == 1 and isinstance(transition[0], (list, tuple)):
             transition = tuple(transition[0])
-        n = self._layout.batch_of(transition)
-        src = self._layout.to_device(transition, self._dev)
+        n = self._layout.rows_if_ready(transition, self._dev)
+        if n is not None:
+            src = transition
+        else:
+            n = self._layout.batch_of(transition)
+            src = self._layout.to_device(transition, self._dev)
         pr = None
         if priorities is not None:
             pr = flat_on_device(priorities, torch.float32, self._dev)
