@@ -10,6 +10,8 @@
 
 namespace mrb {
 
+// Timestamps inside the kernels, for tuning: compiled in only with -DMRB_PROBE (the library is never
+// built that way; a tuning build includes this file with the macro set and reads g_probe back).
 #ifdef MRB_PROBE
 __device__ uint64_t g_probe[16384 * 16];
 #define MRB_TS(var) const uint64_t var = wall_clock64()
