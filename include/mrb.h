@@ -78,7 +78,7 @@ int mrb_version(void);
  *   "row_split"    least number of workgroups per row in the wide-row kernel (0 = auto, max 64)
  *   "sample_path"  prioritized buffers: 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
  *   "lds_levels"   prioritized buffers: tree levels staged in LDS by the LDS-top kernel (0 = auto, max 12)
- *   "fused_rebuild" prioritized buffers: 1 (default) = an update of <= 16 entries or a push under <= 16 leaf tiles
+ *   "fused_rebuild" prioritized buffers: 1 (default) = an update of <= 32 entries or a push under <= 32 leaf tiles
  *                  rebuilds the tree in one launch where the tree has one round of levels below its top;
  *                  0 = one launch per round */
 int mrb_set_option(int64_t h, const char *name, int64_t value);
