@@ -49,3 +49,31 @@ def create_replay_buffer(replay_buffer_config):
     {'number': 1, 'type': UniformReplayBuffer, 'capacity': 100000, 'sample_size': 64,
      'data_shape': [(4,), (1,), (1,), (4,)], 'data_type': [float32, int32, float32, float32]}."""
     return ReplayBufferSpec(replay_buffer_config).build()
+
+
+class ReplayBufferSet:
+    """The buffers of the `replay_buffer` section of an algorithm config, as MSRL holds them
+    (mindspore_rl/core/msrl.py:407-421):
+
+    * a plain entry builds `buffers` (one buffer, or a list when `number` > 1); for a single buffer its
+      sample / insert / full / reset are bound as `replay_buffer_sample`, `replay_buffer_insert`,
+      `replay_buffer_full`, `replay_buffer_reset`, the names the trainers call
+      (mindspore_rl/algorithm/dqn/dqn_trainer.py:80,83);
+    * a section with a true `multi_type_replaybuffer` holds one entry per name; `buffers` is then a dict
+      name -> buffer(s) and nothing is bound.
+    """
+
+    _HANDLERS = ("sample", "insert", "full", "reset")
+
+    def __init__(self, section):
+        if not isinstance(section, dict):
+            raise TypeError("the replay_buffer section is a dict, got %s" % type(section).__name__)
+        if section.get("multi_type_replaybuffer"):
+            self.buffers = {name: create_replay_buffer(entry) for name, entry in section.items()
+                            if name != "multi_type_replaybuffer"}
+            return
+        entry = {k: v for k, v in section.items() if k != "multi_type_replaybuffer"}
+        self.buffers = create_replay_buffer(entry)
+        if not isinstance(self.buffers, list):
+            for name in self._HANDLERS:
+                setattr(self, "replay_buffer_" + name, getattr(self.buffers, name))

@@ -170,6 +170,43 @@ def test_create_replay_buffer_follows_the_reference_config_entry():
         create_replay_buffer(dict(cfg, number=0))
 
 
+def test_replay_buffer_set_binds_the_handlers_msrl_binds():
+    """mindspore_rl/core/msrl.py:407-421: one buffer -> replay_buffer_sample/insert/full/reset bound to it;
+    `number` > 1 -> a list and nothing bound; `multi_type_replaybuffer` -> a dict of named buffers."""
+    from mindrl_amd.core import ReplayBufferSet
+
+    class Fake:
+        def __init__(self, sample_size, capacity, shapes, types):
+            self.capacity, self.rows = capacity, []
+
+        def insert(self, row):
+            self.rows.append(row)
+
+        def sample(self):
+            return self.rows[-1]
+
+        def full(self):
+            return len(self.rows) >= self.capacity
+
+        def reset(self):
+            self.rows = []
+
+    entry = {"number": 1, "type": Fake, "capacity": 2, "sample_size": 1, "data_shape": [(1,)], "data_type": ["int32"]}
+    one = ReplayBufferSet(entry)
+    one.replay_buffer_insert(5), one.replay_buffer_insert(6)
+    assert one.replay_buffer_sample() == 6 and one.replay_buffer_full() and isinstance(one.buffers, Fake)
+    one.replay_buffer_reset()
+    assert one.buffers.rows == []
+    assert isinstance(ReplayBufferSet({k: v for k, v in entry.items() if k != "number"}).buffers, Fake)  # number defaults to 1
+    several = ReplayBufferSet(dict(entry, number=2))
+    assert isinstance(several.buffers, list) and len(several.buffers) == 2 and not hasattr(several, "replay_buffer_sample")
+    named = ReplayBufferSet({"multi_type_replaybuffer": True, "policy": entry, "expert": dict(entry, capacity=9)})
+    assert set(named.buffers) == {"policy", "expert"} and named.buffers["expert"].capacity == 9
+    assert not hasattr(named, "replay_buffer_insert")
+    with pytest.raises(TypeError):
+        ReplayBufferSet([entry])
+
+
 def test_bench_refuses_more_than_one_gpu():
     """Every box has one GPU: `bench.py --gpus N` with N > 1 exits non-zero with a message, before touching a device."""
     import subprocess
