@@ -23,7 +23,8 @@
  *   - `stream` is a hipStream_t (NULL = the null stream). All device work is
  *     enqueued on it in program order. Only *_create, *_destroy, mrb_per_state
  *     (when the running max is asked for), *_check and mrb_per_export_tree wait
- *     for the device; only *_create allocates device memory, with one exception:
+ *     for the device (and, around the option "device_counters", what mrb_set_option
+ *     says there); only *_create allocates device memory, with one exception:
  *     an mrb_per_update of more entries than the buffer has rows and than any
  *     earlier call had enlarges its scratch (hipMalloc; nothing is freed before
  *     *_destroy). Calls that change one handle must be serialised by the caller
@@ -37,7 +38,8 @@
  *     a replayed sample without `uniforms` draws the numbers it drew then. mrb_per_gather and an
  *     mrb_per_update of at most 1024 entries replay correctly against whatever the buffer holds at replay
  *     time; so does mrb_per_sample with `uniforms` while the number of stored rows is what it was when
- *     recorded (a full buffer).
+ *     recorded (a full buffer). With the option "device_counters" (mrb_set_option) the counters live on the
+ *     device and a recorded push / sample / update loop replays as the same calls made again would run.
  *   - storage is structure-of-arrays: field i is one [capacity, field_bytes[i]]
  *     byte matrix (reference layout: uniform_replay_buffer.py:26-47).
  */
@@ -78,6 +80,16 @@ int mrb_version(void);
  *   "row_split"    least number of workgroups per row in the wide-row kernel (0 = auto, max 64)
  *   "sample_path"  prioritized buffers: 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
  *   "lds_levels"   prioritized buffers: tree levels staged in LDS by the LDS-top kernel (0 = auto, max 12)
+ *   "device_counters" prioritized buffers: 1 = the ring position, the number of stored rows and the generator's
+ *                  call counter are kept in device memory, read there by the kernels and advanced there by
+ *                  a one-thread kernel after every push and every generator-driven sample - for callers that
+ *                  record push / sample / update into a HIP graph: every replay then continues where the last
+ *                  one stopped (pushes land in the next slots, draws differ, weights use the current row
+ *                  count). While it is on: a push takes at most `capacity` rows, an update at most 1024
+ *                  entries, a generator-driven sample at most max(4096, min(capacity, 2^20)) rows, sample
+ *                  calls on one handle must not overlap (they share a scratch array), and mrb_per_state and
+ *                  the checkpoint calls wait for the device to read the counters back. Switching it (either
+ *                  way) waits for the device. 0 (default) = host-side counters, passed as kernel arguments.
  *   "fused_rebuild" prioritized buffers: 1 (default) = an update of <= 32 entries or a push under <= 32 leaf tiles
  *                  rebuilds the tree in one launch where the tree has one round of levels below its top;
  *                  0 = one launch per round */

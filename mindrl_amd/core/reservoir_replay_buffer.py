@@ -104,7 +104,8 @@ class ReservoirReplayBuffer:
 
     def set_option(self, name, value):
         """Sets a launch option of this buffer ("row_split"; prioritized buffers also "sample_path",
-        "lds_levels", "fused_rebuild"). Options change how kernels are launched, never a result."""
+        "lds_levels", "fused_rebuild", "device_counters"). Options change how kernels are launched, never a
+        result."""
         _lib.set_option(self._h, name, value)
 
     def __del__(self):

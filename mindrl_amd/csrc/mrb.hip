@@ -345,6 +345,8 @@ struct Per {
     int64_t sample_path = 0;  // option "sample_path": 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
     int64_t lds_levels = 0;   // option "lds_levels": tree levels staged in LDS by the LDS-top kernel (0 = auto)
     int64_t fused = 1;        // option "fused_rebuild": small updates and pushes rebuild the tree in one launch
+    int64_t* counters = nullptr;   // device copy of pushes / size / calls (Counters in mrb_kernels.h)
+    int64_t device_counters = 0;   // option "device_counters": kernels read the counters from the device
     ~Per() {
         if (sum) (void)hipFree(sum);
         if (mn) (void)hipFree(mn);
@@ -416,6 +418,14 @@ int read_and_clear_flags(uint32_t* d_err, uint32_t* flags, hipStream_t s) {
     return MRB_OK;
 }
 
+// Leaf tiles that n consecutive slots of the ring can meet wherever they start: ceil(n / 256) + 1 for the
+// misalignment, one more where the slots wrap around the ring's end; never more than the ring's tiles.
+uint32_t push_units(const UpdateArgs& a) {
+    const uint64_t ring_tiles = ((uint64_t)a.capacity + kBlockNodes - 1) / kBlockNodes;
+    const uint64_t units = ((uint64_t)a.n + kBlockNodes - 1) / kBlockNodes + 2;
+    return (uint32_t)(units < ring_tiles ? units : ring_tiles);
+}
+
 // Rebuilds the tree above the leaves that `a` writes: one launch per round, then the top. A push hands
 // its row copy over (`ride`): it is done by extra workgroups of the first launch.
 int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = nullptr) {
@@ -435,6 +445,8 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
         uint32_t units = 0, tile_base = 0;
         if (a.inline_election) {
             units = (uint32_t)a.n;
+        } else if (!a.indices && a.first_slot < 0) {
+            units = push_units(a);  // the slots' start is only known on the device
         } else if (!a.indices && a.first_slot + a.n <= a.capacity) {
             tile_base = (uint32_t)(a.first_slot / kBlockNodes);
             units = (uint32_t)((a.first_slot + a.n - 1) / kBlockNodes) - tile_base + 1;
@@ -450,7 +462,12 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
     for (int r = 0; r < a.nrounds; ++r) {
         uint32_t tiles = (1u << a.lo[r]) / kBlockNodes;
         uint32_t tile_base = 0;
-        if (r == 0 && !a.indices && a.first_slot + a.n <= a.capacity) {
+        if (r == 0 && !a.indices && a.first_slot < 0) {
+            // a push whose first slot only the device knows: enough waves for every tile the slots can meet;
+            // the kernel places them (tile_base carries their number)
+            tiles = push_units(a);
+            tile_base = tiles;
+        } else if (r == 0 && !a.indices && a.first_slot + a.n <= a.capacity) {
             // a push that does not wrap: only the leaf tiles under its slot range need a wave
             tile_base = (uint32_t)(a.first_slot / kBlockNodes);
             tiles = (uint32_t)((a.first_slot + a.n - 1) / kBlockNodes) - tile_base + 1;
@@ -558,6 +575,27 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
 }
 
 
+// Device-resident counters: host -> device (when the option is switched on, after a load) and back (state
+// queries, when it is switched off). Both wait for the device.
+int counters_to_device(Per& b) {
+    const int64_t v[4] = {b.pushes, b.size, (int64_t)b.calls, 0};
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(b.counters, v, sizeof(v), hipMemcpyHostToDevice));
+    return MRB_OK;
+}
+int counters_from_device(Per& b) {
+    int64_t v[4];
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(v, b.counters, sizeof(v), hipMemcpyDeviceToHost));
+    b.pushes = v[kCntPushes], b.size = v[kCntSize], b.calls = (uint64_t)v[kCntCalls];
+    return MRB_OK;
+}
+int counters_advance(Per& b, int64_t pushed, int64_t calls, hipStream_t s) {
+    hipLaunchKernelGGL(k_counters_advance, dim3(1), dim3(64), 0, s, b.counters, pushed, b.rows.capacity, calls);
+    LAUNCH_CHECK("k_counters_advance");
+    return MRB_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -587,6 +625,14 @@ int mrb_set_option(int64_t h, const char* name, int64_t value) {
         if (!per) return fail(MRB_EINVAL, "lds_levels is an option of prioritized buffers");
         if (value < 0 || value > 12) return fail(MRB_EINVAL, "lds_levels must be in [0, 12]");
         per->lds_levels = value;
+    } else if (!strcmp(name, "device_counters")) {
+        if (!per) return fail(MRB_EINVAL, "device_counters is an option of prioritized buffers");
+        if (value < 0 || value > 1) return fail(MRB_EINVAL, "device_counters must be 0 or 1");
+        if (value != per->device_counters) {
+            const int rc = value ? counters_to_device(*per) : counters_from_device(*per);
+            if (rc) return rc;
+            per->device_counters = value;
+        }
     } else if (!strcmp(name, "fused_rebuild")) {
         if (!per) return fail(MRB_EINVAL, "fused_rebuild is an option of prioritized buffers");
         if (value < 0 || value > 1) return fail(MRB_EINVAL, "fused_rebuild must be 0 or 1");
@@ -786,7 +832,10 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->mn), nodes * sizeof(float)));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->stamp), (size_t)b->leaves * sizeof(unsigned long long)));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->maxp), 16));
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16));
+    // one allocation: the error word (16 bytes), then the device copy of the counters (kernels find them there)
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16 + 4 * sizeof(int64_t)));
+    b->counters = reinterpret_cast<int64_t*>(b->err + 4);
+    HIP_TRY(hipMemset(b->counters, 0, 4 * sizeof(int64_t)));
     // update_priorities scratch, sized once: a call rarely names more entries than there are rows
     b->powered_cap = capacity < 4096 ? 4096 : (capacity > (1ll << 20) ? (1ll << 20) : capacity);
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->powered), (size_t)b->powered_cap * sizeof(float)));
@@ -835,12 +884,18 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     if (nrows > 0x7fffffffll) return fail(MRB_EINVAL, "nrows %lld exceeds 2^31 - 1 rows per call", (long long)nrows);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t cap = b->rows.capacity;
+    if (b->device_counters && nrows > cap)
+        return fail(MRB_ESTATE, "with device_counters a push takes at most capacity (%lld) rows", (long long)cap);
     const int64_t skip = nrows > cap ? nrows - cap : 0;  // rows overwritten within this very call
     const int64_t n = nrows - skip;
     const int64_t first = (b->pushes + skip) % cap;
     PutArgs put{};
     int rc = put_args(b->rows, src_fields, skip, n, first, put);
     if (rc) return rc;
+    if (b->device_counters) {  // the kernels take the first slot from the device
+        put.first_slot = -1;
+        put.src_first = reinterpret_cast<int64_t>(b->counters);
+    }
     if (put.blocks > 2048) {
         // a large copy gets its own launch; a small one rides along in the first tree launch
         hipLaunchKernelGGL(k_rows_put, dim3(put.blocks), dim3(kWG), 0, s, put);
@@ -860,7 +915,7 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
         a.priorities = opt_priorities + skip;
         a.fold_max = fold;
     }
-    a.first_slot = first;
+    a.first_slot = b->device_counters ? -1 : first;
     a.n = n;
     rc = tree_rebuild(*b, a, s, put.blocks ? &put : nullptr);
     if (rc) return rc;
@@ -869,6 +924,10 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
         a.n = nrows;
         hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)nrows)), dim3(kWG), 0, s, a);
         LAUNCH_CHECK("k_update_stamp");
+    }
+    if (b->device_counters) {
+        rc = counters_advance(*b, nrows, 0, s);
+        if (rc) return rc;
     }
     b->pushes += nrows;
     b->size = b->size + nrows < cap ? b->size + nrows : cap;
@@ -880,6 +939,9 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
     if (n > 0xffffffffll) return fail(MRB_EINVAL, "n %lld exceeds 2^32 - 1 entries per call", (long long)n);
     if (!indices || !priorities) return fail(MRB_EINVAL, "indices or priorities is NULL");
+    if (b->device_counters && n > 1024)
+        return fail(MRB_ESTATE, "with device_counters an update takes at most 1024 entries (larger ones elect their "
+                                "entries with tags the host counts, which a graph replay would repeat)");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (n > b->powered_cap) {
         // more entries than any call so far (and than the capacity): a larger array, at least twice the
@@ -938,6 +1000,21 @@ static int per_sample_impl(Per* b, int64_t nbatch, int64_t batch, float beta, co
     a.out_idx = out_indices;
     a.out_w = out_weights;
     a.err = b->err;
+    if (b->device_counters) {
+        a.size = -1;  // the kernels take the number of stored rows from the device
+        if (!uniforms) {
+            // the generator's call counter is on the device: its draws are written out first (into the scratch
+            // update_priorities uses; calls on one handle are ordered) and the sample kernel reads them
+            if (nbatch * batch > b->powered_cap)
+                return fail(MRB_ESTATE, "with device_counters a generator-driven sample takes at most %lld rows",
+                            (long long)b->powered_cap);
+            hipLaunchKernelGGL(k_fill_uniforms, dim3(grid_exact((uint64_t)(nbatch * batch))), dim3(kWG), 0, s, b->powered,
+                               b->seed, b->counters, batch, nbatch);
+            LAUNCH_CHECK("k_fill_uniforms");
+            a.uniforms = b->powered;
+        }
+    }
+    const float* const draws = a.uniforms;  // the caller's, the written-out generator's, or NULL
     const int64_t max_bytes = widest_field(b->rows);
     int path = (int)b->sample_path;
     if (path == 0) path = (batch >= 8192 && max_bytes <= 256) ? 2 : 1;
@@ -949,11 +1026,11 @@ static int per_sample_impl(Per* b, int64_t nbatch, int64_t batch, float beta, co
         int levels = b->lds_levels > 0 ? (int)b->lds_levels : 9;
         if (levels > b->depth) levels = b->depth;
         const uint32_t ntop = (2u << levels) < 4 ? 4 : (2u << levels);
-        const size_t lds = ntop * sizeof(float) + kWG * sizeof(int64_t);
+        const size_t lds = ntop * sizeof(float) + (kWG + 1) * sizeof(int64_t);
         for (int64_t i = 0; i < nbatch; ++i) {
             SampleArgs ai = a;
             IoTable ti = t;
-            ai.uniforms = uniforms ? uniforms + i * batch : nullptr;
+            ai.uniforms = draws ? draws + i * batch : nullptr;
             ai.calls = a.calls + (uint64_t)i;
             ai.out_idx = out_indices + i * batch;
             ai.out_w = out_weights + i * batch;
@@ -963,7 +1040,10 @@ static int per_sample_impl(Per* b, int64_t nbatch, int64_t batch, float beta, co
             LAUNCH_CHECK("k_per_sample_lds");
         }
     }
-    if (!uniforms) b->calls += (uint64_t)nbatch;
+    if (!uniforms) {
+        b->calls += (uint64_t)nbatch;
+        if (b->device_counters) return counters_advance(*b, 0, nbatch, s);
+    }
     return MRB_OK;
 }
 
@@ -1003,6 +1083,10 @@ int mrb_per_export_tree(int64_t h, float* sum_heap, float* min_heap, int64_t* le
 
 int mrb_per_state(int64_t h, int64_t* size, int64_t* head, float* max_priority, void* stream) {
     GET_PER(b, h);
+    if (b->device_counters) {  // the device's counters are the current ones (a graph replay advances only them)
+        const int rc = counters_from_device(*b);
+        if (rc) return rc;
+    }
     if (size) *size = b->size;
     if (head) *head = b->pushes % b->rows.capacity;
     if (max_priority) {
@@ -1147,6 +1231,10 @@ int mrb_urb_set_counters(int64_t h, const int64_t* in4) {
 int mrb_per_get_counters(int64_t h, int64_t* out4) {
     GET_PER(b, h);
     if (!out4) return fail(MRB_EINVAL, "out4 is NULL");
+    if (b->device_counters) {
+        const int rc = counters_from_device(*b);
+        if (rc) return rc;
+    }
     out4[0] = b->size, out4[1] = b->pushes, out4[2] = (int64_t)b->seed, out4[3] = (int64_t)b->calls;
     return MRB_OK;
 }
@@ -1160,7 +1248,7 @@ int mrb_per_set_counters(int64_t h, const int64_t* in4) {
         return fail(MRB_EINVAL, "size %lld does not follow from %lld pushes into capacity %lld", (long long)in4[0],
                     (long long)in4[1], (long long)cap);
     b->size = in4[0], b->pushes = in4[1], b->seed = (uint64_t)in4[2], b->calls = (uint64_t)in4[3];
-    return MRB_OK;
+    return b->device_counters ? counters_to_device(*b) : MRB_OK;
 }
 
 int mrb_res_get_counters(int64_t h, int64_t* out4) {

@@ -137,19 +137,40 @@ struct PutArgs {
     IoTable t;
     int64_t capacity, first_slot, src_capacity, src_first;
     uint32_t blocks;  // workgroups doing this copy when it rides along in another kernel's launch (0: none)
+    // first_slot < 0: the buffer's counters live on the device (see Counters below), the rows go to
+    // (pushes mod capacity) onwards, and src_first - unused then, the source is never a ring - holds the
+    // counters' address
 };
+
+// A prioritized buffer's counters as device memory, for callers that record their loop into a HIP
+// graph: kernels then take the ring position, the number of stored rows and the generator's call
+// counter from here, and a one-thread kernel advances them after each call, so that every replay
+// continues where the one before stopped.
+// Kernels are told through a negative first slot / row count in their arguments and find the counters
+// behind the buffer's error word (one allocation: 16 bytes of flags, then the counters), so that the
+// arguments of the ordinary case are what they were.
+constexpr int kCntPushes = 0, kCntSize = 1, kCntCalls = 2;
+
+__device__ __forceinline__ const int64_t* counters_behind(const uint32_t* err) {
+    return reinterpret_cast<const int64_t*>(err + 4);
+}
+__device__ __forceinline__ int64_t ring_position(const int64_t* counters, int64_t capacity) {
+    return (int64_t)((uint64_t)counters[kCntPushes] % (uint64_t)capacity);
+}
 
 // The copy itself, by workgroup `block` of `nblocks` (grid-stride over the granules).
 __device__ __forceinline__ void rows_put_part(const PutArgs& p, uint32_t block, uint32_t nblocks) {
     const IoTable& t = p.t;
     const uint64_t total = t.prefix[t.nfields];
     const uint64_t stride = (uint64_t)nblocks * blockDim.x;
+    const int64_t first_slot =
+        p.first_slot >= 0 ? p.first_slot : ring_position(reinterpret_cast<const int64_t*>(p.src_first), p.capacity);
     for (uint64_t w = (uint64_t)block * blockDim.x + threadIdx.x; w < total; w += stride) {
         const int f = field_of(t, w);
         uint64_t row;
         uint32_t unit;
         split_work(w - t.prefix[f], t.units[f], row, unit);
-        int64_t slot = p.first_slot + (int64_t)row;
+        int64_t slot = first_slot + (int64_t)row;
         if (slot >= p.capacity) slot -= p.capacity;
         uint64_t src_row = row;
         if (p.src_capacity > 0) {
@@ -252,7 +273,7 @@ struct SampleArgs {
     uint64_t seed, calls;
     int64_t leaves;
     int64_t capacity;
-    int64_t size;
+    int64_t size;           // rows stored; negative: read from the device (see Counters)
     const float* mn;        // min tree, heap order
     int64_t* out_idx;
     float* out_w;
@@ -274,9 +295,9 @@ __device__ __forceinline__ float is_weight(float p, float total, float pmin, flo
     return powf_det(p / total * fsize, -beta) / max_w;
 }
 
-__device__ __forceinline__ void sample_flags(const SampleArgs& a, float total, int64_t idx) {
+__device__ __forceinline__ void sample_flags(const SampleArgs& a, float total, int64_t idx, int64_t size) {
     if (!(total > 0.0f) || total > 3.0e38f) atomicOr(a.err, MRB_DERR_TOTAL);
-    if (idx >= a.size) atomicOr(a.err, MRB_DERR_UNFILLED);
+    if (idx >= size) atomicOr(a.err, MRB_DERR_UNFILLED);
 }
 
 // ---------------------------------------------------------------------------
@@ -338,7 +359,7 @@ struct SampleTail {
     int64_t* out_idx;
     float* out_w;
     uint32_t* err;
-    int64_t size;
+    int64_t size;  // rows stored; negative: read from the device (see Counters)
     float beta;
 };
 
@@ -693,7 +714,9 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
     if (part != 0) return;
     // lane 0: (p / total * size)^-beta, lane 1: (pmin / total * size)^-beta
     const float total = s_total;
-    const float fsize = (float)s_tail.size;
+    int64_t size = s_tail.size;
+    if (size < 0) size = counters_behind(s_tail.err)[kCntSize];  // device-resident counters (see Counters)
+    const float fsize = (float)size;
     const float x = lane == 0 ? s_picked : s_pmin;
     float r = 0.0f;
     if (lane < 2) r = powf_det_call(x / total * fsize, -s_tail.beta);
@@ -702,7 +725,7 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
         s_tail.out_idx[k] = idx;
         s_tail.out_w[k] = r / max_w;
         if (!(total > 0.0f) || total > 3.0e38f) atomicOr(s_tail.err, MRB_DERR_TOTAL);
-        if (idx >= s_tail.size) atomicOr(s_tail.err, MRB_DERR_UNFILLED);
+        if (idx >= size) atomicOr(s_tail.err, MRB_DERR_UNFILLED);
     }
     MRB_TS(ts_wend);
     MRB_TS_OUT(1, ts_start);
@@ -777,8 +800,10 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
     if (threadIdx.x >= kWG) {
         // The helper wave: the weights' common denominator (pmin / total * size)^-beta, once per
         // workgroup, off the strata's path (two loads and a power: as long as staging the top).
+        // (the number of stored rows: the argument, or read from the device when the counters live there)
+        if (threadIdx.x == kWG) s_slot[kWG] = a.size >= 0 ? a.size : counters_behind(a.err)[kCntSize];
         __syncthreads();
-        if (threadIdx.x == kWG) s_max_w = powf_det(mn[1] / sum[1] * (float)a.size, -beta);
+        if (threadIdx.x == kWG) s_max_w = powf_det(mn[1] / sum[1] * (float)s_slot[kWG], -beta);
         __syncthreads();
         return;
     }
@@ -912,8 +937,9 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
             if (f < t.nfields && t.units[f] == 1)
                 own[f].load(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f], t.vec_log2[f]);
         a.out_idx[k] = idx;
-        weight = powf_det(picked / total * (float)a.size, -beta);
-        sample_flags(a, total, idx);
+        const int64_t size = s_slot[kWG];  // left there by the helper wave before the first barrier
+        weight = powf_det(picked / total * (float)size, -beta);
+        sample_flags(a, total, idx, size);
         s_slot[threadIdx.x] = slot;
     }
     MRB_TS(ts4);
@@ -984,7 +1010,7 @@ struct UpdateArgs {
     const int64_t* indices;   // NULL: entry j targets slot (first_slot + j) mod capacity
     const float* priorities;  // NULL: the targeted leaves take the running max priority as it is
     int64_t n;
-    int64_t first_slot;
+    int64_t first_slot;       // negative: (pushes mod capacity), read from the device (see Counters)
     // buffer
     int64_t capacity;
     int64_t leaves;
@@ -1049,7 +1075,7 @@ __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
 //   range + priorities: entry (leaf - first_slot) mod capacity; an invalid priority leaves the
 //                   fresh slot at the running max, as a plain push would
 //   range only:     the running max priority
-__device__ __forceinline__ bool leaf_value(const UpdateArgs& a, int64_t leaf, float& q) {
+__device__ __forceinline__ bool leaf_value(const UpdateArgs& a, int64_t first_slot, int64_t leaf, float& q) {
     if (a.indices) {
         const unsigned long long st = a.stamp[leaf];
         if ((uint32_t)(st >> 32) != a.epoch) return false;
@@ -1057,7 +1083,7 @@ __device__ __forceinline__ bool leaf_value(const UpdateArgs& a, int64_t leaf, fl
         return true;
     }
     if (leaf >= a.capacity) return false;
-    int64_t j = leaf - a.first_slot;
+    int64_t j = leaf - first_slot;
     if (j < 0) j += a.capacity;
     if (j >= a.n) return false;
     if (a.priorities) {
@@ -1072,9 +1098,9 @@ __device__ __forceinline__ bool leaf_value(const UpdateArgs& a, int64_t leaf, fl
 }
 
 // Does the pushed slot range [first_slot, first_slot + n) mod capacity meet leaves [lo, hi)?
-__device__ __forceinline__ bool range_meets(const UpdateArgs& a, int64_t lo, int64_t hi) {
-    const int64_t end = a.first_slot + a.n;
-    if (lo < (end < a.capacity ? end : a.capacity) && hi > a.first_slot) return true;
+__device__ __forceinline__ bool range_meets(const UpdateArgs& a, int64_t first_slot, int64_t lo, int64_t hi) {
+    const int64_t end = first_slot + a.n;
+    if (lo < (end < a.capacity ? end : a.capacity) && hi > first_slot) return true;
     return end > a.capacity && lo < end - a.capacity;
 }
 
@@ -1124,18 +1150,21 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
                                            int g_next, uint32_t lane, int* win = nullptr) {
     const uint32_t level_nodes = 1u << lo;
     const bool leaf_level = lo == a.depth;
+    // where a push's slots start (a.first_slot, or read from the device)
+    const int64_t first_slot =
+        !leaf_level || a.indices ? 0 : a.first_slot >= 0 ? a.first_slot : ring_position(counters_behind(a.err), a.capacity);
     if (level_nodes < 4) {
         // one or two nodes: scalar, lane 0
         if (lane == 0) {
             float s0 = a.sum[level_nodes], m0 = a.mn[level_nodes], q;
-            if (leaf_level && leaf_value(a, 0, q)) {
+            if (leaf_level && leaf_value(a, first_slot, 0, q)) {
                 s0 = m0 = q;
                 a.sum[level_nodes] = q;
                 a.mn[level_nodes] = q;
             }
             if (level_nodes == 2) {
                 float s1 = a.sum[3], m1 = a.mn[3];
-                if (leaf_level && leaf_value(a, 1, q)) {
+                if (leaf_level && leaf_value(a, first_slot, 1, q)) {
                     s1 = m1 = q;
                     a.sum[3] = q;
                     a.mn[3] = q;
@@ -1193,7 +1222,7 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
             active = dirty_in[off >> g] == a.epoch;
         } else if (leaf_level && !a.indices) {
             const int64_t b0 = (int64_t)(off >> g) << g;
-            active = range_meets(a, b0, b0 + (1ll << g));
+            active = range_meets(a, first_slot, b0, b0 + (1ll << g));
         }
     }
     float4 vs = make_float4(0.f, 0.f, 0.f, 0.f), vm = vs;
@@ -1209,10 +1238,10 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
                 if (jw2 >= 0) { vs.z = vm.z = powf_det_call(a.priorities[jw2], a.alpha); wrote = true; }
                 if (jw3 >= 0) { vs.w = vm.w = powf_det_call(a.priorities[jw3], a.alpha); wrote = true; }
             } else {
-                if (leaf_value(a, off + 0, q)) { vs.x = vm.x = q; wrote = true; }
-                if (leaf_value(a, off + 1, q)) { vs.y = vm.y = q; wrote = true; }
-                if (leaf_value(a, off + 2, q)) { vs.z = vm.z = q; wrote = true; }
-                if (leaf_value(a, off + 3, q)) { vs.w = vm.w = q; wrote = true; }
+                if (leaf_value(a, first_slot, off + 0, q)) { vs.x = vm.x = q; wrote = true; }
+                if (leaf_value(a, first_slot, off + 1, q)) { vs.y = vm.y = q; wrote = true; }
+                if (leaf_value(a, first_slot, off + 2, q)) { vs.z = vm.z = q; wrote = true; }
+                if (leaf_value(a, first_slot, off + 3, q)) { vs.w = vm.w = q; wrote = true; }
             }
             if (wrote) {
                 *reinterpret_cast<float4*>(a.sum + first + 4 * lane) = vs;
@@ -1276,10 +1305,10 @@ __global__ __launch_bounds__(kWG) void k_tree_sparse(UpdateArgs a) {
         const int64_t leaf0 = (int64_t)((block << g0) + 4 * sub);
         float q;
         bool wrote = false;
-        if (leaf_value(a, leaf0 + 0, q)) { vs.x = vm.x = q; wrote = true; }
-        if (leaf_value(a, leaf0 + 1, q)) { vs.y = vm.y = q; wrote = true; }
-        if (leaf_value(a, leaf0 + 2, q)) { vs.z = vm.z = q; wrote = true; }
-        if (leaf_value(a, leaf0 + 3, q)) { vs.w = vm.w = q; wrote = true; }
+        if (leaf_value(a, 0, leaf0 + 0, q)) { vs.x = vm.x = q; wrote = true; }
+        if (leaf_value(a, 0, leaf0 + 1, q)) { vs.y = vm.y = q; wrote = true; }
+        if (leaf_value(a, 0, leaf0 + 2, q)) { vs.z = vm.z = q; wrote = true; }
+        if (leaf_value(a, 0, leaf0 + 3, q)) { vs.w = vm.w = q; wrote = true; }
         if (wrote) {
             *reinterpret_cast<float4*>(a.sum + first + 4 * sub) = vs;
             *reinterpret_cast<float4*>(a.mn + first + 4 * sub) = vm;
@@ -1469,6 +1498,14 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
         entry_duty(a, j, (uint32_t)a.n, lane);
         return;
     }
+    if (round == 0 && !a.indices && a.first_slot < 0) {
+        // a push whose slots start at a position only the device knows: the launch brings enough waves for the
+        // tiles the slots can meet; they start at the tile of the first slot and wrap around the level
+        const uint32_t unit = blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
+        if (unit >= tile_base) return;  // tile_base carries the number of such waves here
+        const uint32_t ring_tiles = (uint32_t)((a.capacity + kBlockNodes - 1) / kBlockNodes);  // the ring ends at `capacity`
+        tile = ((uint32_t)(ring_position(counters_behind(a.err), a.capacity) / kBlockNodes) + unit) % ring_tiles;
+    }
     if (tile >= ntiles) return;
     tile_round(a, lo, g, tile, true, (elect || (round == 0 && !a.indices)) ? nullptr : a.dirty[round],
                last_round ? nullptr : a.dirty[round + 1], last_round ? 0 : a.g[round + 1], lane,
@@ -1516,7 +1553,11 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
             entry_tile(a, a.g[0], unit, lane, s_win[wave], nullptr, 0);
             entry_duty(a, unit, units, lane);
         } else {
-            tile_round(a, a.lo[0], a.g[0], tile_base + unit, true, nullptr, nullptr, 0, lane);
+            // (device-resident counters: the tiles start at the first slot's tile and wrap around the level)
+            const uint32_t ring_tiles = (uint32_t)((a.capacity + kBlockNodes - 1) / kBlockNodes);  // the ring ends at `capacity`
+            const uint32_t tile = a.first_slot >= 0 ? tile_base + unit
+                                                    : ((uint32_t)(ring_position(counters_behind(a.err), a.capacity) / kBlockNodes) + unit) % ring_tiles;
+            tile_round(a, a.lo[0], a.g[0], tile, true, nullptr, nullptr, 0, lane);
         }
     }
     __threadfence_block();  // the tiles' highest nodes, written by other waves of this workgroup, are read below
@@ -1719,6 +1760,28 @@ __global__ __launch_bounds__(kDrWG) void k_discounted_return_tiled(const float* 
         }
         lds_barrier();
     }
+}
+
+// Device-resident counters (see Counters): after a push, and after a sample that used the generator.
+__global__ void k_counters_advance(int64_t* counters, int64_t pushed, int64_t capacity, int64_t calls) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        if (pushed) {
+            counters[kCntPushes] += pushed;
+            const int64_t size = counters[kCntSize] + pushed;
+            counters[kCntSize] = size < capacity ? size : capacity;
+        }
+        counters[kCntCalls] += calls;
+    }
+}
+
+// The generator's draws for `nbatch` batches, written out for a sample kernel to read: with the call
+// counter on the device the kernel cannot take it as an argument.
+__global__ __launch_bounds__(kWG) void k_fill_uniforms(float* dst, uint64_t seed, const int64_t* counters, int64_t batch,
+                                                       int64_t nbatch) {
+    const int64_t i = (int64_t)blockIdx.x * kWG + threadIdx.x;
+    if (i >= batch * nbatch) return;
+    const int64_t nth = i / batch;
+    dst[i] = rng_uniform(seed, (uint64_t)counters[kCntCalls] + (uint64_t)nth, (uint64_t)(i - nth * batch));
 }
 
 // Fills a float array with one value (tree initialisation: sums 0, mins FLT_MAX).

@@ -195,6 +195,61 @@ def test_hip_graph_replays_update_and_sample(mrb, orc, path):
     g.destroy()
 
 
+@pytest.mark.parametrize("cap", [3000, 70000])
+def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap):
+    """push 3 rows + generator-driven sample + update_priorities of the sampled rows, recorded ONCE with the
+    option device_counters and replayed 12 times on new rows and priorities: the buffer fills up, the ring wraps,
+    the draws advance - every replay equals the oracle's push, sample, update; eager calls between replays keep
+    working, and the counters read back agree."""
+    rng = np.random.default_rng(cap)
+    shapes, dtypes = [(300,), (1,), (2,)], [np.float32, np.int32, np.uint8]
+    batch, npush = 48, 3
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=13, shapes=shapes, dtypes=dtypes)
+    fill = cap - 20  # not full: the row count changes during the replays, then the ring wraps
+    rows = random_rows(rng, fill, shapes, dtypes)
+    g.insert(*to_dev(rows)), c.push(rows, fill)
+    g.set_option("device_counters", 1)
+    new_rows = [torch.zeros((npush,) + tuple(s), dtype=t).cuda() for s, t in zip(shapes, torch_types(dtypes))]
+    pr_dev = torch.ones(batch, dtype=torch.float32, device="cuda")
+    out = (torch.empty(batch, dtype=torch.int64, device="cuda"), torch.empty(batch, dtype=torch.float32, device="cuda"),
+           g._layout.empty(batch, g._dev))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        g.insert(*new_rows)
+        g.sample(0.5, out=out)
+        g.update_priorities(out[0], pr_dev)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for rep in range(12):
+        fresh = random_rows(rng, npush, shapes, dtypes)
+        pr = (rng.pareto(1.5, batch) + 1e-6).astype(np.float32)
+        for dst, src in zip(new_rows, fresh):
+            dst.copy_(torch.from_numpy(src))
+        pr_dev.copy_(torch.from_numpy(pr))
+        graph.replay()
+        torch.cuda.synchronize()
+        c.push(fresh, npush)
+        want = c.sample(batch, 0.5)
+        assert_sample_equal((out[0], out[1]) + tuple(out[2]), want, "cap %d replay %d" % (cap, rep))
+        c.update(want[0], pr)
+        assert_tree_equal(g, c, "cap %d replay %d" % (cap, rep))
+        assert g.size() == c.size and g._state()[1] == c.head
+        if rep % 3 == 1:  # eager calls in between use the same counters
+            extra = random_rows(rng, 5, shapes, dtypes)
+            g.insert(*to_dev(extra)), c.push(extra, 5)
+            assert_sample_equal(g.sample(0.9), c.sample(batch, 0.9), "eager after replay %d" % rep)
+    with pytest.raises(ValueError):
+        g.update_priorities(torch.zeros(2000, dtype=torch.int64).cuda(), torch.ones(2000).cuda())
+    g.set_option("device_counters", 0)
+    assert g.size() == c.size
+    assert_sample_equal(g.sample(0.3), c.sample(batch, 0.3), "after switching back")
+    del graph
+    g.destroy()
+
+
 def test_sample_output_ring(mrb, orc):
     """sample() hands out preallocated output sets in turn: `output_ring` calls return distinct tensors, the
     next call reuses the first set; output_ring=0 allocates fresh tensors; an explicit out= is written in

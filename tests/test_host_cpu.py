@@ -100,7 +100,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
     assert sum("k_per_sample_wide" in k for k in kernels) == 8 and sum("k_rows_gather_wide" in k for k in kernels) == 4
-    assert len(kernels) == 25, sorted(kernels)
+    assert len(kernels) == 27, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)
@@ -123,7 +123,8 @@ def test_only_the_documented_entry_points_wait_or_allocate():
     waits = re.compile(r"hipDeviceSynchronize|hipStreamSynchronize|hipEventSynchronize|hipMemcpy\(")
     allocs = re.compile(r"hipMalloc|hipFree|hipHostMalloc")
     may_wait = {"mrb_urb_create", "mrb_per_create", "mrb_res_create", "mrb_urb_destroy", "mrb_per_destroy",
-                "mrb_res_destroy", "mrb_per_state", "mrb_per_export_tree", "read_and_clear_flags", "rows_alloc"}
+                "mrb_res_destroy", "mrb_per_state", "mrb_per_export_tree", "read_and_clear_flags", "rows_alloc",
+                "counters_to_device", "counters_from_device"}
     may_alloc = {"mrb_urb_create", "mrb_per_create", "mrb_res_create", "rows_alloc", "mrb_per_update"}
     for name, body in bodies.items():
         if name not in may_wait:
@@ -134,6 +135,10 @@ def test_only_the_documented_entry_points_wait_or_allocate():
     # the check functions wait through this helper and nothing else does
     users = [n for n, b in bodies.items() if "read_and_clear_flags(" in b]
     assert sorted(users) == ["mrb_per_check", "mrb_urb_check"]
+    # device-resident counters are copied (with a wait) only where the header says so: switching the option,
+    # state queries and the checkpoint calls - never by push, sample or update
+    users = {n for n, b in bodies.items() if re.search(r"counters_(to|from)_device\(", b)}
+    assert users == {"mrb_set_option", "mrb_per_state", "mrb_per_get_counters", "mrb_per_set_counters"}, users
     # the allocation-free entry point and the core it shares with mrb_per_update
     for name in ("mrb_per_update_noalloc", "per_update", "tree_rebuild", "next_epoch", "static_scratch"):
         assert not allocs.search(bodies[name]) and not waits.search(bodies[name]), name
