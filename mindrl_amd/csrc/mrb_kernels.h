@@ -1237,6 +1237,33 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
                 if (jw1 >= 0) { vs.y = vm.y = powf_det_call(a.priorities[jw1], a.alpha); wrote = true; }
                 if (jw2 >= 0) { vs.z = vm.z = powf_det_call(a.priorities[jw2], a.alpha); wrote = true; }
                 if (jw3 >= 0) { vs.w = vm.w = powf_det_call(a.priorities[jw3], a.alpha); wrote = true; }
+            } else if (!a.indices && a.priorities) {
+                // a push with priorities: the lane's four priorities are requested together, then raised to
+                // alpha one after the other (asked for one by one, each power would wait for its own load)
+                float pv[4];
+                bool in[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    int64_t j = (int64_t)off + c - first_slot;
+                    if (j < 0) j += a.capacity;
+                    in[c] = (int64_t)off + c < a.capacity && j < a.n;
+                    pv[c] = in[c] ? a.priorities[j] : 0.0f;
+                }
+                float qv[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    qv[c] = 0.0f;
+                    if (in[c]) {
+                        const bool ok = valid_priority(pv[c]);
+                        qv[c] = ok ? powf_det_call(pv[c], a.alpha) : *a.maxp;  // invalid: the fresh slot stays at the running max
+                        if (a.fold_max == 2 && !ok) atomicOr(a.err, MRB_DERR_PRIORITY);
+                        wrote = true;
+                    }
+                }
+                if (in[0]) vs.x = vm.x = qv[0];
+                if (in[1]) vs.y = vm.y = qv[1];
+                if (in[2]) vs.z = vm.z = qv[2];
+                if (in[3]) vs.w = vm.w = qv[3];
             } else {
                 if (leaf_value(a, first_slot, off + 0, q)) { vs.x = vm.x = q; wrote = true; }
                 if (leaf_value(a, first_slot, off + 1, q)) { vs.y = vm.y = q; wrote = true; }
