@@ -284,8 +284,10 @@ class PerRun:
 
     def loop(self, i, sp=None):
         self.sample(i, sp)
-        self.L.mrb_per_update(self.h, self.idx.data_ptr(), self.upr[i % 64].data_ptr(), self.upd, sp or self.sp)
-        self.L.mrb_per_push(self.h, self.sptr, self.ins_n, self.ins_pr, sp or self.sp)
+        rc = self.L.mrb_per_update(self.h, self.idx.data_ptr(), self.upr[i % 64].data_ptr(), self.upd, sp or self.sp)
+        rc = rc or self.L.mrb_per_push(self.h, self.sptr, self.ins_n, self.ins_pr, sp or self.sp)
+        if rc:
+            self._lib.check(rc)
 
 
 def bench_per(a):
@@ -408,26 +410,27 @@ def per_extras(a, torch, r):
     extras["loop_steps_per_s"] = 1.0 / timed(lambda i: r.loop(W + i % K))
     # the same loop recorded ONCE into a HIP graph (50 steps) with the buffer's counters kept on the device, so
     # that every replay continues where the last one stopped; replayed 10 times
-    r.buf.set_option("device_counters", 1)
-    n_l = min(K, 50)
-    lgraph = torch.cuda.CUDAGraph()
-    lside = torch.cuda.Stream()
-    with torch.cuda.stream(lside):
-        lsp = C.c_void_p(lside.cuda_stream)
-        lgraph.capture_begin()
-        for i in range(n_l):
-            r.loop(W + i, lsp)
-        lgraph.capture_end()
-    torch.cuda.synchronize()
-    lgraph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(10):
+    if r.upd <= 1024:  # device-resident counters take updates of at most 1024 entries
+        r.buf.set_option("device_counters", 1)
+        n_l = min(K, 50)
+        lgraph = torch.cuda.CUDAGraph()
+        lside = torch.cuda.Stream()
+        with torch.cuda.stream(lside):
+            lsp = C.c_void_p(lside.cuda_stream)
+            lgraph.capture_begin()
+            for i in range(n_l):
+                r.loop(W + i, lsp)
+            lgraph.capture_end()
+        torch.cuda.synchronize()
         lgraph.replay()
-    torch.cuda.synchronize()
-    extras["loop_graph_replay_steps_per_s"] = 10 * n_l / (time.perf_counter() - t0)
-    del lgraph
-    r.buf.set_option("device_counters", 0)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            lgraph.replay()
+        torch.cuda.synchronize()
+        extras["loop_graph_replay_steps_per_s"] = 10 * n_l / (time.perf_counter() - t0)
+        del lgraph
+        r.buf.set_option("device_counters", 0)
     if not r.loop_step:
         extras["sample_us_per_call"] = timed(lambda i: r.sample(W + i % K)) * 1e6
         # spread over the run: an event after every 10 calls (an event after every call would add its own ~3 us),

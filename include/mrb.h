@@ -90,7 +90,7 @@ int mrb_version(void);
  *                  calls on one handle must not overlap (they share a scratch array), and mrb_per_state and
  *                  the checkpoint calls wait for the device to read the counters back. Switching it (either
  *                  way) waits for the device. 0 (default) = host-side counters, passed as kernel arguments.
- *   "fused_rebuild" prioritized buffers: 1 (default) = an update of <= 32 entries or a push under <= 32 leaf tiles
+ *   "fused_rebuild" prioritized buffers: 1 (default) = an update of <= 16 entries or a push under <= 16 leaf tiles
  *                  rebuilds the tree in one launch where the tree has one round of levels below its top;
  *                  0 = one launch per round */
 int mrb_set_option(int64_t h, const char *name, int64_t value);

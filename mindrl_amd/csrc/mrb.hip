@@ -438,9 +438,10 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
         a.nrounds = 0;
         a.top_depth = a.depth;
     }
-    // One round below the top and little tile work (an update of at most 32 entries: a wave per entry; a push
-    // that does not wrap, under at most 32 leaf tiles: a wave per tile): one launch of one workgroup of 16
-    // waves, each taking one or two units, that goes on to the top.
+    // One round below the top and at most 16 waves of work (an update: a wave per entry; a push that does
+    // not wrap: a wave per leaf tile under its slots): one launch of one workgroup that goes on to the top.
+    // (More units per wave do not pay: the 16 waves of a workgroup share one compute unit's issue slots, and a
+    // second unit costs a wave as much as the second launch it would save; four cost twice as much.)
     if (a.nrounds == 1 && b.fused) {
         uint32_t units = 0, tile_base = 0;
         if (a.inline_election) {
@@ -451,7 +452,7 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
             tile_base = (uint32_t)(a.first_slot / kBlockNodes);
             units = (uint32_t)((a.first_slot + a.n - 1) / kBlockNodes) - tile_base + 1;
         }
-        if (units > 0 && units <= 2u * (kFusedWG / 64)) {
+        if (units > 0 && units <= (uint32_t)(kFusedWG / 64)) {
             PutArgs put = ride ? *ride : none;
             put.blocks = (put.blocks + 3) / 4;  // the ride-along copy was sized for workgroups a quarter as large
             hipLaunchKernelGGL(k_tree_fused, dim3(1 + put.blocks), dim3(kFusedWG), 0, s, a, tile_base, units, put);

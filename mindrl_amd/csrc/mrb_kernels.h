@@ -1556,15 +1556,14 @@ __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) 
 }
 
 // ---------------------------------------------------------------------------
-// A push of few rows, or an update of a few entries, on a tree with one round below the top, in ONE
-// launch: the tile work fits the 16 waves of one workgroup (a wave per leaf tile of a push, or per
-// entry of an update; the host allows up to two per wave, beyond which the second launch is the
-// cheaper way), and the same workgroup goes on to the top after a barrier. Within one
+// A push of few rows, or an update of at most 16 entries, on a tree with one round below the top,
+// in ONE launch: the tile work fits the 16 waves of one workgroup (a wave per leaf tile of a push,
+// or per entry of an update), and the same workgroup goes on to the top after a barrier. Within one
 // workgroup that needs no fence: its waves share a compute unit, and the nodes the top reads were
 // never in that unit's cache before they were written. (Handing the tiles of SEVERAL workgroups to a
 // last one through agent-scope stores, a counter and agent-scope loads was measured too: the three
 // trips through memory cost 2.9 us, more than the second launch they save.)
-//   units      entries (update) or leaf tiles from tile_base on (push); a wave each, or two each in turn
+//   units      waves with work: entries (update) or leaf tiles from tile_base on (push), at most 16
 // ---------------------------------------------------------------------------
 constexpr int kFusedWG = 1024;
 
@@ -1575,7 +1574,7 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
         return;
     }
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (uint32_t unit = wave; unit < units; unit += kFusedWG / 64) {  // a few units more than waves: one after the other
+    if (const uint32_t unit = wave; unit < units) {
         if (a.inline_election) {
             entry_tile(a, a.g[0], unit, lane, s_win[wave], nullptr, 0);
             entry_duty(a, unit, units, lane);
