@@ -534,6 +534,9 @@ UpdateArgs update_args(Per& b) {
 // p^alpha between the stamp pass and the leaf writes. Allocates nothing.
 int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t n, float* powered, hipStream_t s) {
     Per* b = &pb;
+    if (b->device_counters && n > 1024)
+        return fail(MRB_ESTATE, "with device_counters an update takes at most 1024 entries (larger ones elect their "
+                                "entries with tags the host counts, which a graph replay would repeat)");
     int rc = next_epoch(*b, s);
     if (rc) return rc;
     UpdateArgs a = update_args(*b);
@@ -940,9 +943,6 @@ int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, i
     if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
     if (n > 0xffffffffll) return fail(MRB_EINVAL, "n %lld exceeds 2^32 - 1 entries per call", (long long)n);
     if (!indices || !priorities) return fail(MRB_EINVAL, "indices or priorities is NULL");
-    if (b->device_counters && n > 1024)
-        return fail(MRB_ESTATE, "with device_counters an update takes at most 1024 entries (larger ones elect their "
-                                "entries with tags the host counts, which a graph replay would repeat)");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (n > b->powered_cap) {
         // more entries than any call so far (and than the capacity): a larger array, at least twice the
