@@ -1077,6 +1077,16 @@ def test_sparse_updates_on_very_large_trees(mrb, orc, cap):
         assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(256, 0.5, u), "n %d" % n)
     assert_tree_equal(g, c, "cap %d" % cap)
     assert np.float32(g.max_priority) == np.float32(c.max_priority)
+    # pushes with priorities on the full ring: 5000 rows (the leaf-level waves collect the call's largest
+    # p^alpha for the top workgroup), one of them above the running max; then 300 rows
+    for n in (5000, 300):
+        more = [np.ones((n, 1), np.uint8)]
+        mp = (rng.pareto(1.5, n) + 1e-6).astype(np.float32)
+        mp[n // 2] = np.float32(c.max_priority) * 3 + 1
+        g.insert(*to_dev(more), priorities=torch.from_numpy(mp).cuda())
+        c.push(more, n, mp)
+        assert_tree_equal(g, c, "cap %d push %d with priorities" % (cap, n))
+        assert np.float32(g.max_priority) == np.float32(c.max_priority)
     # invalid entries are skipped and flagged, valid ones in the same call still land
     g.update_priorities(torch.tensor([5, cap + 3, -1, 9]).cuda(), torch.tensor([2.0, 1.0, 1.0, float("nan")]).cuda())
     c.update([5], [2.0])
