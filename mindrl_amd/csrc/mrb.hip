@@ -544,8 +544,9 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
     a.indices = indices;
     a.priorities = priorities;
     a.n = n;
-    // Few entries on a very large tree: rebuild the lowest levels per entry, not per tile.
-    const bool sparse = b->s_g0 > 0 && n <= (b->leaves >> 8);
+    // Few entries (but more than the 1024 that elect among themselves, below) on a very large tree: rebuild
+    // the lowest levels per entry, not per tile.
+    const bool sparse = b->s_g0 > 0 && n > 1024 && n <= (b->leaves >> 8);
     if (sparse) {
         a.sparse_g0 = b->s_g0;
         a.nrounds = b->s_rounds;

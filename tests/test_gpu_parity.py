@@ -195,14 +195,15 @@ def test_hip_graph_replays_update_and_sample(mrb, orc, path):
     g.destroy()
 
 
-@pytest.mark.parametrize("cap", [3000, 70000])
+@pytest.mark.parametrize("cap", [3000, 70000, 3_000_000])
 def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap):
     """push 3 rows + generator-driven sample + update_priorities of the sampled rows, recorded ONCE with the
     option device_counters and replayed 12 times on new rows and priorities: the buffer fills up, the ring wraps,
     the draws advance - every replay equals the oracle's push, sample, update; eager calls between replays keep
     working, and the counters read back agree."""
     rng = np.random.default_rng(cap)
-    shapes, dtypes = [(300,), (1,), (2,)], [np.float32, np.int32, np.uint8]
+    # (trees of 12, 17 and 22 levels: the top alone, one round fused with it, two rounds in launches of their own)
+    shapes, dtypes = ([(300,), (1,), (2,)], [np.float32, np.int32, np.uint8]) if cap < 10 ** 6 else ([(2,), (1,)], [np.float32, np.int32])
     batch, npush = 48, 3
     g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=13, shapes=shapes, dtypes=dtypes)
     fill = cap - 20  # not full: the row count changes during the replays, then the ring wraps
@@ -1056,8 +1057,9 @@ def test_config5_tree_descent_stress(mrb, orc):
 
 @pytest.mark.parametrize("cap", [3_000_000, 20_000_000])
 def test_sparse_updates_on_very_large_trees(mrb, orc, cap):
-    """Trees of 22 and 25 levels: updates with few entries take the entry-driven lowest round
-    (groups of 4 and 8 lanes per entry); sizes 1, 1000 (10 % duplicates, some invalid) and 60,000."""
+    """Trees of 22 and 25 levels: updates of up to 1024 entries elect among themselves (sizes 1, 7, 1000 with
+    10 % duplicates), larger ones with few entries for the tree take the entry-driven lowest round (60,000:
+    groups of 4 and 8 lanes per entry)."""
     shapes, dtypes = [(1,)], [np.uint8]
     rng = np.random.default_rng(cap % 1000)
     g, c = make_pair(mrb, orc, 0.6, cap, 256, seed=3, shapes=shapes, dtypes=dtypes)
