@@ -195,8 +195,8 @@ def test_hip_graph_replays_update_and_sample(mrb, orc, path):
     g.destroy()
 
 
-@pytest.mark.parametrize("cap", [3000, 70000, 3_000_000])
-def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap):
+@pytest.mark.parametrize("cap,path", [(3000, 1), (70000, 1), (70000, 2), (3_000_000, 1)])
+def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap, path):
     """push 3 rows + generator-driven sample + update_priorities of the sampled rows, recorded ONCE with the
     option device_counters and replayed 12 times on new rows and priorities: the buffer fills up, the ring wraps,
     the draws advance - every replay equals the oracle's push, sample, update; eager calls between replays keep
@@ -210,7 +210,10 @@ def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap):
     rows = random_rows(rng, fill, shapes, dtypes)
     g.insert(*to_dev(rows)), c.push(rows, fill)
     g.set_option("device_counters", 1)
+    g.set_option("sample_path", path)
     new_rows = [torch.zeros((npush,) + tuple(s), dtype=t).cuda() for s, t in zip(shapes, torch_types(dtypes))]
+    prio_rows = [torch.zeros((2,) + tuple(s), dtype=t).cuda() for s, t in zip(shapes, torch_types(dtypes))]
+    prio_dev = torch.ones(2, dtype=torch.float32, device="cuda")  # a second push, with priorities of its own
     pr_dev = torch.ones(batch, dtype=torch.float32, device="cuda")
     out = (torch.empty(batch, dtype=torch.int64, device="cuda"), torch.empty(batch, dtype=torch.float32, device="cuda"),
            g._layout.empty(batch, g._dev))
@@ -220,19 +223,23 @@ def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap):
     with torch.cuda.stream(side):
         graph.capture_begin()
         g.insert(*new_rows)
+        g.insert(*prio_rows, priorities=prio_dev)
         g.sample(0.5, out=out)
         g.update_priorities(out[0], pr_dev)
         graph.capture_end()
     torch.cuda.synchronize()
     for rep in range(12):
         fresh = random_rows(rng, npush, shapes, dtypes)
+        fresh2 = random_rows(rng, 2, shapes, dtypes)
+        ppr = (rng.pareto(1.5, 2) + 1e-6).astype(np.float32)
         pr = (rng.pareto(1.5, batch) + 1e-6).astype(np.float32)
-        for dst, src in zip(new_rows, fresh):
+        for dst, src in zip(new_rows + prio_rows, fresh + fresh2):
             dst.copy_(torch.from_numpy(src))
-        pr_dev.copy_(torch.from_numpy(pr))
+        pr_dev.copy_(torch.from_numpy(pr)), prio_dev.copy_(torch.from_numpy(ppr))
         graph.replay()
         torch.cuda.synchronize()
         c.push(fresh, npush)
+        c.push(fresh2, 2, ppr)
         want = c.sample(batch, 0.5)
         assert_sample_equal((out[0], out[1]) + tuple(out[2]), want, "cap %d replay %d" % (cap, rep))
         c.update(want[0], pr)
@@ -242,6 +249,9 @@ def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap):
             extra = random_rows(rng, 5, shapes, dtypes)
             g.insert(*to_dev(extra)), c.push(extra, 5)
             assert_sample_equal(g.sample(0.9), c.sample(batch, 0.9), "eager after replay %d" % rep)
+            two = g.sample_many(2, 0.6)  # two batches in one launch: the generator moves on by two calls
+            for i in range(2):
+                assert_sample_equal([x[i] for x in two], c.sample(batch, 0.6), "eager sample_many after replay %d" % rep)
     with pytest.raises(ValueError):
         g.update_priorities(torch.zeros(2000, dtype=torch.int64).cuda(), torch.ones(2000).cuda())
     g.set_option("device_counters", 0)
