@@ -249,6 +249,11 @@ def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap, path
             extra = random_rows(rng, 5, shapes, dtypes)
             g.insert(*to_dev(extra)), c.push(extra, 5)
             assert_sample_equal(g.sample(0.9), c.sample(batch, 0.9), "eager after replay %d" % rep)
+            if cap >= 70000:  # a push too large for the one-launch rebuild, with priorities, placed by the device
+                big = random_rows(rng, 4500, shapes, dtypes)
+                bpr = (rng.pareto(1.5, 4500) + 1e-6).astype(np.float32)
+                g.insert(*to_dev(big), priorities=torch.from_numpy(bpr).cuda()), c.push(big, 4500, bpr)
+                assert_tree_equal(g, c, "cap %d big push after replay %d" % (cap, rep))
             two = g.sample_many(2, 0.6)  # two batches in one launch: the generator moves on by two calls
             for i in range(2):
                 assert_sample_equal([x[i] for x in two], c.sample(batch, 0.6), "eager sample_many after replay %d" % rep)
