@@ -80,7 +80,7 @@ int mrb_version(void);
  *   "row_split"    least number of workgroups per row in the wide-row kernel (0 = auto, max 64)
  *   "sample_path"  prioritized buffers: 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
  *   "lds_levels"   prioritized buffers: tree levels staged in LDS by the LDS-top kernel (0 = auto, max 12)
- *   "device_counters" prioritized buffers: 1 = the ring position, the number of stored rows and the generator's
+ *   "device_counters" prioritized and uniform buffers: 1 = the ring position, the number of stored rows and the generator's
  *                  call counter are kept in device memory, read there by the kernels and advanced there by
  *                  a one-thread kernel after every push and every generator-driven sample - for callers that
  *                  record push / sample / update into a HIP graph: every replay then continues where the last
@@ -90,6 +90,10 @@ int mrb_version(void);
  *                  calls on one handle must not overlap (they share a scratch array), and mrb_per_state and
  *                  the checkpoint calls wait for the device to read the counters back. Switching it (either
  *                  way) waits for the device. 0 (default) = host-side counters, passed as kernel arguments.
+ *                  Uniform buffers: count, head and the generator's call counter; an append takes at most
+ *                  `capacity` rows, a sample at most 65,536 (its slots are drawn into a device array that
+ *                  overlapping sample / get_item calls on one handle would share), mrb_urb_append_from is
+ *                  refused, and mrb_urb_state, mrb_urb_reset, mrb_urb_seed and the checkpoint calls wait.
  *   "fused_rebuild" prioritized buffers: 1 (default) = an update of <= 16 entries or a push under <= 16 leaf tiles
  *                  rebuilds the tree in one launch where the tree has one round of levels below its top;
  *                  0 = one launch per round */

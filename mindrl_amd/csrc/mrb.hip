@@ -290,9 +290,13 @@ struct Urb {
     RowStore rows;
     int64_t count = 0, head = 0;
     uint64_t seed = 0, calls = 0;
-    uint32_t* err = nullptr;
+    uint32_t* err = nullptr;       // 16 bytes of flags, then the device copy of the counters (kUrb* in mrb_kernels.h)
+    int64_t* counters = nullptr;   // = err + 16 bytes
+    int64_t* slots = nullptr;      // device array of kUrbDrawMax slots: drawn there when the counters live on the device
+    int64_t device_counters = 0;   // option "device_counters"
     ~Urb() {
         if (err) (void)hipFree(err);
+        if (slots) (void)hipFree(slots);
     }
 };
 
@@ -595,6 +599,25 @@ int counters_from_device(Per& b) {
     b.pushes = v[kCntPushes], b.size = v[kCntSize], b.calls = (uint64_t)v[kCntCalls];
     return MRB_OK;
 }
+int counters_to_device(Urb& b) {
+    const int64_t cap = b.rows.capacity;
+    const int64_t v[4] = {b.count < cap && b.head == 0 ? b.count : b.head, b.count, (int64_t)b.calls, b.head};
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(b.counters, v, sizeof(v), hipMemcpyHostToDevice));
+    return MRB_OK;
+}
+int counters_from_device(Urb& b) {
+    int64_t v[4];
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(v, b.counters, sizeof(v), hipMemcpyDeviceToHost));
+    b.count = v[kUrbCount], b.head = v[kUrbHead], b.calls = (uint64_t)v[kUrbCalls];
+    return MRB_OK;
+}
+int counters_advance(Urb& b, int64_t rows, int64_t calls, hipStream_t s) {
+    hipLaunchKernelGGL(k_urb_advance, dim3(1), dim3(64), 0, s, b.counters, rows, b.rows.capacity, calls);
+    LAUNCH_CHECK("k_urb_advance");
+    return MRB_OK;
+}
 int counters_advance(Per& b, int64_t pushed, int64_t calls, hipStream_t s) {
     hipLaunchKernelGGL(k_counters_advance, dim3(1), dim3(64), 0, s, b.counters, pushed, b.rows.capacity, calls);
     LAUNCH_CHECK("k_counters_advance");
@@ -631,12 +654,17 @@ int mrb_set_option(int64_t h, const char* name, int64_t value) {
         if (value < 0 || value > 12) return fail(MRB_EINVAL, "lds_levels must be in [0, 12]");
         per->lds_levels = value;
     } else if (!strcmp(name, "device_counters")) {
-        if (!per) return fail(MRB_EINVAL, "device_counters is an option of prioritized buffers");
+        if (!per && !urb) return fail(MRB_EINVAL, "device_counters is an option of prioritized and uniform buffers");
         if (value < 0 || value > 1) return fail(MRB_EINVAL, "device_counters must be 0 or 1");
-        if (value != per->device_counters) {
+        if (per && value != per->device_counters) {
             const int rc = value ? counters_to_device(*per) : counters_from_device(*per);
             if (rc) return rc;
             per->device_counters = value;
+        }
+        if (urb && value != urb->device_counters) {
+            const int rc = value ? counters_to_device(*urb) : counters_from_device(*urb);
+            if (rc) return rc;
+            urb->device_counters = value;
         }
     } else if (!strcmp(name, "fused_rebuild")) {
         if (!per) return fail(MRB_EINVAL, "fused_rebuild is an option of prioritized buffers");
@@ -656,8 +684,10 @@ int mrb_urb_create(int64_t capacity, int nfields, const int64_t* field_bytes, in
     auto b = std::make_shared<Urb>();
     int rc = rows_alloc(b->rows, capacity, nfields, field_bytes);
     if (rc) return rc;
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16));
-    HIP_TRY(hipMemset(b->err, 0, 16));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16 + 4 * sizeof(int64_t)));
+    HIP_TRY(hipMemset(b->err, 0, 16 + 4 * sizeof(int64_t)));
+    b->counters = reinterpret_cast<int64_t*>(b->err + 4);
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->slots), kUrbDrawMax * sizeof(int64_t)));
     HIP_TRY(hipDeviceSynchronize());  // the zero-fills ran on the null stream; the caller's stream may not wait for it
     std::lock_guard<std::mutex> lk(g_mu);
     *out_handle = g_next++;
@@ -675,7 +705,21 @@ int mrb_urb_append(int64_t h, const void* const* src_fields, int64_t nrows, void
     // More rows than slots: only the last `cap` survive, at the positions a row-by-row append leaves them.
     const int64_t skip = nrows > cap ? nrows - cap : 0;
     const int64_t first = (w + skip) % cap;
-    int rc = rows_put(b->rows, src_fields, skip, nrows - skip, first, static_cast<hipStream_t>(stream));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (b->device_counters) {
+        // the write position is read on the device, and advanced there after the copy
+        if (nrows > cap) return fail(MRB_ESTATE, "with device_counters an append takes at most capacity (%lld) rows", (long long)cap);
+        PutArgs p{};
+        int rc = put_args(b->rows, src_fields, 0, nrows, 0, p);
+        if (rc) return rc;
+        p.first_slot = -1;
+        p.src_first = reinterpret_cast<int64_t>(b->counters);
+        hipLaunchKernelGGL(k_rows_put, dim3(p.blocks), dim3(kWG), 0, s, p);
+        LAUNCH_CHECK("k_rows_put");
+        urb_advance(*b, nrows);
+        return counters_advance(*b, nrows, 0, s);
+    }
+    int rc = rows_put(b->rows, src_fields, skip, nrows - skip, first, s);
     if (rc) return rc;
     urb_advance(*b, nrows);
     return MRB_OK;
@@ -688,6 +732,8 @@ int mrb_urb_append_from(int64_t h, int64_t src, int64_t first_logical, int64_t n
     auto from = find_urb(src);
     if (!from) return fail(MRB_EHANDLE, "unknown uniform buffer handle %lld", (long long)src);
     if (from.get() == b.get()) return fail(MRB_EINVAL, "source and destination are the same buffer");
+    if (b->device_counters || from->device_counters)
+        return fail(MRB_ESTATE, "a buffer-to-buffer append needs both buffers' counters on the host (device_counters 0)");
     if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
     if (first_logical < 0) first_logical += from->count;
     if (first_logical < 0 || first_logical + n > from->count)
@@ -730,9 +776,17 @@ int mrb_urb_get_item(int64_t h, int64_t logical_index, void* const* dst_fields, 
     if (i < 0) i += b->count;
     if (i < 0 || i >= b->count)
         return fail(MRB_EINVAL, "index %lld outside the %lld stored rows", (long long)logical_index, (long long)b->count);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (b->device_counters) {
+        // count and head are read on the device: the slot is worked out there and the gather takes it as a given index
+        hipLaunchKernelGGL(k_urb_slots, dim3(1), dim3(kWG), 0, s, b->slots, b->seed, b->counters, (int64_t)1, logical_index, 1,
+                           b->err);
+        LAUNCH_CHECK("k_urb_slots");
+        return gather_rows(b->rows, b->slots, -1, b->rows.capacity, b->seed, b->calls, 1, nullptr, dst_fields, b->err, s);
+    }
     const int64_t t = b->count - b->head;
     const int64_t slot = i < t ? i + b->head : i - t;
-    return urb_gather_impl(*b, nullptr, slot, 1, nullptr, dst_fields, static_cast<hipStream_t>(stream));
+    return urb_gather_impl(*b, nullptr, slot, 1, nullptr, dst_fields, s);
 }
 
 int mrb_urb_gather(int64_t h, const int64_t* indices, int64_t n, void* const* dst_fields, void* stream) {
@@ -740,6 +794,9 @@ int mrb_urb_gather(int64_t h, const int64_t* indices, int64_t n, void* const* ds
     if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
     if (!indices) return fail(MRB_EINVAL, "indices is NULL");
     if (b->count <= 0) return fail(MRB_ESTATE, "gather from an empty buffer");
+    if (b->device_counters)  // the row count is on the device: slots are checked against the capacity only
+        return gather_rows(b->rows, indices, -1, b->rows.capacity, b->seed, b->calls, n, nullptr, dst_fields, b->err,
+                           static_cast<hipStream_t>(stream));
     return urb_gather_impl(*b, indices, -1, n, nullptr, dst_fields, static_cast<hipStream_t>(stream));
 }
 
@@ -748,7 +805,21 @@ int mrb_urb_sample(int64_t h, int64_t n, int64_t* out_indices, void* const* dst_
     if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
     if (n > b->count)
         return fail(MRB_ESTATE, "sample size %lld exceeds the %lld stored rows", (long long)n, (long long)b->count);
-    int rc = urb_gather_impl(*b, nullptr, -1, n, out_indices, dst_fields, static_cast<hipStream_t>(stream));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (b->device_counters) {
+        // count and the generator's call counter are read on the device: the slots are drawn there, the gather
+        // takes them as given indices, and the call counter moves on there
+        if (n > kUrbDrawMax)
+            return fail(MRB_ESTATE, "with device_counters a sample takes at most %lld rows", (long long)kUrbDrawMax);
+        hipLaunchKernelGGL(k_urb_slots, dim3(grid_exact((uint64_t)n)), dim3(kWG), 0, s, b->slots, b->seed, b->counters, n,
+                           (int64_t)0, 0, b->err);
+        LAUNCH_CHECK("k_urb_slots");
+        int rc = gather_rows(b->rows, b->slots, -1, b->rows.capacity, b->seed, b->calls, n, out_indices, dst_fields, b->err, s);
+        if (rc) return rc;
+        b->calls += 1;
+        return counters_advance(*b, 0, 1, s);
+    }
+    int rc = urb_gather_impl(*b, nullptr, -1, n, out_indices, dst_fields, s);
     if (rc) return rc;
     b->calls += 1;
     return MRB_OK;
@@ -756,13 +827,21 @@ int mrb_urb_sample(int64_t h, int64_t n, int64_t* out_indices, void* const* dst_
 
 int mrb_urb_seed(int64_t h, uint64_t seed) {
     GET_URB(b, h);
+    if (b->device_counters) {
+        const int rc = counters_from_device(*b);
+        if (rc) return rc;
+    }
     b->seed = seed;
     b->calls = 0;
-    return MRB_OK;
+    return b->device_counters ? counters_to_device(*b) : MRB_OK;
 }
 
 int mrb_urb_state(int64_t h, int32_t* count, int32_t* head) {
     GET_URB(b, h);
+    if (b->device_counters) {  // the device's counters are the current ones (a graph replay advances only them)
+        const int rc = counters_from_device(*b);
+        if (rc) return rc;
+    }
     if (count) *count = (int32_t)b->count;
     if (head) *head = (int32_t)b->head;
     return MRB_OK;
@@ -770,6 +849,12 @@ int mrb_urb_state(int64_t h, int32_t* count, int32_t* head) {
 
 int mrb_urb_reset(int64_t h) {
     GET_URB(b, h);
+    if (b->device_counters) {  // no stream to order it on: the counters come back, are reset and go out again
+        int rc = counters_from_device(*b);
+        if (rc) return rc;
+        b->count = 0;
+        return counters_to_device(*b);
+    }
     b->count = 0;
     return MRB_OK;
 }
@@ -1215,6 +1300,10 @@ int mrb_res_destroy(int64_t h) {
 int mrb_urb_get_counters(int64_t h, int64_t* out4) {
     GET_URB(b, h);
     if (!out4) return fail(MRB_EINVAL, "out4 is NULL");
+    if (b->device_counters) {
+        const int rc = counters_from_device(*b);
+        if (rc) return rc;
+    }
     out4[0] = b->count, out4[1] = b->head, out4[2] = (int64_t)b->seed, out4[3] = (int64_t)b->calls;
     return MRB_OK;
 }
@@ -1227,7 +1316,7 @@ int mrb_urb_set_counters(int64_t h, const int64_t* in4) {
         return fail(MRB_EINVAL, "count %lld / head %lld do not fit capacity %lld", (long long)in4[0], (long long)in4[1],
                     (long long)cap);
     b->count = in4[0], b->head = in4[1], b->seed = (uint64_t)in4[2], b->calls = (uint64_t)in4[3];
-    return MRB_OK;
+    return b->device_counters ? counters_to_device(*b) : MRB_OK;
 }
 
 int mrb_per_get_counters(int64_t h, int64_t* out4) {

@@ -1800,6 +1800,59 @@ __global__ void k_counters_advance(int64_t* counters, int64_t pushed, int64_t ca
     }
 }
 
+// The uniform buffer's device-resident counters: [0] the next write position, [1] count, [2] the generator's
+// call counter, [3] head. kUrb* name them; the row copy finds its position at [0] like a prioritized push.
+constexpr int kUrbWrite = 0, kUrbCount = 1, kUrbCalls = 2, kUrbHead = 3;
+constexpr int64_t kUrbDrawMax = 1 << 16;  // most rows a sample draws through the device-side index array
+
+// count / head after an append of n rows (n <= capacity; the write position is chosen once per call: `count`
+// while the buffer has never wrapped, else `head`), after a reset (n < 0), after `calls` generator-driven samples.
+__global__ void k_urb_advance(int64_t* c, int64_t n, int64_t cap, int64_t calls) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    int64_t count = c[kUrbCount], head = c[kUrbHead];
+    if (n < 0) {
+        count = 0;
+    } else if (n > 0) {
+        if (count < cap && head == 0) {
+            const int64_t room = cap - count;
+            if (n <= room) {
+                count += n;
+            } else {
+                count = cap;
+                head = (n - room) % cap;
+            }
+        } else {
+            head = (head + n) % cap;
+            count = count + n < cap ? count + n : cap;
+        }
+    }
+    c[kUrbCount] = count;
+    c[kUrbHead] = head;
+    c[kUrbWrite] = count < cap && head == 0 ? count : head;
+    c[kUrbCalls] += calls;
+}
+
+// The slots of a generator-driven sample (uniform in [0, count), with replacement), or - logical >= -count -
+// the slot of one logical position (0 = oldest, negative counts back from the newest), written out for a
+// gather at given slots: with the counters on the device the gather cannot take them as arguments.
+__global__ __launch_bounds__(kWG) void k_urb_slots(int64_t* dst, uint64_t seed, const int64_t* c, int64_t n,
+                                                   int64_t logical, int one_item, uint32_t* err) {
+    const int64_t i = (int64_t)blockIdx.x * kWG + threadIdx.x;
+    if (i >= n) return;
+    const int64_t count = c[kUrbCount], head = c[kUrbHead];
+    if (!one_item) {
+        dst[i] = count > 0 ? rng_below(seed, (uint64_t)c[kUrbCalls], (uint64_t)i, count) : 0;
+        return;
+    }
+    int64_t at = logical < 0 ? logical + count : logical;
+    if (at < 0 || at >= count) {
+        atomicOr(err, MRB_DERR_INDEX);
+        at = 0;
+    }
+    const int64_t t = count - head;
+    dst[0] = at < t ? at + head : at - t;
+}
+
 // The generator's draws for `nbatch` batches, written out for a sample kernel to read: with the call
 // counter on the device the kernel cannot take it as an argument.
 __global__ __launch_bounds__(kWG) void k_fill_uniforms(float* dst, uint64_t seed, const int64_t* counters, int64_t batch,

@@ -75,6 +75,72 @@ def test_uniform_ring_random_ops(mrb, orc, layout, cap):
     g.destroy()
 
 
+@pytest.mark.parametrize("layout,cap", [(0, 37), (1, 5000)])
+def test_uniform_loop_recorded_into_a_hip_graph_with_device_counters(mrb, orc, layout, cap):
+    """The loop the reference compiles as one graph (mindspore_rl/algorithm/dqn/dqn_trainer.py:65-88: insert, then
+    sample, every step) on the uniform buffer: insert 3 rows + sample, recorded ONCE with device_counters and
+    replayed 20 times on new rows - the buffer grows, fills, wraps and the draws move on; every replay against the
+    oracle, with eager get_item / gather / insert / reset between replays and the counters read back."""
+    shapes, dtypes = URB_LAYOUTS[layout]
+    rng = np.random.default_rng(7 * cap + layout)
+    batch, nin = 8, 3
+    g = mrb.URB(batch, cap, shapes, torch_types(dtypes), seed=21)
+    c = orc.OracleUniform(cap, shapes, dtypes, seed=21)
+    first = random_rows(rng, cap - 25, shapes, dtypes)
+    g.insert(to_dev(first)), c.append(first, cap - 25)
+    g.set_option("device_counters", 1)
+    new_rows = [torch.zeros((nin,) + tuple(s), dtype=t).cuda() for s, t in zip(shapes, torch_types(dtypes))]
+    out = g._layout.empty(batch, g._dev)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        g.insert(new_rows)
+        g.sample(out=out)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for rep in range(20):
+        fresh = random_rows(rng, nin, shapes, dtypes)
+        for dst, src in zip(new_rows, fresh):
+            dst.copy_(torch.from_numpy(src))
+        graph.replay()
+        torch.cuda.synchronize()
+        c.append(fresh, nin)
+        _, want = c.sample(batch)
+        for a, b in zip(out, want):
+            assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8)), (cap, rep)
+        assert int(g.count) == c.count and int(g.head) == c.head, (cap, rep)
+        for f in range(len(shapes)):
+            assert np.array_equal(t2n(g.buffer[f]).view(np.uint8), c.field(f).view(np.uint8)), (cap, rep, f)
+        if rep % 4 == 1:  # eager calls in between
+            j = int(rng.integers(-c.count, c.count))
+            for a, b in zip(g.get_item(j), c.get_item(j)):
+                assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+            idx = rng.integers(0, c.count, 19)
+            for a, b in zip(g.sample(indices=torch.from_numpy(idx).cuda()), c.gather(idx)):
+                assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+            more = random_rows(rng, 7, shapes, dtypes)
+            g.insert(to_dev(more)), c.append(more, 7)
+            gi, gf = g.sample_with_indices()
+            ci, cf = c.sample(batch)
+            assert np.array_equal(t2n(gi), ci)
+            for a, b in zip(gf, cf):
+                assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8))
+        if rep == 13:
+            g.reset(), c.reset()
+            refill = random_rows(rng, batch + 2, shapes, dtypes)
+            g.insert(to_dev(refill)), c.append(refill, batch + 2)
+    g.check()
+    g.set_option("device_counters", 0)
+    assert int(g.count) == c.count and int(g.head) == c.head
+    gi, gf = g.sample_with_indices()
+    ci, cf = c.sample(batch)
+    assert np.array_equal(t2n(gi), ci)
+    del graph
+    g.destroy()
+
+
 def test_config2_sac_shape_full_size(mrb, orc):
     """BASELINE config 2 at its real size: capacity 1,000,000, rows f32[17] + f32[6] + f32[1] + f32[17] + bool
     (165 B, mindspore_rl/algorithm/sac/config.py:95-100), filled by 1000 appends of 1000 rows

@@ -100,7 +100,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
     assert sum("k_per_sample_wide" in k for k in kernels) == 8 and sum("k_rows_gather_wide" in k for k in kernels) == 4
-    assert len(kernels) == 27, sorted(kernels)
+    assert len(kernels) == 29, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)
@@ -138,7 +138,8 @@ def test_only_the_documented_entry_points_wait_or_allocate():
     # device-resident counters are copied (with a wait) only where the header says so: switching the option,
     # state queries and the checkpoint calls - never by push, sample or update
     users = {n for n, b in bodies.items() if re.search(r"counters_(to|from)_device\(", b)}
-    assert users == {"mrb_set_option", "mrb_per_state", "mrb_per_get_counters", "mrb_per_set_counters"}, users
+    assert users == {"mrb_set_option", "mrb_per_state", "mrb_per_get_counters", "mrb_per_set_counters", "mrb_urb_state",
+                     "mrb_urb_reset", "mrb_urb_seed", "mrb_urb_get_counters", "mrb_urb_set_counters"}, users
     # the allocation-free entry point and the core it shares with mrb_per_update
     for name in ("mrb_per_update_noalloc", "per_update", "tree_rebuild", "next_epoch", "static_scratch"):
         assert not allocs.search(bodies[name]) and not waits.search(bodies[name]), name
