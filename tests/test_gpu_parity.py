@@ -1229,3 +1229,84 @@ def test_config3_atari_shape_properties(mrb, orc, cap):
     assert_tree_equal(g, c, "config 3 shape")
     assert g.check() == 0
     g.destroy()
+
+
+FUZZ_LAYOUTS = [([(3,), (1,)], [np.float32, np.int32]), ([(300,), (1,), (3,)], [np.float32, np.int32, np.uint8]),
+                ([(1,), (2,)], [np.int32, np.float32]),
+                ([(64,), (1,), (1,), (64,), (1,)], [np.float32, np.int32, np.float32, np.float32, np.bool_])]
+FUZZ_CAPS = [1, 3, 200, 257, 4096, 5000, 9000, 16384, 40000, 70000, 131072, 300000, 1 << 20, (1 << 20) + 7, 2_500_000,
+             5_000_000]
+
+
+@pytest.mark.parametrize("block", range(6))
+def test_random_configurations_and_operation_sequences(mrb, orc, block):
+    """Ten seeded random cases per block: capacity (trees of 0 to 23 levels), row layout, alpha, batch, sample
+    kernel, fused or per-round rebuilds, workgroups per row, counters on the host or on the device - then a random
+    sequence of pushes (with and without priorities, from 1 row to more than the capacity), updates (sizes on both
+    sides of every threshold, duplicates, many entries in one leaf tile, zero priorities), samples with given
+    draws, with the generator, several batches per launch. Trees, size, head, running max and every sample are
+    compared with the oracle after every operation."""
+    for case in range(10):
+        seed = 7000 + 10 * block + case
+        rng = np.random.default_rng(seed)
+        cap = int(FUZZ_CAPS[rng.integers(0, len(FUZZ_CAPS))])
+        shapes, dtypes = FUZZ_LAYOUTS[rng.integers(0, len(FUZZ_LAYOUTS))] if cap < 400000 else FUZZ_LAYOUTS[2]
+        alpha = float(rng.choice([0.0, 0.4, 0.6, 1.0, 1.5]))
+        batch = int(rng.choice([1, 8, 33, 64, 256]))
+        g, c = make_pair(mrb, orc, alpha, cap, batch, seed=seed + 1, shapes=shapes, dtypes=dtypes)
+        g.set_option("sample_path", int(rng.integers(0, 3)))
+        g.set_option("fused_rebuild", int(rng.integers(0, 2)))
+        g.set_option("row_split", int(rng.choice([0, 0, 2, 3])))
+        dev = bool(rng.integers(0, 2))
+        g.set_option("device_counters", int(dev))
+        tag = "seed %d cap %d alpha %.1f batch %d dev %d" % (seed, cap, alpha, batch, dev)
+        fill, done = int(rng.choice([cap, cap, max(1, cap // 2), max(1, cap - 5)])), 0
+        while done < fill:
+            n = min(fill - done, 1 << 18)
+            rows = random_rows(rng, n, shapes, dtypes)
+            pr = (rng.pareto(1.5, n) + 1e-6).astype(np.float32) if rng.integers(0, 2) else None
+            g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda() if pr is not None else None)
+            c.push(rows, n, pr) if pr is not None else c.push(rows, n)
+            done += n
+        assert_tree_equal(g, c, tag + " prefill")
+        for step in range(int(rng.integers(6, 14))):
+            op = int(rng.integers(0, 5))
+            what = "%s step %d op %d" % (tag, step, op)
+            if op == 0:
+                hi = min(cap, 6000) if dev else min(2 * cap + 2, 6000)
+                n = max(1, min(int(rng.choice([1, 3, int(rng.integers(1, 300)), int(rng.integers(1, hi + 1))])), hi))
+                rows = random_rows(rng, n, shapes, dtypes)
+                pr = None
+                if rng.integers(0, 2):
+                    pr = (rng.pareto(1.5, n) + 1e-6).astype(np.float32)
+                    if rng.integers(0, 3) == 0:
+                        pr[rng.integers(0, n)] = np.float32(c.max_priority) * 2 + 1
+                g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda() if pr is not None else None)
+                c.push(rows, n, pr) if pr is not None else c.push(rows, n)
+            elif op == 1:
+                hi = 1024 if dev else 3000
+                n = int(rng.choice([1, 7, 16, 17, 64, int(rng.integers(1, hi + 1)), hi]))
+                idx = rng.integers(0, cap, n)
+                if n > 4 and rng.integers(0, 2):
+                    idx[: n // 3] = idx[0]
+                if n > 4 and rng.integers(0, 2):
+                    idx[n // 2:] = np.minimum(idx[n // 2] // 256 * 256 + rng.integers(0, 256, n - n // 2), cap - 1)
+                pr = (rng.pareto(1.5, n) + 1e-6).astype(np.float32)
+                if cap > 100 and rng.integers(0, 4) == 0:
+                    pr[rng.integers(0, n)] = 0.0
+                g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda()), c.update(idx, pr)
+            elif op == 2:
+                u, beta = rng.random(batch).astype(np.float32), float(rng.uniform(0, 1))
+                assert_sample_equal(g.sample(beta, uniforms=torch.from_numpy(u).cuda()), c.sample(batch, beta, u), what)
+            elif op == 3:
+                beta = float(rng.uniform(0, 1))
+                assert_sample_equal(g.sample(beta), c.sample(batch, beta), what)
+            else:
+                nb, beta = int(rng.integers(1, 5)), float(rng.uniform(0, 1))
+                got = g.sample_many(nb, beta)
+                for i in range(nb):
+                    assert_sample_equal([x[i] for x in got], c.sample(batch, beta), what + " batch %d" % i)
+            assert_tree_equal(g, c, what)
+            assert g.size() == c.size and g._state()[1] == c.head, what
+            assert np.float32(g.max_priority) == np.float32(c.max_priority), what
+        g.destroy()
