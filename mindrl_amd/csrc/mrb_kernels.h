@@ -1487,7 +1487,14 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, int* w
     const int g1 = top < kRoundLevels ? top : kRoundLevels;
     const uint32_t tiles = (1u << top) <= (uint32_t)kBlockNodes ? 1u : (1u << top) / kBlockNodes;
     if (a.inline_election && top == a.depth) entry_duty(a, wave, nwaves, lane);
-    for (uint32_t t = wave; t < tiles; t += nwaves)
+    // A push that does not wrap changed the nodes above one run of slots only: above the leaf level, the
+    // tiles outside that run hold what they held, and the waves they would occupy stay out of the way.
+    uint32_t t_lo = 0, t_hi = tiles - 1;
+    if (!a.indices && top != a.depth && a.first_slot >= 0 && a.first_slot + a.n <= a.capacity) {
+        t_lo = (uint32_t)(a.first_slot >> (a.depth - top)) / kBlockNodes;
+        t_hi = (uint32_t)((a.first_slot + a.n - 1) >> (a.depth - top)) / kBlockNodes;
+    }
+    for (uint32_t t = t_lo + wave; t <= t_hi; t += nwaves)
         tile_round(a, top, g1, t, top == a.depth && g1 >= 2, nullptr, nullptr, 0, lane, win + wave * kBlockNodes);
     if (top > g1) {
         __threadfence_block();  // the tiles' parents, written by other waves of this workgroup, are read below
