@@ -1494,8 +1494,19 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, int* w
         t_lo = (uint32_t)(a.first_slot >> (a.depth - top)) / kBlockNodes;
         t_hi = (uint32_t)((a.first_slot + a.n - 1) >> (a.depth - top)) / kBlockNodes;
     }
-    for (uint32_t t = t_lo + wave; t <= t_hi; t += nwaves)
-        tile_round(a, top, g1, t, top == a.depth && g1 >= 2, nullptr, nullptr, 0, lane, win + wave * kBlockNodes);
+    if (top != a.depth && g1 == kRoundLevels) {
+        // full tiles above the leaf level: nothing to elect, no clean blocks - the nodes and their eight levels
+        // of parents, without tile_round's cases (sixteen waves share this compute unit's issue slots)
+        for (uint32_t t = t_lo + wave; t <= t_hi; t += nwaves) {
+            const uint32_t first = (1u << top) + t * kBlockNodes;
+            const float4 vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * lane);
+            const float4 vm = *reinterpret_cast<const float4*>(a.mn + first + 4 * lane);
+            tile_parents(a, kRoundLevels, first, lane, true, vs, vm);
+        }
+    } else {
+        for (uint32_t t = t_lo + wave; t <= t_hi; t += nwaves)
+            tile_round(a, top, g1, t, top == a.depth && g1 >= 2, nullptr, nullptr, 0, lane, win + wave * kBlockNodes);
+    }
     if (top > g1) {
         __threadfence_block();  // the tiles' parents, written by other waves of this workgroup, are read below
         __syncthreads();
