@@ -374,7 +374,7 @@ def bench_per(a):
     else:
         out["roofline"] = roofline(kernel_name, algo_bytes, dev_s / K, wall / K, a.workload, formula, defaults)
     if not a.no_extras:
-        out["extras"] = per_extras(a, torch, r)
+        out["extras"] = per_extras(a, torch, r, algo_bytes)
     if a.no_cpu_baseline:
         out["cpu_baseline"] = None
     elif r.loop_step:
@@ -386,7 +386,7 @@ def bench_per(a):
     return 0
 
 
-def per_extras(a, torch, r):
+def per_extras(a, torch, r, algo_bytes):
     """Untimed side figures: the other operations of the config's step, the same sample steps replayed from
     a HIP graph, and issued round robin on several streams (independent calls, one output set per stream)."""
     L, h, sp, K, W, batch = r.L, r.h, r.sp, r.K, r.W, r.batch
@@ -483,19 +483,18 @@ def per_extras(a, torch, r):
         for _ in range(4):
             st = torch.cuda.Stream()
             f = r.buf._layout.empty(batch, r.buf._dev)
-            sets.append((C.c_void_p(st.cuda_stream), (torch.empty(batch, dtype=torch.int64, device="cuda"),
-                                                      torch.empty(batch, dtype=torch.float32, device="cuda"), f), st))
+            io_, wo_ = torch.empty(batch, dtype=torch.int64, device="cuda"), torch.empty(batch, dtype=torch.float32, device="cuda")
+            sets.append((C.c_void_p(st.cuda_stream), (io_.data_ptr(), wo_.data_ptr(), r.pointers(f)), (io_, wo_, f, st)))
         torch.cuda.synchronize()
         pipelined = {}
         for ns in (2, 4):
             def rr(i):
-                s_, (i_, w_, f_), _ = sets[i % ns]
-                r.sample(W + i % K, s_, (i_.data_ptr(), w_.data_ptr(), r.pointers(f_)))
+                s_, out_, _ = sets[i % ns]
+                r.sample(W + i % K, s_, out_)
             pipelined[str(ns)] = timed(rr, max(n_it, 200)) * 1e6
         extras["streams_round_robin_us_per_call"] = pipelined
         row_bytes = sum(r.buf._layout.bytes)
-        extras["streams_round_robin_frac_of_peak"] = (batch * (2 * row_bytes + 12) / (min(pipelined.values()) * 1e-6)
-                                                      / 1e9 / HBM_PEAK_GBS)
+        extras["streams_round_robin_frac_of_peak"] = algo_bytes / (min(pipelined.values()) * 1e-6) / 1e9 / HBM_PEAK_GBS
         # several batches per launch (mrb_per_sample_many): the launch and the descent are paid once for
         # all of them, which is what a learner that prefetches batches between priority updates can use
         many = {}
@@ -523,7 +522,7 @@ def per_extras(a, torch, r):
             torch.cuda.synchronize()
             us = e0.elapsed_time(e1) * 1e3 / (reps * nb)
             many[str(nb)] = {"us_per_batch": us,
-                             "frac_of_peak": batch * (2 * row_bytes + 12) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+                             "frac_of_peak": algo_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
             del fo, io, wo
         extras["sample_many_batches_per_launch"] = many
     r.buf.check()

@@ -434,14 +434,6 @@ uint32_t push_units(const UpdateArgs& a) {
 // its row copy over (`ride`): it is done by extra workgroups of the first launch.
 int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = nullptr) {
     PutArgs none{};  // blocks == 0: no copy rides along
-    // A push of at most 1024 rows into a tree of at most 16 levels is one launch: the single workgroup of
-    // k_tree_top starts at the leaf level and skips the tiles outside the slot range (such a call is
-    // launch-bound, not work-bound). Measured on 16,384 leaves: 6.3 us instead of 8.0. Updates keep their
-    // leaf round: their waves scan the entries, which one workgroup does more slowly (11.5 vs 9.8 us).
-    if (a.nrounds > 0 && !a.indices && a.n <= 1024 && a.depth <= 16) {
-        a.nrounds = 0;
-        a.top_depth = a.depth;
-    }
     // One round below the top and at most 16 waves of work (an update: a wave per entry; a push that does
     // not wrap: a wave per leaf tile under its slots): one launch of one workgroup that goes on to the top.
     // (More units per wave do not pay: the 16 waves of a workgroup share one compute unit's issue slots, and a
@@ -463,6 +455,14 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
             LAUNCH_CHECK("k_tree_fused");
             return MRB_OK;
         }
+    }
+    // A push of at most 1024 rows into a tree of at most 16 levels is one launch: the single workgroup of
+    // k_tree_top starts at the leaf level and skips the tiles outside the slot range (such a call is
+    // launch-bound, not work-bound). Measured on 16,384 leaves: 6.3 us instead of 8.0. Updates keep their
+    // leaf round: their waves scan the entries, which one workgroup does more slowly (11.5 vs 9.8 us).
+    if (a.nrounds > 0 && !a.indices && a.n <= 1024 && a.depth <= 16) {
+        a.nrounds = 0;
+        a.top_depth = a.depth;
     }
     for (int r = 0; r < a.nrounds; ++r) {
         uint32_t tiles = (1u << a.lo[r]) / kBlockNodes;
@@ -899,23 +899,20 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     }
     b->alpha = alpha;
     b->seed = seed;
-    // Rebuild plan: the top (<= 12 levels) belongs to the last workgroup of the last round; the levels
-    // below it are split as evenly as possible into rounds of 2..8 levels.
+    // Rebuild plan: a tree of at most 12 levels is one workgroup's work (the top). A taller one gets as few
+    // rounds (launches of a wave per 256-node tile) below its top as possible, and every round takes the full
+    // 8 levels, which leaves the top - one workgroup, the end of every call's chain of launches - as low as
+    // it can be: up to 8 levels it is one tile and one pass, beyond that tiles, a barrier and a second pass.
     b->top_depth = b->depth < kTopMaxDepth ? b->depth : kTopMaxDepth;
-    int rest = b->depth - b->top_depth;
-    if (rest == 1) {  // a round needs at least two levels (a lane's four nodes must share a block)
-        rest = 2;
-        b->top_depth -= 1;
+    if (const int rest = b->depth - b->top_depth; rest > 0) {
+        // (21 levels: a top one level deeper, 32 tiles, saves a whole round, i.e. a launch)
+        b->nrounds = rest == kRoundLevels + 1 ? 1 : (rest + kRoundLevels - 1) / kRoundLevels;
+        b->top_depth = b->depth - kRoundLevels * b->nrounds;
     }
-    if (rest == kRoundLevels + 1) {  // 21 levels: a top one level deeper (32 tiles) saves a whole round, i.e. a launch
-        rest = kRoundLevels;
-        b->top_depth += 1;
-    }
-    b->nrounds = (rest + kRoundLevels - 1) / kRoundLevels;
     for (int r = 0, lo = b->depth; r < b->nrounds; ++r) {
         b->lo[r] = lo;
-        b->g[r] = rest / b->nrounds + (r < rest % b->nrounds ? 1 : 0);
-        lo -= b->g[r];
+        b->g[r] = kRoundLevels;
+        lo -= kRoundLevels;
     }
     const size_t nodes = 2 * (size_t)b->leaves;
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->sum), nodes * sizeof(float)));
@@ -1242,7 +1239,9 @@ int mrb_res_push(int64_t h, const void* const* src_fields, int64_t nrows, void* 
     if (elect) {
         b->epoch += 1;
         if ((uint32_t)b->epoch == 0) {
-            HIP_TRY(hipMemsetAsync(b->stamp, 0, (size_t)cap * sizeof(unsigned long long), s));
+            // by a fill kernel, not a memset node: the caller may be capturing this stream
+            fill_zero(b->stamp, (size_t)cap * sizeof(unsigned long long), s);
+            LAUNCH_CHECK("k_fill_f32");
             b->epoch += 1;
         }
         hipLaunchKernelGGL(k_res_elect, dim3(grid_exact((uint64_t)nrows)), dim3(kWG), 0, s, b->stamp, b->total, nrows,
@@ -1396,7 +1395,9 @@ int mrb_discounted_return(const float* reward, const uint8_t* done, const float*
     if (!(gamma >= 0.0f && gamma <= 1.0f))
         return fail(MRB_EINVAL, "The discounted factor should be a number in range [0, 1], but got %g.", (double)gamma);
     const int64_t cols = batch * inner;
-    if (cols > (1ll << 40) / timesteps) return fail(MRB_EINVAL, "problem too large");
+    if (cols > (1ll << 31) || cols > (1ll << 40) / timesteps)
+        return fail(MRB_EINVAL, "%lld columns of %lld steps exceed one call (at most 2^31 columns, 2^40 elements)",
+                    (long long)cols, (long long)timesteps);
     if (cols <= 256 * kDrCols) {
         // few columns (at most one 64-column tile per compute unit): a thread per column cannot keep
         // enough loads in flight; stage chunks through LDS
