@@ -164,6 +164,25 @@ __device__ __forceinline__ float lane_value(float x, uint32_t src_lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)src_lane));
 }
 
+// The value lane ^ (1 << S) holds, S = 0..3, moved inside the register file (DPP) rather than through the
+// LDS crossbar a generic shuffle takes. For S = 2 and 3 the source is the mirrored lane of the 8- or 16-lane
+// group: it holds what lane ^ (1 << S) holds once the lanes of every aligned group of 2^S lanes agree, which
+// is the case after butterfly steps 0 .. S-1 of a commutative operation.
+template <int S>
+__device__ __forceinline__ float butterfly_peer(float x) {
+    static_assert(S >= 0 && S <= 3, "within a row of 16 lanes");
+    return dpp_move<S == 0 ? 0xB1 : S == 1 ? 0x4E : S == 2 ? 0x141 : 0x140>(x);
+}
+
+// Largest value of the wave, in every lane (max is exact: the order of the comparisons does not matter).
+__device__ __forceinline__ float wave_max(float q) {
+    q = fmaxf(q, butterfly_peer<0>(q));
+    q = fmaxf(q, butterfly_peer<1>(q));
+    q = fmaxf(q, butterfly_peer<2>(q));
+    q = fmaxf(q, butterfly_peer<3>(q));
+    return fmaxf(fmaxf(lane_value(q, 0), lane_value(q, 16)), fmaxf(lane_value(q, 32), lane_value(q, 48)));
+}
+
 // Walks the g levels held in `v` (this lane's 16 consecutive bottom nodes), starting
 // at the group's root with `mass`. Returns the offset of the node reached among the
 // group's 2^g bottom nodes; `mass` is left as the remainder, `picked` receives that

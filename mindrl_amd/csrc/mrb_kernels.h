@@ -1066,7 +1066,7 @@ __global__ __launch_bounds__(kWG) void k_update_stamp(UpdateArgs a) {
         }
     }
     // wave max, then one integer atomic per wave
-    for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+    q = wave_max(q);
     if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
 }
 
@@ -1119,6 +1119,18 @@ __device__ __forceinline__ bool range_meets(const UpdateArgs& a, int64_t first_s
 // The g levels above a tile whose nodes (four per lane, vs / vm) are final: parents by in-lane
 // operations and wave shuffles, stored by the lanes of dirty blocks (`active`). `first`: heap index
 // of the tile's first node.
+// One butterfly step of tile_parents: level 3 + S above the tile, one node per 2^(S+1) lanes.
+template <int S>
+__device__ __forceinline__ void parents_step(const UpdateArgs& a, int g, uint32_t first, uint32_t lane, bool active,
+                                             float& cs, float& cm) {
+    cs = cs + butterfly_peer<S>(cs);
+    cm = fminf(cm, butterfly_peer<S>(cm));
+    if (active && g >= 3 + S && (lane & ((2u << S) - 1)) == 0) {
+        a.sum[(first >> (3 + S)) + (lane >> (S + 1))] = cs;
+        a.mn[(first >> (3 + S)) + (lane >> (S + 1))] = cm;
+    }
+}
+
 __device__ __forceinline__ void tile_parents(const UpdateArgs& a, int g, uint32_t first, uint32_t lane, bool active,
                                              const float4& vs, const float4& vm) {
     // one level up: two nodes per lane; two levels up: one node per lane
@@ -1133,15 +1145,21 @@ __device__ __forceinline__ void tile_parents(const UpdateArgs& a, int g, uint32_
         a.sum[(first >> 2) + lane] = cs;
         a.mn[(first >> 2) + lane] = cm;
     }
-    // three to eight levels up: 32, 16, 8, 4, 2, 1 nodes per full tile
-#pragma unroll
-    for (int s = 0; s < 6; ++s) {
-        cs = cs + __shfl_xor(cs, 1 << s);
-        cm = fminf(cm, __shfl_xor(cm, 1 << s));
-        if (active && g >= 3 + s && (lane & ((2u << s) - 1)) == 0) {
-            a.sum[(first >> (3 + s)) + (lane >> (s + 1))] = cs;
-            a.mn[(first >> (3 + s)) + (lane >> (s + 1))] = cm;
-        }
+    // three to six levels up: 32, 16, 8, 4 nodes per full tile, a butterfly inside each row of 16 lanes
+    parents_step<0>(a, g, first, lane, active, cs, cm);
+    parents_step<1>(a, g, first, lane, active, cs, cm);
+    parents_step<2>(a, g, first, lane, active, cs, cm);
+    parents_step<3>(a, g, first, lane, active, cs, cm);
+    // seven and eight levels up: the four rows' values, read as scalars (left + right as everywhere)
+    const float s_lo = lane_value(cs, 0) + lane_value(cs, 16), s_hi = lane_value(cs, 32) + lane_value(cs, 48);
+    const float m_lo = fminf(lane_value(cm, 0), lane_value(cm, 16)), m_hi = fminf(lane_value(cm, 32), lane_value(cm, 48));
+    if (active && g >= 7 && (lane & 31) == 0) {
+        a.sum[(first >> 7) + (lane >> 5)] = lane < 32 ? s_lo : s_hi;
+        a.mn[(first >> 7) + (lane >> 5)] = lane < 32 ? m_lo : m_hi;
+    }
+    if (active && g >= 8 && lane == 0) {
+        a.sum[first >> 8] = s_lo + s_hi;
+        a.mn[first >> 8] = fminf(m_lo, m_hi);
     }
 }
 
@@ -1282,7 +1300,7 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
         // a value no larger than the running max: folding it in raises the running max to exactly what a pass
         // over the call's priorities would
         float q = active ? fmaxf(fmaxf(vs.x, vs.y), fmaxf(vs.z, vs.w)) : 0.0f;
-        for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+        q = wave_max(q);
         if (lane == 0 && q > 0.0f) raise_max(a.maxp_next, q);
     }
     tile_parents(a, g, first, lane, active, vs, vm);
@@ -1296,6 +1314,20 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
 // group loads the block, replaces the leaves the stamps name, rebuilds the g0 levels
 // above with the same pairwise operations as tile_round and marks the next round's block.
 // ---------------------------------------------------------------------------
+// One butterfly step of k_tree_sparse inside an entry's group of lanes: level 3 + S above its block.
+template <int S>
+__device__ __forceinline__ void sparse_step(const UpdateArgs& a, int g0, uint64_t first, uint32_t sub, bool active,
+                                            float& cs, float& cm) {
+    if (S < g0 - 2) {  // wave-uniform
+        cs = cs + butterfly_peer<S>(cs);
+        cm = fminf(cm, butterfly_peer<S>(cm));
+        if (active && (sub & ((2u << S) - 1)) == 0) {
+            a.sum[(first >> (3 + S)) + (sub >> (S + 1))] = cs;
+            a.mn[(first >> (3 + S)) + (sub >> (S + 1))] = cm;
+        }
+    }
+}
+
 __global__ __launch_bounds__(kWG) void k_tree_sparse(UpdateArgs a) {
     const int g0 = a.sparse_g0;
     const uint32_t group = 1u << (g0 - 2);
@@ -1351,17 +1383,10 @@ __global__ __launch_bounds__(kWG) void k_tree_sparse(UpdateArgs a) {
         a.sum[(first >> 2) + sub] = cs;
         a.mn[(first >> 2) + sub] = cm;
     }
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-        if (s < g0 - 2) {  // wave-uniform
-            cs = cs + __shfl_xor(cs, 1 << s);
-            cm = fminf(cm, __shfl_xor(cm, 1 << s));
-            if (active && (sub & ((2u << s) - 1)) == 0) {
-                a.sum[(first >> (3 + s)) + (sub >> (s + 1))] = cs;
-                a.mn[(first >> (3 + s)) + (sub >> (s + 1))] = cm;
-            }
-        }
-    }
+    sparse_step<0>(a, g0, first, sub, active, cs, cm);
+    sparse_step<1>(a, g0, first, sub, active, cs, cm);
+    sparse_step<2>(a, g0, first, sub, active, cs, cm);
+    sparse_step<3>(a, g0, first, sub, active, cs, cm);
 }
 
 // Small update without a stamp pass: what k_update_stamp does besides electing — flag invalid
@@ -1379,7 +1404,7 @@ __device__ __forceinline__ void entry_duty(const UpdateArgs& a, uint32_t wave_id
             if (!valid_priority(p)) atomicOr(a.err, MRB_DERR_PRIORITY);
             if (idx_ok && valid_priority(p)) q = powf_det_call(p, a.alpha);
         }
-        for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+        q = wave_max(q);
         if (lane == 0 && q > 0.0f) raise_max(a.maxp, q);
     }
 }
@@ -1407,7 +1432,7 @@ __device__ __forceinline__ void fold_push_max(const UpdateArgs& a) {
             atomicOr(a.err, MRB_DERR_PRIORITY);
         }
     }
-    for (int s = 32; s >= 1; s >>= 1) q = fmaxf(q, __shfl_xor(q, s));
+    q = wave_max(q);
     if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
 }
 
