@@ -1110,7 +1110,7 @@ __device__ __forceinline__ bool range_meets(const UpdateArgs& a, int64_t first_s
 //              a block is dirty if its word in dirty_in carries this call's epoch or, at the
 //              leaf level of a push (dirty_in NULL), if it meets the pushed slot range
 //   dirty_out  next round's words, marked for every block rebuilt here (may be NULL)
-//   win        this wave's 256 ints of LDS, used at the leaf level of a small update
+//   win        this wave's 256 eight-byte words of LDS, used at the leaf level of a small update
 //              (a.inline_election): the wave scans the call's entries itself, the last entry
 //              aimed at each of its leaves wins through an LDS integer max (last write wins),
 //              and the blocks holding a winner are the dirty ones
@@ -1119,6 +1119,14 @@ __device__ __forceinline__ bool range_meets(const UpdateArgs& a, int64_t first_s
 // The g levels above a tile whose nodes (four per lane, vs / vm) are final: parents by in-lane
 // operations and wave shuffles, stored by the lanes of dirty blocks (`active`). `first`: heap index
 // of the tile's first node.
+// The LDS word a small update's entry bids for its leaf with: the entry's position in the call (plus one, so
+// that zero means no bid) above its priority's bits. An integer max over the bids elects the last entry aimed
+// at the leaf, and the winner's priority comes back with it (no second trip to the call's arrays).
+__device__ __forceinline__ unsigned long long election_key(int64_t j, float p) {
+    return ((unsigned long long)(j + 1) << 32) | (unsigned long long)__float_as_uint(p);
+}
+__device__ __forceinline__ float elected_priority(unsigned long long key) { return __uint_as_float((uint32_t)key); }
+
 // One butterfly step of tile_parents: level 3 + S above the tile, one node per 2^(S+1) lanes.
 template <int S>
 __device__ __forceinline__ void parents_step(const UpdateArgs& a, int g, uint32_t first, uint32_t lane, bool active,
@@ -1165,7 +1173,7 @@ __device__ __forceinline__ void tile_parents(const UpdateArgs& a, int g, uint32_
 
 __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, uint32_t tile, bool sparse,
                                            const uint32_t* __restrict__ dirty_in, uint32_t* __restrict__ dirty_out,
-                                           int g_next, uint32_t lane, int* win = nullptr) {
+                                           int g_next, uint32_t lane, unsigned long long* win = nullptr) {
     const uint32_t level_nodes = 1u << lo;
     const bool leaf_level = lo == a.depth;
     // where a push's slots start (a.first_slot, or read from the device)
@@ -1200,12 +1208,12 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
     const uint32_t first = level_nodes + tile * kBlockNodes;  // heap index of the tile's first node
     bool active = 4 * lane < tile_nodes;
     const bool elect = leaf_level && a.inline_election && win != nullptr;
-    int jw0 = -1, jw1 = -1, jw2 = -1, jw3 = -1;  // winning entry of each of this lane's leaves
+    unsigned long long w0 = 0, w1 = 0, w2 = 0, w3 = 0;  // winning entry of each of this lane's leaves (election_key)
     if (elect) {
-        win[4 * lane + 0] = -1;
-        win[4 * lane + 1] = -1;
-        win[4 * lane + 2] = -1;
-        win[4 * lane + 3] = -1;
+        win[4 * lane + 0] = 0;
+        win[4 * lane + 1] = 0;
+        win[4 * lane + 2] = 0;
+        win[4 * lane + 3] = 0;
         __builtin_amdgcn_wave_barrier();
         // four entries per lane and trip: their loads go out together, then the election
         for (int64_t base = 0; base < a.n; base += 64 * 4) {
@@ -1221,16 +1229,16 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
             for (int q = 0; q < 4; ++q) {
                 if (idx[q] >= 0 && idx[q] < a.capacity && valid_priority(pr[q]) &&
                     (uint32_t)((uint64_t)idx[q] / kBlockNodes) == tile)
-                    atomicMax(&win[idx[q] % kBlockNodes], (int)(base + 64 * q + lane));
+                    atomicMax(&win[idx[q] % kBlockNodes], election_key(base + 64 * q + lane, pr[q]));
             }
         }
         __threadfence_block();  // LDS operations of a wave complete in order; this also stops the compiler
         __builtin_amdgcn_wave_barrier();
-        jw0 = win[4 * lane + 0];
-        jw1 = win[4 * lane + 1];
-        jw2 = win[4 * lane + 2];
-        jw3 = win[4 * lane + 3];
-        const unsigned long long hit = __ballot(jw0 >= 0 || jw1 >= 0 || jw2 >= 0 || jw3 >= 0);
+        w0 = win[4 * lane + 0];
+        w1 = win[4 * lane + 1];
+        w2 = win[4 * lane + 2];
+        w3 = win[4 * lane + 3];
+        const unsigned long long hit = __ballot((w0 | w1 | w2 | w3) != 0);
         const uint32_t lanes_per_block = g >= 8 ? 64u : (1u << g) / 4u;
         const unsigned long long block_lanes =
             lanes_per_block >= 64 ? ~0ull : ((1ull << lanes_per_block) - 1) << (lane & ~(lanes_per_block - 1));
@@ -1251,10 +1259,10 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
             float q;
             bool wrote = false;
             if (elect) {
-                if (jw0 >= 0) { vs.x = vm.x = powf_det_call(a.priorities[jw0], a.alpha); wrote = true; }
-                if (jw1 >= 0) { vs.y = vm.y = powf_det_call(a.priorities[jw1], a.alpha); wrote = true; }
-                if (jw2 >= 0) { vs.z = vm.z = powf_det_call(a.priorities[jw2], a.alpha); wrote = true; }
-                if (jw3 >= 0) { vs.w = vm.w = powf_det_call(a.priorities[jw3], a.alpha); wrote = true; }
+                if (w0) { vs.x = vm.x = powf_det_call(elected_priority(w0), a.alpha); wrote = true; }
+                if (w1) { vs.y = vm.y = powf_det_call(elected_priority(w1), a.alpha); wrote = true; }
+                if (w2) { vs.z = vm.z = powf_det_call(elected_priority(w2), a.alpha); wrote = true; }
+                if (w3) { vs.w = vm.w = powf_det_call(elected_priority(w3), a.alpha); wrote = true; }
             } else if (!a.indices && a.priorities) {
                 // a push with priorities: the lane's four priorities are requested together, then raised to
                 // alpha one after the other (asked for one by one, each power would wait for its own load)
@@ -1443,7 +1451,7 @@ __device__ __forceinline__ void fold_push_max(const UpdateArgs& a) {
 // depend on: the entry, the first entries of the scan and then the tile are requested before the
 // election runs.
 // dirty_out: the next round's words, marked for every block rebuilt here (NULL when the top comes next).
-__device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t j, uint32_t lane, int* win,
+__device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t j, uint32_t lane, unsigned long long* win,
                                            uint32_t* __restrict__ dirty_out, int g_next) {
     constexpr int kPer = 4;  // entries per lane and trip of the scan
     int64_t idx[kPer];
@@ -1456,10 +1464,10 @@ __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t 
         idx[q] = e < a.n ? a.indices[e] : -1;
         pr[q] = e < a.n ? a.priorities[e] : -1.0f;
     }
-    win[4 * lane + 0] = -1;
-    win[4 * lane + 1] = -1;
-    win[4 * lane + 2] = -1;
-    win[4 * lane + 3] = -1;
+    win[4 * lane + 0] = 0;
+    win[4 * lane + 1] = 0;
+    win[4 * lane + 2] = 0;
+    win[4 * lane + 3] = 0;
     if (idx_j < 0 || idx_j >= a.capacity || !valid_priority(p_j)) return;  // wave-uniform: an entry that is skipped
     const uint32_t tile = (uint32_t)((uint64_t)idx_j / kBlockNodes);
     const uint32_t first = (1u << a.depth) + tile * kBlockNodes;
@@ -1479,22 +1487,22 @@ __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t 
         for (int q = 0; q < kPer; ++q) {
             if (idx[q] >= 0 && idx[q] < a.capacity && valid_priority(pr[q]) &&
                 (uint32_t)((uint64_t)idx[q] / kBlockNodes) == tile)
-                atomicMax(&win[idx[q] % kBlockNodes], (int)(base + 64 * q + lane));  // the last entry wins
+                atomicMax(&win[idx[q] % kBlockNodes], election_key(base + 64 * q + lane, pr[q]));  // the last entry wins
         }
     }
     __threadfence_block();  // LDS operations of a wave complete in order; this also stops the compiler
     __builtin_amdgcn_wave_barrier();
-    const int jw0 = win[4 * lane + 0], jw1 = win[4 * lane + 1], jw2 = win[4 * lane + 2], jw3 = win[4 * lane + 3];
-    const unsigned long long hit = __ballot(jw0 >= 0 || jw1 >= 0 || jw2 >= 0 || jw3 >= 0);
+    const unsigned long long w0 = win[4 * lane + 0], w1 = win[4 * lane + 1], w2 = win[4 * lane + 2], w3 = win[4 * lane + 3];
+    const unsigned long long hit = __ballot((w0 | w1 | w2 | w3) != 0);
     const uint32_t lanes_per_block = g >= 8 ? 64u : (1u << g) / 4u;
     const unsigned long long block_lanes =
         lanes_per_block >= 64 ? ~0ull : ((1ull << lanes_per_block) - 1) << (lane & ~(lanes_per_block - 1));
     const bool active = (hit & block_lanes) != 0;  // this lane's block of 2^g leaves holds a winner
-    if (jw0 >= 0) vs.x = vm.x = powf_det_call(a.priorities[jw0], a.alpha);
-    if (jw1 >= 0) vs.y = vm.y = powf_det_call(a.priorities[jw1], a.alpha);
-    if (jw2 >= 0) vs.z = vm.z = powf_det_call(a.priorities[jw2], a.alpha);
-    if (jw3 >= 0) vs.w = vm.w = powf_det_call(a.priorities[jw3], a.alpha);
-    if (jw0 >= 0 || jw1 >= 0 || jw2 >= 0 || jw3 >= 0) {
+    if (w0) vs.x = vm.x = powf_det_call(elected_priority(w0), a.alpha);
+    if (w1) vs.y = vm.y = powf_det_call(elected_priority(w1), a.alpha);
+    if (w2) vs.z = vm.z = powf_det_call(elected_priority(w2), a.alpha);
+    if (w3) vs.w = vm.w = powf_det_call(elected_priority(w3), a.alpha);
+    if (w0 | w1 | w2 | w3) {
         *reinterpret_cast<float4*>(a.sum + first + 4 * lane) = vs;
         *reinterpret_cast<float4*>(a.mn + first + 4 * lane) = vm;
     }
@@ -1505,9 +1513,9 @@ __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t 
 
 // Rebuilds everything above depth `top` (<= 16) with one workgroup: first up to 8 levels over
 // the tiles of that depth (shared out among the waves), then the rest in one tile. When `top`
-// is the leaf level, clean tiles are skipped like in a round. `win`: 256 ints of LDS per wave
+// is the leaf level, clean tiles are skipped like in a round. `win`: 256 eight-byte words of LDS per wave
 // (see tile_round).
-__device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, int* win) {
+__device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, unsigned long long* win) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int g1 = top < kRoundLevels ? top : kRoundLevels;
     const uint32_t tiles = (1u << top) <= (uint32_t)kBlockNodes ? 1u : (1u << top) / kBlockNodes;
@@ -1544,7 +1552,7 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, int* w
 // `tile_base`: the launch covers tiles tile_base, tile_base + 1, ... only (a push knows which leaf
 // tiles its slot range meets).
 __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, uint32_t tile_base, PutArgs put) {
-    __shared__ int s_win[kWG / 64][kBlockNodes];
+    __shared__ unsigned long long s_win[kWG / 64][kBlockNodes];
     const uint32_t tile_blocks = gridDim.x - put.blocks;
     if (blockIdx.x >= tile_blocks) {
         rows_put_part(put, blockIdx.x - tile_blocks, put.blocks);
@@ -1589,7 +1597,7 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
 // multi-die part costs far more than a launch.
 constexpr int kTopWG = 1024;
 __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) {
-    __shared__ int s_win[kTopWG / 64][kBlockNodes];
+    __shared__ unsigned long long s_win[kTopWG / 64][kBlockNodes];
     if (blockIdx.x >= 1) {
         rows_put_part(put, blockIdx.x - 1, put.blocks);
         return;
@@ -1611,7 +1619,7 @@ __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) 
 constexpr int kFusedWG = 1024;
 
 __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t tile_base, uint32_t units, PutArgs put) {
-    __shared__ int s_win[kFusedWG / 64][kBlockNodes];
+    __shared__ unsigned long long s_win[kFusedWG / 64][kBlockNodes];
     if (blockIdx.x >= 1) {
         rows_put_part(put, blockIdx.x - 1, put.blocks);
         return;
