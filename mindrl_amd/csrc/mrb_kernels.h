@@ -1397,9 +1397,10 @@ __global__ __launch_bounds__(kWG) void k_tree_sparse(UpdateArgs a) {
     sparse_step<3>(a, g0, first, sub, active, cs, cm);
 }
 
-// Small update without a stamp pass: what k_update_stamp does besides electing — flag invalid
-// entries and fold every valid p^alpha into the running max — is shared out among the waves,
-// 64 entries at a time.
+// Small update on a tree whose leaves the top workgroup itself rebuilds (no stamp pass, no wave per entry):
+// what k_update_stamp does besides electing — flag invalid entries and fold every valid p^alpha into the
+// running max — is shared out among the waves, 64 entries at a time. (Where a wave per entry runs,
+// entry_tile does this for its own entry.)
 __device__ __forceinline__ void entry_duty(const UpdateArgs& a, uint32_t wave_id, uint32_t nwaves, uint32_t lane) {
     for (int64_t base = (int64_t)wave_id * 64; base < a.n; base += (int64_t)nwaves * 64) {
         const int64_t j = base + lane;
@@ -1468,11 +1469,22 @@ __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t 
     win[4 * lane + 1] = 0;
     win[4 * lane + 2] = 0;
     win[4 * lane + 3] = 0;
-    if (idx_j < 0 || idx_j >= a.capacity || !valid_priority(p_j)) return;  // wave-uniform: an entry that is skipped
+    // what k_update_stamp does for an entry besides electing: flag it if it is invalid (and skip it) ...
+    const bool idx_ok = idx_j >= 0 && idx_j < a.capacity, p_ok = valid_priority(p_j);
+    if (!idx_ok || !p_ok) {  // wave-uniform
+        if (lane == 0 && !idx_ok) atomicOr(a.err, MRB_DERR_INDEX);
+        if (lane == 0 && !p_ok) atomicOr(a.err, MRB_DERR_PRIORITY);
+        return;
+    }
     const uint32_t tile = (uint32_t)((uint64_t)idx_j / kBlockNodes);
     const uint32_t first = (1u << a.depth) + tile * kBlockNodes;
     float4 vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * lane);
     float4 vm = *reinterpret_cast<const float4*>(a.mn + first + 4 * lane);
+    // ... and fold its p^alpha into the running max. The power is taken here, inlined, while the tile and the
+    // scan's entries are on their way (a call would wait for every load in flight first): it is nearly always
+    // the value this wave's own leaf gets, and it costs as much as the tile's trip to memory.
+    const float q_j = powf_det(p_j, a.alpha);
+    if (lane == 0 && q_j > 0.0f) raise_max(a.maxp, q_j);
     __builtin_amdgcn_wave_barrier();
     for (int64_t base = 0; base < a.n; base += 64 * kPer) {
         if (base > 0) {
@@ -1498,10 +1510,26 @@ __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t 
     const unsigned long long block_lanes =
         lanes_per_block >= 64 ? ~0ull : ((1ull << lanes_per_block) - 1) << (lane & ~(lanes_per_block - 1));
     const bool active = (hit & block_lanes) != 0;  // this lane's block of 2^g leaves holds a winner
-    if (w0) vs.x = vm.x = powf_det_call(elected_priority(w0), a.alpha);
-    if (w1) vs.y = vm.y = powf_det_call(elected_priority(w1), a.alpha);
-    if (w2) vs.z = vm.z = powf_det_call(elected_priority(w2), a.alpha);
-    if (w3) vs.w = vm.w = powf_det_call(elected_priority(w3), a.alpha);
+    // The winners' powers: this wave's own entry has its power already; the other entries that won a leaf of
+    // the tile (few, if any) take theirs together, one per lane and trip, whichever of the lane's leaves it is.
+    const unsigned long long own = (unsigned long long)(j + 1) << 32;
+    uint32_t pending = 0;
+    if (w0) { if ((w0 >> 32 << 32) == own) vs.x = vm.x = q_j; else pending |= 1u; }
+    if (w1) { if ((w1 >> 32 << 32) == own) vs.y = vm.y = q_j; else pending |= 2u; }
+    if (w2) { if ((w2 >> 32 << 32) == own) vs.z = vm.z = q_j; else pending |= 4u; }
+    if (w3) { if ((w3 >> 32 << 32) == own) vs.w = vm.w = q_j; else pending |= 8u; }
+    while (__any(pending != 0)) {
+        if (pending) {
+            const int c = __ffs(pending) - 1;
+            const unsigned long long w = c == 0 ? w0 : c == 1 ? w1 : c == 2 ? w2 : w3;
+            const float q = powf_det_call(elected_priority(w), a.alpha);
+            if (c == 0) vs.x = vm.x = q;
+            if (c == 1) vs.y = vm.y = q;
+            if (c == 2) vs.z = vm.z = q;
+            if (c == 3) vs.w = vm.w = q;
+            pending &= pending - 1;
+        }
+    }
     if (w0 | w1 | w2 | w3) {
         *reinterpret_cast<float4*>(a.sum + first + 4 * lane) = vs;
         *reinterpret_cast<float4*>(a.mn + first + 4 * lane) = vm;
@@ -1573,7 +1601,6 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
         if ((int64_t)j >= a.n) return;
         entry_tile(a, g, j, lane, s_win[threadIdx.x >> 6], last_round ? nullptr : a.dirty[round + 1],
                    last_round ? 0 : a.g[round + 1]);
-        entry_duty(a, j, (uint32_t)a.n, lane);
         return;
     }
     if (round == 0 && !a.indices && a.first_slot < 0) {
@@ -1628,7 +1655,6 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
     if (const uint32_t unit = wave; unit < units) {
         if (a.inline_election) {
             entry_tile(a, a.g[0], unit, lane, s_win[wave], nullptr, 0);
-            entry_duty(a, unit, units, lane);
         } else {
             // (device-resident counters: the tiles start at the first slot's tile and wrap around the level)
             const uint32_t ring_tiles = (uint32_t)((a.capacity + kBlockNodes - 1) / kBlockNodes);  // the ring ends at `capacity`
