@@ -1454,7 +1454,8 @@ __device__ __forceinline__ void fold_push_max(const UpdateArgs& a) {
 // dirty_out: the next round's words, marked for every block rebuilt here (NULL when the top comes next).
 __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t j, uint32_t lane, unsigned long long* win,
                                            uint32_t* __restrict__ dirty_out, int g_next) {
-    constexpr int kPer = 4;  // entries per lane and trip of the scan
+    constexpr int kPer = 8;  // entries per lane and trip of the scan: a call of up to 512 entries is one trip,
+                             // all of its loads requested before anything waits
     int64_t idx[kPer];
     float pr[kPer];
     const int64_t idx_j = a.indices[j];
@@ -1497,6 +1498,7 @@ __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t 
         }
 #pragma unroll
         for (int q = 0; q < kPer; ++q) {
+            if (base + 64 * q >= a.n) break;  // wave-uniform: no entries left
             if (idx[q] >= 0 && idx[q] < a.capacity && valid_priority(pr[q]) &&
                 (uint32_t)((uint64_t)idx[q] / kBlockNodes) == tile)
                 atomicMax(&win[idx[q] % kBlockNodes], election_key(base + 64 * q + lane, pr[q]));  // the last entry wins
