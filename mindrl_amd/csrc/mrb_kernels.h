@@ -1259,10 +1259,15 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
             float q;
             bool wrote = false;
             if (elect) {
-                if (w0) { vs.x = vm.x = powf_det_call(elected_priority(w0), a.alpha); wrote = true; }
-                if (w1) { vs.y = vm.y = powf_det_call(elected_priority(w1), a.alpha); wrote = true; }
-                if (w2) { vs.z = vm.z = powf_det_call(elected_priority(w2), a.alpha); wrote = true; }
-                if (w3) { vs.w = vm.w = powf_det_call(elected_priority(w3), a.alpha); wrote = true; }
+                if (w0 | w1 | w2 | w3) {
+                    const float4 pw = powf_det_x4(make_float4(elected_priority(w0), elected_priority(w1), elected_priority(w2),
+                                                              elected_priority(w3)), a.alpha);  // the four together
+                    if (w0) vs.x = vm.x = pw.x;
+                    if (w1) vs.y = vm.y = pw.y;
+                    if (w2) vs.z = vm.z = pw.z;
+                    if (w3) vs.w = vm.w = pw.w;
+                    wrote = true;
+                }
             } else if (!a.indices && a.priorities) {
                 // a push with priorities: the lane's four priorities are requested together, then raised to
                 // alpha one after the other (asked for one by one, each power would wait for its own load)
@@ -1275,21 +1280,21 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
                     in[c] = (int64_t)off + c < a.capacity && j < a.n;
                     pv[c] = in[c] ? a.priorities[j] : 0.0f;
                 }
-                float qv[4];
+                if (in[0] || in[1] || in[2] || in[3]) {
+                    const float4 pw = powf_det_x4(make_float4(pv[0], pv[1], pv[2], pv[3]), a.alpha);  // the four together
+                    const float qv[4] = {pw.x, pw.y, pw.z, pw.w};
+                    float* const vsp[4] = {&vs.x, &vs.y, &vs.z, &vs.w};
+                    float* const vmp[4] = {&vm.x, &vm.y, &vm.z, &vm.w};
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    qv[c] = 0.0f;
-                    if (in[c]) {
-                        const bool ok = valid_priority(pv[c]);
-                        qv[c] = ok ? powf_det_call(pv[c], a.alpha) : *a.maxp;  // invalid: the fresh slot stays at the running max
-                        if (a.fold_max == 2 && !ok) atomicOr(a.err, MRB_DERR_PRIORITY);
-                        wrote = true;
+                    for (int c = 0; c < 4; ++c) {
+                        if (in[c]) {
+                            const bool ok = valid_priority(pv[c]);
+                            *vsp[c] = *vmp[c] = ok ? qv[c] : *a.maxp;  // invalid: the fresh slot stays at the running max
+                            if (a.fold_max == 2 && !ok) atomicOr(a.err, MRB_DERR_PRIORITY);
+                            wrote = true;
+                        }
                     }
                 }
-                if (in[0]) vs.x = vm.x = qv[0];
-                if (in[1]) vs.y = vm.y = qv[1];
-                if (in[2]) vs.z = vm.z = qv[2];
-                if (in[3]) vs.w = vm.w = qv[3];
             } else {
                 if (leaf_value(a, first_slot, off + 0, q)) { vs.x = vm.x = q; wrote = true; }
                 if (leaf_value(a, first_slot, off + 1, q)) { vs.y = vm.y = q; wrote = true; }
