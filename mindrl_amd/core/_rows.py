@@ -16,8 +16,17 @@ def device():
     return torch.device("cuda", torch.cuda.current_device())
 
 
+# torch's own accessors of the current device and its current stream, without the Stream object that
+# torch.cuda.current_stream() builds on every call (2.9 us a call against 0.1 us; the calls here are 4-9 us).
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def stream_ptr():
-    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """The current stream of the current device as the integer value of its hipStream_t (0 = the null stream)."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 class _DeviceView:
