@@ -478,7 +478,7 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
             tiles = (uint32_t)((a.first_slot + a.n - 1) / kBlockNodes) - tile_base + 1;
         }
         const PutArgs& put = (r == 0 && ride) ? *ride : none;
-        if (r == 0 && a.inline_election) tiles = (uint32_t)a.n;  // a wave per entry (see k_tree_update)
+        if (r == 0 && a.inline_election) tiles = (a.n > kPairedAbove ? 2u : 1u) * (uint32_t)a.n;  // one or two waves per entry (see k_tree_update)
         hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4 + put.blocks), dim3(kWG), 0, s, a, r, tile_base, put);
         LAUNCH_CHECK("k_tree_update");
     }

@@ -232,6 +232,10 @@ __device__ __forceinline__ float lane_value(float x, uint32_t src_lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)src_lane));
 }
 
+// A workgroup barrier for data handed over in LDS only: it waits for the wave's LDS operations, not for
+// its global loads and stores, which __syncthreads() would also wait for.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // The value lane ^ (1 << S) holds, S = 0..3, moved inside the register file (DPP) rather than through the
 // LDS crossbar a generic shuffle takes. For S = 2 and 3 the source is the mirrored lane of the 8- or 16-lane
 // group: it holds what lane ^ (1 << S) holds once the lanes of every aligned group of 2^S lanes agree, which

@@ -1450,75 +1450,75 @@ __device__ __forceinline__ void fold_push_max(const UpdateArgs& a) {
     if ((threadIdx.x & 63) == 0 && q > 0.0f) raise_max(a.maxp, q);
 }
 
-// A small update's wave: rebuilds the 256-leaf tile that entry j falls into, with every entry of
-// the call that falls into it (the last one aimed at a leaf wins, elected by an LDS integer max over
-// a scan of the call's entries), and the g levels above it. Entries that share a tile make their
-// waves write the same values to the same nodes. The loads are kept apart from what they do not
-// depend on: the entry, the first entries of the scan and then the tile are requested before the
-// election runs.
-// dirty_out: the next round's words, marked for every block rebuilt here (NULL when the top comes next).
-__device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t j, uint32_t lane, unsigned long long* win,
-                                           uint32_t* __restrict__ dirty_out, int g_next) {
-    constexpr int kPer = 8;  // entries per lane and trip of the scan: a call of up to 512 entries is one trip,
+// A small update, driven by its entries: the 256-leaf tile that entry j falls into is rebuilt with every entry
+// of the call that falls into it (the last one aimed at a leaf wins, elected by an LDS integer max over a scan
+// of the call's entries), and the g levels above it. Entries that share a tile have the same values written
+// to the same nodes. The pieces below are put together twice: entry_tile (one wave does everything) and
+// entry_pair (two waves share an entry: one takes the power and the tile, the other the election).
+constexpr int kScanPer = 8;  // entries per lane and trip of the scan: a call of up to 512 entries is one trip,
                              // all of its loads requested before anything waits
-    int64_t idx[kPer];
-    float pr[kPer];
-    const int64_t idx_j = a.indices[j];
-    const float p_j = a.priorities[j];
+
+// Requests the first trip's entries.
+__device__ __forceinline__ void scan_request(const UpdateArgs& a, uint32_t lane, int64_t (&idx)[kScanPer], float (&pr)[kScanPer]) {
 #pragma unroll
-    for (int q = 0; q < kPer; ++q) {
+    for (int q = 0; q < kScanPer; ++q) {
         const int64_t e = 64 * q + lane;
         idx[q] = e < a.n ? a.indices[e] : -1;
         pr[q] = e < a.n ? a.priorities[e] : -1.0f;
     }
+}
+
+__device__ __forceinline__ void clear_bids(unsigned long long* win, uint32_t lane) {
     win[4 * lane + 0] = 0;
     win[4 * lane + 1] = 0;
     win[4 * lane + 2] = 0;
     win[4 * lane + 3] = 0;
-    // what k_update_stamp does for an entry besides electing: flag it if it is invalid (and skip it) ...
-    const bool idx_ok = idx_j >= 0 && idx_j < a.capacity, p_ok = valid_priority(p_j);
-    if (!idx_ok || !p_ok) {  // wave-uniform
-        if (lane == 0 && !idx_ok) atomicOr(a.err, MRB_DERR_INDEX);
-        if (lane == 0 && !p_ok) atomicOr(a.err, MRB_DERR_PRIORITY);
-        return;
-    }
-    const uint32_t tile = (uint32_t)((uint64_t)idx_j / kBlockNodes);
-    const uint32_t first = (1u << a.depth) + tile * kBlockNodes;
-    float4 vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * lane);
-    float4 vm = *reinterpret_cast<const float4*>(a.mn + first + 4 * lane);
-    // ... and fold its p^alpha into the running max. The power is taken here, inlined, while the tile and the
-    // scan's entries are on their way (a call would wait for every load in flight first): it is nearly always
-    // the value this wave's own leaf gets, and it costs as much as the tile's trip to memory.
-    const float q_j = powf_det(p_j, a.alpha);
-    if (lane == 0 && q_j > 0.0f) raise_max(a.maxp, q_j);
-    __builtin_amdgcn_wave_barrier();
-    for (int64_t base = 0; base < a.n; base += 64 * kPer) {
+}
+
+// Every valid entry of the call that falls into `tile` bids for its leaf (idx / pr hold the first trip).
+__device__ __forceinline__ void scan_bids(const UpdateArgs& a, uint32_t tile, uint32_t lane, unsigned long long* win,
+                                          int64_t (&idx)[kScanPer], float (&pr)[kScanPer]) {
+    for (int64_t base = 0; base < a.n; base += 64 * kScanPer) {
         if (base > 0) {
 #pragma unroll
-            for (int q = 0; q < kPer; ++q) {
+            for (int q = 0; q < kScanPer; ++q) {
                 const int64_t e = base + 64 * q + lane;
                 idx[q] = e < a.n ? a.indices[e] : -1;
                 pr[q] = e < a.n ? a.priorities[e] : -1.0f;
             }
         }
 #pragma unroll
-        for (int q = 0; q < kPer; ++q) {
+        for (int q = 0; q < kScanPer; ++q) {
             if (base + 64 * q >= a.n) break;  // wave-uniform: no entries left
             if (idx[q] >= 0 && idx[q] < a.capacity && valid_priority(pr[q]) &&
                 (uint32_t)((uint64_t)idx[q] / kBlockNodes) == tile)
                 atomicMax(&win[idx[q] % kBlockNodes], election_key(base + 64 * q + lane, pr[q]));  // the last entry wins
         }
     }
-    __threadfence_block();  // LDS operations of a wave complete in order; this also stops the compiler
-    __builtin_amdgcn_wave_barrier();
+}
+
+// What k_update_stamp does for an entry besides electing: flags it if it is invalid. Returns whether it is valid.
+__device__ __forceinline__ bool entry_valid(const UpdateArgs& a, int64_t idx_j, float p_j, uint32_t lane, bool flag) {
+    const bool idx_ok = idx_j >= 0 && idx_j < a.capacity, p_ok = valid_priority(p_j);
+    if (flag && lane == 0 && !idx_ok) atomicOr(a.err, MRB_DERR_INDEX);
+    if (flag && lane == 0 && !p_ok) atomicOr(a.err, MRB_DERR_PRIORITY);
+    return idx_ok && p_ok;
+}
+
+// After the election: the tile (vs / vm as memory held it) takes the winners' powers, is stored, and its g
+// levels of parents with it. q_j: p^alpha of entry j, the power nearly every leaf written here gets; the other
+// entries that won a leaf of the tile (few, if any) take theirs together, one per lane and trip.
+// dirty_out: the next round's words, marked for every block rebuilt here (NULL when the top comes next).
+__device__ __forceinline__ void entry_finish(const UpdateArgs& a, int g, uint32_t j, uint32_t tile, uint32_t lane,
+                                             const unsigned long long* win, float4 vs, float4 vm, float q_j,
+                                             uint32_t* __restrict__ dirty_out, int g_next) {
+    const uint32_t first = (1u << a.depth) + tile * kBlockNodes;
     const unsigned long long w0 = win[4 * lane + 0], w1 = win[4 * lane + 1], w2 = win[4 * lane + 2], w3 = win[4 * lane + 3];
     const unsigned long long hit = __ballot((w0 | w1 | w2 | w3) != 0);
     const uint32_t lanes_per_block = g >= 8 ? 64u : (1u << g) / 4u;
     const unsigned long long block_lanes =
         lanes_per_block >= 64 ? ~0ull : ((1ull << lanes_per_block) - 1) << (lane & ~(lanes_per_block - 1));
     const bool active = (hit & block_lanes) != 0;  // this lane's block of 2^g leaves holds a winner
-    // The winners' powers: this wave's own entry has its power already; the other entries that won a leaf of
-    // the tile (few, if any) take theirs together, one per lane and trip, whichever of the lane's leaves it is.
     const unsigned long long own = (unsigned long long)(j + 1) << 32;
     uint32_t pending = 0;
     if (w0) { if ((w0 >> 32 << 32) == own) vs.x = vm.x = q_j; else pending |= 1u; }
@@ -1544,6 +1544,72 @@ __device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t 
     const uint32_t off = tile * kBlockNodes + 4 * lane;  // this lane's first leaf
     if (active && dirty_out && (off & ((1u << g) - 1)) == 0) dirty_out[(off >> g) >> g_next] = a.epoch;
     tile_parents(a, g, first, lane, active, vs, vm);
+}
+
+// One wave per entry. The loads are kept apart from what they do not depend on: the entry, the first entries
+// of the scan and then the tile are requested before anything is computed.
+__device__ __forceinline__ void entry_tile(const UpdateArgs& a, int g, uint32_t j, uint32_t lane, unsigned long long* win,
+                                           uint32_t* __restrict__ dirty_out, int g_next) {
+    int64_t idx[kScanPer];
+    float pr[kScanPer];
+    const int64_t idx_j = a.indices[j];
+    const float p_j = a.priorities[j];
+    scan_request(a, lane, idx, pr);
+    clear_bids(win, lane);
+    if (!entry_valid(a, idx_j, p_j, lane, true)) return;  // wave-uniform: an entry that is skipped
+    const uint32_t tile = (uint32_t)((uint64_t)idx_j / kBlockNodes);
+    const uint32_t first = (1u << a.depth) + tile * kBlockNodes;
+    const float4 vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * lane);
+    const float4 vm = *reinterpret_cast<const float4*>(a.mn + first + 4 * lane);
+    // The entry's p^alpha, folded into the running max as k_update_stamp would. The power is taken here, inlined,
+    // while the tile and the scan's entries are on their way (a call would wait for every load in flight first):
+    // it is nearly always the value this wave's own leaf gets, and it costs as much as the tile's trip to memory.
+    const float q_j = powf_det(p_j, a.alpha);
+    if (lane == 0 && q_j > 0.0f) raise_max(a.maxp, q_j);
+    __builtin_amdgcn_wave_barrier();
+    scan_bids(a, tile, lane, win, idx, pr);
+    __threadfence_block();  // LDS operations of a wave complete in order; this also stops the compiler
+    __builtin_amdgcn_wave_barrier();
+    entry_finish(a, g, j, tile, lane, win, vs, vm, q_j, dirty_out, g_next);
+}
+
+// Calls of more entries than this give each entry two waves (entry_pair): the scan of a short call is too short
+// to be worth a second wave and a barrier (64 entries: no gain on the call, 0.5 us lost in a loop of calls).
+constexpr int64_t kPairedAbove = 128;
+
+// Two waves per entry (`role` 0 and 1, in one workgroup, `win` shared by the two): the power - some 110
+// dependent double-precision operations - and the election are each a wave's worth of instructions in a row;
+// side by side they take the time of the longer one. Every wave of the workgroup reaches the one barrier.
+__device__ __forceinline__ void entry_pair(const UpdateArgs& a, int g, uint32_t j, uint32_t role, uint32_t lane,
+                                           unsigned long long* win, uint32_t* __restrict__ dirty_out, int g_next) {
+    const bool have = (int64_t)j < a.n;  // wave-uniform
+    const int64_t idx_j = have ? a.indices[j] : -1;
+    const float p_j = have ? a.priorities[j] : -1.0f;
+    if (role == 1) {
+        // the election
+        int64_t idx[kScanPer];
+        float pr[kScanPer];
+        if (have) scan_request(a, lane, idx, pr);
+        clear_bids(win, lane);
+        if (have && entry_valid(a, idx_j, p_j, lane, false))
+            scan_bids(a, (uint32_t)((uint64_t)idx_j / kBlockNodes), lane, win, idx, pr);
+        lds_barrier();
+        return;
+    }
+    // the tile and the power
+    const bool valid = have && entry_valid(a, idx_j, p_j, lane, true);
+    const uint32_t tile = valid ? (uint32_t)((uint64_t)idx_j / kBlockNodes) : 0u;
+    const uint32_t first = (1u << a.depth) + tile * kBlockNodes;
+    float4 vs = make_float4(0.f, 0.f, 0.f, 0.f), vm = vs;
+    float q_j = 0.0f;
+    if (valid) {
+        vs = *reinterpret_cast<const float4*>(a.sum + first + 4 * lane);
+        vm = *reinterpret_cast<const float4*>(a.mn + first + 4 * lane);
+        q_j = powf_det(p_j, a.alpha);
+        if (lane == 0 && q_j > 0.0f) raise_max(a.maxp, q_j);
+    }
+    lds_barrier();
+    if (valid) entry_finish(a, g, j, tile, lane, win, vs, vm, q_j, dirty_out, g_next);
 }
 
 // Rebuilds everything above depth `top` (<= 16) with one workgroup: first up to 8 levels over
@@ -1604,10 +1670,17 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
         // falls into, with every entry of the call that falls into it; entries sharing a tile make
         // their waves write the same values to the same nodes. (4096 tiles scanned for 512 entries
         // cost three times as much as the rebuild itself.)
+        uint32_t* const dirty_next = last_round ? nullptr : a.dirty[round + 1];
+        const int g_next = last_round ? 0 : a.g[round + 1];
+        if (a.n > kPairedAbove) {
+            // two waves per entry (see entry_pair; the launch brings a workgroup per two entries)
+            const uint32_t pair = threadIdx.x >> 7, role = (threadIdx.x >> 6) & 1u;
+            entry_pair(a, g, blockIdx.x * (kWG / 128) + pair, role, lane, s_win[pair], dirty_next, g_next);
+            return;
+        }
         const uint32_t j = tile;  // tile_base is 0 here
         if ((int64_t)j >= a.n) return;
-        entry_tile(a, g, j, lane, s_win[threadIdx.x >> 6], last_round ? nullptr : a.dirty[round + 1],
-                   last_round ? 0 : a.g[round + 1]);
+        entry_tile(a, g, j, lane, s_win[threadIdx.x >> 6], dirty_next, g_next);
         return;
     }
     if (round == 0 && !a.indices && a.first_slot < 0) {
@@ -1729,10 +1802,7 @@ __global__ __launch_bounds__(kWG) void k_discounted_return(const float* __restri
 // One barrier per stage; no wave waits for a load it has just issued. The memory system so sees
 // loads and stores all the time, instead of a load phase, a phase without traffic and a store
 // phase per chunk. The arithmetic and its order are those of k_discounted_return.
-// A workgroup barrier for data handed over in LDS only: it waits for the wave's LDS operations, not for
-// its global loads and stores, which __syncthreads() would also wait for - here those are the next
-// chunk's requests and the last chunk's results, meant to stay in flight across the barrier.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// (lds_barrier: here the next chunk's requests and the last chunk's results stay in flight across it.)
 
 constexpr int kDrChunk = 128;
 constexpr int kDrCols = 64;
