@@ -899,6 +899,49 @@ def test_reference_scenario(mrb):
     assert h.dtype == torch.int64 and tuple(h.shape) == (1,)
 
 
+@pytest.mark.parametrize("cap", [10_000, 300_000, 5_000_000])
+@pytest.mark.parametrize("n", [40, 300, 700, 2000])
+def test_updates_with_invalid_entries_among_many(mrb, orc, cap, n):
+    """Invalid entries (index outside the ring; negative, NaN or infinite priority) inside calls of 40 .. 2000
+    entries - one wave per entry, two waves per entry, the stamp pass and, on the 23-level tree, the
+    entry-driven lowest round - are skipped and flagged while every valid entry lands as if the invalid ones
+    were not there: also where the LAST entry aimed at a leaf is the invalid one (the valid one before it
+    wins) and where an invalid entry shares its tile with valid ones."""
+    rng = np.random.default_rng(7000 + n + cap % 97)
+    shapes, dtypes = [(1,)], [np.int32]
+    g = mrb.PER(0.6, cap, 16, shapes, torch_types(dtypes), seed0=5)
+    c = orc.OraclePER(0.6, cap, shapes, dtypes, seed=5)
+    for start in range(0, cap, 1 << 18):
+        m = min(1 << 18, cap - start)
+        rows = [np.zeros((m, 1), np.int32)]
+        g.insert(*to_dev(rows))
+        c.push(rows, m)
+    for rep in range(3):
+        idx = rng.integers(0, cap, n)
+        idx[n // 2:] = np.minimum(idx[n // 2] // 256 * 256 + rng.integers(0, 256, n - n // 2), cap - 1)  # one crowded tile
+        pr = (rng.pareto(1.5, n) + 1e-6).astype(np.float32)
+        bad_idx = rng.choice(n, max(2, n // 10), replace=False)
+        idx[bad_idx[0::2]] = cap + rng.integers(0, 1000, len(bad_idx[0::2]))
+        idx[bad_idx[1::2]] = -1 - rng.integers(0, 1000, len(bad_idx[1::2]))
+        bad_pr = rng.choice(n, max(3, n // 10), replace=False)
+        pr[bad_pr] = np.resize(np.array([-1.0, np.nan, np.inf], np.float32), len(bad_pr))
+        # a leaf whose last entry is invalid: the valid entry before it must win
+        idx[n - 1] = idx[1] = int(rng.integers(0, cap))
+        pr[1], pr[n - 1] = 3.25, np.nan
+        ok = (idx >= 0) & (idx < cap) & np.isfinite(pr) & (pr >= 0)
+        assert ok[1] and not ok[n - 1] and ok.sum() < n
+        g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda())
+        c.update(idx[ok], pr[ok])
+        flags = C.c_uint32(0)
+        assert mrb.lib.lib().mrb_per_check(g._h, C.byref(flags), None) == 0
+        assert flags.value & mrb.lib.DERR_INDEX and flags.value & mrb.lib.DERR_PRIORITY, flags.value
+        assert_tree_equal(g, c, "cap %d n %d rep %d" % (cap, n, rep))
+        assert np.float32(g.max_priority) == np.float32(c.max_priority)
+        u = rng.random(16).astype(np.float32)
+        assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(16, 0.5, u), "after rep %d" % rep)
+    g.destroy()
+
+
 def test_per_error_paths(mrb):
     L = mrb.lib.lib()
     assert L.mrb_backend() == 1
