@@ -565,6 +565,12 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
             a.g[r] = b->s_g[r];
         }
     }
+    // At most 64 entries: one wave walks the entries' paths, leaves to root, in one launch (k_tree_paths).
+    if (!sparse && b->fused && n <= kPathEntries && b->depth <= kPathMaxDepth) {
+        hipLaunchKernelGGL(k_tree_paths, dim3(1), dim3(64), 0, s, a);
+        LAUNCH_CHECK("k_tree_paths");
+        return MRB_OK;
+    }
     // A small call on a tree of at least four leaves needs no stamp pass: the leaf-level waves scan the
     // entries themselves (one launch less).
     if (!sparse && n <= kElectMax && b->depth >= 2) {

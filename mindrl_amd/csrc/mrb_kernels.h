@@ -1750,6 +1750,105 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
 }
 
 // ---------------------------------------------------------------------------
+// update_priorities of at most 64 entries in ONE launch of ONE wave, along the entries' paths instead of by
+// tiles: an entry changes its leaf and the `depth` nodes above it, 15 nodes of a 14-level tree where its tile
+// has 511, so a single wave has time for all of it and no second launch is needed for the top.
+//   1. a lane per entry; the valid ones are sorted by (leaf, position in the call) with a bitonic network. Of
+//      the entries aimed at one leaf the last lane of the run - the latest entry - stays active.
+//   2. every active lane requests the siblings of the nodes on its path (their addresses follow from the
+//      leaf), then takes its power while they are on their way.
+//   3. level by level, from the leaves up: the parent is left + right, where the other child is the lane's
+//      sibling as memory holds it unless another entry of the call has changed it - then it is the value
+//      that entry's lane carries, and because the active lanes stay sorted by node it can only be the next
+//      active lane (for a left child) or the one before (for a right child). Of two lanes that meet in a
+//      parent the left child's goes on. Every node is the single rounded sum / min of its two final
+//      children, as everywhere.
+// Keys are 32 bits: leaf * 64 + lane, so the tree has at most 2^25 leaves here.
+// ---------------------------------------------------------------------------
+constexpr int kPathEntries = 64;
+constexpr int kPathMaxDepth = 25;
+
+__device__ __forceinline__ uint32_t bitonic_sort_wave(uint32_t key, uint32_t lane) {
+#pragma unroll
+    for (uint32_t k = 2; k <= 64; k <<= 1) {
+#pragma unroll
+        for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+            const uint32_t other = (uint32_t)__shfl_xor((int)key, (int)j);
+            const bool take_min = ((lane & j) == 0) == ((lane & k) == 0);
+            key = take_min ? (key < other ? key : other) : (key > other ? key : other);
+        }
+    }
+    return key;
+}
+
+__global__ __launch_bounds__(64) void k_tree_paths(UpdateArgs a) {
+    const uint32_t lane = threadIdx.x;
+    // the entries: flags for the invalid ones, keys for the valid ones
+    int64_t idx = -1;
+    float p = -1.0f;
+    if ((int64_t)lane < a.n) {
+        idx = a.indices[lane];
+        p = a.priorities[lane];
+    }
+    const bool have = (int64_t)lane < a.n;
+    const bool idx_ok = idx >= 0 && idx < a.capacity, p_ok = valid_priority(p);
+    if (__any(have && !idx_ok) && lane == 0) atomicOr(a.err, MRB_DERR_INDEX);
+    if (__any(have && !p_ok) && lane == 0) atomicOr(a.err, MRB_DERR_PRIORITY);
+    const bool valid = have && idx_ok && p_ok;
+    const uint32_t key = bitonic_sort_wave(valid ? ((uint32_t)idx << 6) | lane : 0xffffffffu, lane);
+    // this lane's entry from here on: the one the sort put here
+    const bool mine = key != 0xffffffffu;
+    const uint32_t leaf = key >> 6, pos = key & 63u;
+    const uint32_t next_key = (uint32_t)__shfl_down((int)key, 1);
+    bool act = mine && (lane == 63 || (next_key >> 6) != leaf || next_key == 0xffffffffu);  // the last entry aimed at the leaf
+    uint32_t v = (uint32_t)a.leaves + leaf;  // heap index of the node this lane carries
+    // siblings along the path, as memory holds them (level L's in [L - 1])
+    float sib_s[kPathMaxDepth], sib_m[kPathMaxDepth];
+#pragma unroll
+    for (int L = kPathMaxDepth; L >= 1; --L) {
+        sib_s[L - 1] = 0.0f;
+        sib_m[L - 1] = 0.0f;
+        if (L <= a.depth && act) {
+            const uint32_t node = (v >> (a.depth - L)) ^ 1u;
+            sib_s[L - 1] = a.sum[node];
+            sib_m[L - 1] = a.mn[node];
+        }
+    }
+    // the powers (every valid entry's counts for the running max, also one that loses its leaf)
+    const float p_here = __shfl(p, (int)pos);
+    const float q = mine ? powf_det(p_here, a.alpha) : 0.0f;
+    const float qmax = wave_max(q);
+    if (lane == 0 && qmax > 0.0f) raise_max(a.maxp, qmax);
+    float cs = q, cm = q;
+    if (act) {
+        a.sum[v] = cs;
+        a.mn[v] = cm;
+    }
+#pragma unroll
+    for (int L = kPathMaxDepth; L >= 1; --L) {
+        if (L <= a.depth) {  // wave-uniform
+            const unsigned long long lanes = __ballot(act);
+            const bool left = (v & 1u) == 0;
+            const unsigned long long above = lanes & ~((2ull << lane) - 1ull), below = lanes & ((1ull << lane) - 1ull);
+            const int nb = left ? (above ? __ffsll((long long)above) - 1 : -1) : (below ? 63 - __clzll((long long)below) : -1);
+            const int src = nb < 0 ? (int)lane : nb;
+            const uint32_t nv = (uint32_t)__shfl((int)v, src);
+            const float ns = __shfl(cs, src), nm = __shfl(cm, src);
+            const bool met = act && nb >= 0 && nv == (v ^ 1u);  // the other child is another entry's node
+            const float os = met ? ns : sib_s[L - 1], om = met ? nm : sib_m[L - 1];
+            cs = left ? cs + os : os + cs;
+            cm = left ? fminf(cm, om) : fminf(om, cm);
+            v >>= 1;
+            if (met && !left) act = false;  // the left child's lane carries the parent
+            if (act) {
+                a.sum[v] = cs;
+                a.mn[v] = cm;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Discounted return (mindspore_rl/utils/discounted_return.py:84-92): one thread per
 // (batch, inner) column walks the time axis backwards; neighbouring threads hold
 // neighbouring columns, so every step's loads and stores are coalesced. The loads do
