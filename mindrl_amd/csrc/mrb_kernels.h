@@ -1768,16 +1768,51 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
 constexpr int kPathEntries = 64;
 constexpr int kPathMaxDepth = 25;
 
-__device__ __forceinline__ uint32_t bitonic_sort_wave(uint32_t key, uint32_t lane) {
-#pragma unroll
-    for (uint32_t k = 2; k <= 64; k <<= 1) {
-#pragma unroll
-        for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-            const uint32_t other = (uint32_t)__shfl_xor((int)key, (int)j);
-            const bool take_min = ((lane & j) == 0) == ((lane & k) == 0);
-            key = take_min ? (key < other ? key : other) : (key > other ? key : other);
-        }
+// The key lane ^ J holds: inside a row of 16 lanes through DPP (quad permutations, row rotations), across rows
+// through the LDS crossbar.
+template <uint32_t J>
+__device__ __forceinline__ uint32_t xor_peer(uint32_t key, uint32_t lane) {
+    if (J == 1) return (uint32_t)__builtin_amdgcn_mov_dpp((int)key, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+    if (J == 2) return (uint32_t)__builtin_amdgcn_mov_dpp((int)key, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    if (J == 8) return (uint32_t)__builtin_amdgcn_mov_dpp((int)key, 0x128, 0xF, 0xF, true);  // row_ror:8
+    if (J == 4) {
+        const uint32_t up = (uint32_t)__builtin_amdgcn_mov_dpp((int)key, 0x12C, 0xF, 0xF, true);    // row_ror:12 = lane + 4
+        const uint32_t down = (uint32_t)__builtin_amdgcn_mov_dpp((int)key, 0x124, 0xF, 0xF, true);  // row_ror:4 = lane - 4
+        return (lane & 4u) ? down : up;
     }
+    return (uint32_t)__shfl_xor((int)key, (int)J);
+}
+
+template <uint32_t K, uint32_t J>
+__device__ __forceinline__ uint32_t sort_step(uint32_t key, uint32_t lane) {
+    const uint32_t other = xor_peer<J>(key, lane);
+    const bool take_min = ((lane & J) == 0) == ((lane & K) == 0);
+    return take_min ? (key < other ? key : other) : (key > other ? key : other);
+}
+
+// Ascending bitonic sort of one key per lane over the wave.
+__device__ __forceinline__ uint32_t bitonic_sort_wave(uint32_t key, uint32_t lane) {
+    key = sort_step<2, 1>(key, lane);
+    key = sort_step<4, 2>(key, lane);
+    key = sort_step<4, 1>(key, lane);
+    key = sort_step<8, 4>(key, lane);
+    key = sort_step<8, 2>(key, lane);
+    key = sort_step<8, 1>(key, lane);
+    key = sort_step<16, 8>(key, lane);
+    key = sort_step<16, 4>(key, lane);
+    key = sort_step<16, 2>(key, lane);
+    key = sort_step<16, 1>(key, lane);
+    key = sort_step<32, 16>(key, lane);
+    key = sort_step<32, 8>(key, lane);
+    key = sort_step<32, 4>(key, lane);
+    key = sort_step<32, 2>(key, lane);
+    key = sort_step<32, 1>(key, lane);
+    key = sort_step<64, 32>(key, lane);
+    key = sort_step<64, 16>(key, lane);
+    key = sort_step<64, 8>(key, lane);
+    key = sort_step<64, 4>(key, lane);
+    key = sort_step<64, 2>(key, lane);
+    key = sort_step<64, 1>(key, lane);
     return key;
 }
 
