@@ -571,6 +571,14 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
         LAUNCH_CHECK("k_tree_paths");
         return MRB_OK;
     }
+    // A few hundred entries on a small tree: one workgroup, a thread per entry, walks the paths in one launch
+    // (k_tree_wg; on deeper trees or with more entries one compute unit's memory traffic costs more than a launch).
+    if (!sparse && b->fused && n <= kWgBestEntries && b->depth >= 2 && b->depth <= kWgMaxDepth) {
+        const uint32_t threads = n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
+        hipLaunchKernelGGL(k_tree_wg, dim3(1), dim3(threads), 0, s, a);
+        LAUNCH_CHECK("k_tree_wg");
+        return MRB_OK;
+    }
     // A small call on a tree of at least four leaves needs no stamp pass: the leaf-level waves scan the
     // entries themselves (one launch less).
     if (!sparse && n <= kElectMax && b->depth >= 2) {

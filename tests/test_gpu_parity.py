@@ -942,6 +942,59 @@ def test_updates_with_invalid_entries_among_many(mrb, orc, cap, n):
     g.destroy()
 
 
+@pytest.mark.parametrize("cap", [4, 37, 1000, 2048, 4096, 5000, 10_000, 16_384])
+def test_updates_of_a_few_hundred_entries_on_small_trees(mrb, orc, cap):
+    """update_priorities of 65 .. 384 entries on trees of 2 .. 14 levels (one launch of one workgroup that walks
+    the entries' paths: the tree's top in LDS, the nodes below it in LDS hash tables, two levels per step): random
+    indices, consecutive slots (neighbouring paths meet at every level), a handful of leaves hit by every entry
+    (the latest entry wins each) and invalid entries among valid ones - trees, running max and flags as the
+    oracle's after every call; with the one-launch option off the same calls give the same bits."""
+    rng = np.random.default_rng(8100 + cap)
+    shapes, dtypes = [(2,)], [np.float32]
+    g = mrb.PER(0.7, cap, 8, shapes, torch_types(dtypes), seed0=3)
+    g2 = mrb.PER(0.7, cap, 8, shapes, torch_types(dtypes), seed0=3)
+    g2.set_option("fused_rebuild", 0)
+    c = orc.OraclePER(0.7, cap, shapes, dtypes, seed=3)
+    fill = cap - cap // 5  # some leaves stay unfilled: their minimum is FLT_MAX until an update reaches them
+    rows = [rng.normal(size=(fill, 2)).astype(np.float32)]
+    g.insert(*to_dev(rows))
+    g2.insert(*to_dev(rows))
+    c.push(rows, fill)
+    for n in (65, 100, 128, 255, 256, 321, 384):
+        for mode in ("random", "consecutive", "crowded", "invalid"):
+            if mode == "random":
+                idx = rng.integers(0, cap, n)
+            elif mode == "consecutive":
+                idx = (rng.integers(0, cap) + np.arange(n)) % cap
+            elif mode == "crowded":
+                idx = rng.integers(0, min(cap, 7), n) + rng.integers(0, max(1, cap - 7))
+            else:
+                idx = rng.integers(0, cap, n)
+                idx[rng.choice(n, 5, replace=False)] = cap + rng.integers(0, 100, 5)
+                idx[rng.choice(n, 3, replace=False)] = -1 - rng.integers(0, 100, 3)
+            pr = (rng.pareto(1.5, n) + 1e-6).astype(np.float32)
+            if mode == "invalid":
+                pr[rng.choice(n, 6, replace=False)] = np.array([-1.0, np.nan, np.inf, -np.inf, -0.5, np.nan], np.float32)
+                idx[n - 1] = idx[2] = int(rng.integers(0, cap))  # the last entry aimed at a leaf is invalid:
+                pr[2], pr[n - 1] = 1.75, np.nan                   # the valid one before it wins
+            ok = (idx >= 0) & (idx < cap) & np.isfinite(pr) & (pr >= 0)
+            for buf in (g, g2):
+                buf.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda())
+            c.update(idx[ok], pr[ok])
+            what = "cap %d n %d %s" % (cap, n, mode)
+            for buf in (g, g2):
+                flags = C.c_uint32(0)
+                assert mrb.lib.lib().mrb_per_check(buf._h, C.byref(flags), None) == 0
+                want = (mrb.lib.DERR_INDEX | mrb.lib.DERR_PRIORITY) if mode == "invalid" else 0
+                assert flags.value == want, (what, flags.value)
+                assert_tree_equal(buf, c, what)
+                assert bits(np.float32(buf.max_priority)) == bits(np.float32(c.max_priority)), what
+    u = rng.random(8).astype(np.float32)
+    assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(8, 0.5, u), "cap %d" % cap)
+    g.destroy()
+    g2.destroy()
+
+
 def test_per_error_paths(mrb):
     L = mrb.lib.lib()
     assert L.mrb_backend() == 1
