@@ -1275,6 +1275,46 @@ def test_sparse_updates_on_very_large_trees(mrb, orc, cap):
     g.destroy()
 
 
+def test_tree_of_27_levels(mrb, orc):
+    """Capacity 2^26 + 11 (a tree of 27 levels, 2^27 leaves: three node groups of nine levels per descent; deeper
+    than the path kernels take, so small updates elect among themselves in the tile kernels): the full ring
+    pushed with priorities, updates of 50, 1000 (10 % duplicates) and 200,000 entries (the entry-driven lowest
+    round), a push that wraps the ring, samples through the wide-row kernel and through the LDS-top kernel -
+    indices, rows, weights, both trees and the running max as the oracle's."""
+    cap = (1 << 26) + 11
+    shapes, dtypes = [(1,)], [np.uint8]
+    rng = np.random.default_rng(2627)
+    g, c = make_pair(mrb, orc, 0.5, cap, 256, seed=3, shapes=shapes, dtypes=dtypes)
+    rows = [(np.arange(cap, dtype=np.int64) % 251).astype(np.uint8)[:, None]]
+    pr = rng.lognormal(0, 1, cap).astype(np.float32)
+    g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda())
+    c.push(rows, cap)
+    c.update(np.arange(cap), pr)
+    del pr
+    for n in (50, 1000, 200_000):
+        idx = rng.integers(0, cap, n)
+        if n >= 1000:
+            idx[rng.integers(0, n, n // 10)] = idx[rng.integers(0, n, n // 10)]
+        up = rng.pareto(1.5, n).astype(np.float32) + np.float32(1e-6)
+        g.update_priorities(torch.from_numpy(idx).cuda(), torch.from_numpy(up).cuda())
+        c.update(idx, up)
+        u = rng.random(256).astype(np.float32)
+        assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(256, 0.5, u), "n %d" % n)
+    more = [np.full((300, 1), 7, np.uint8)]
+    g.insert(*to_dev(more))
+    c.push(more, 300)
+    assert_tree_equal(g, c, "27 levels")
+    assert np.float32(g.max_priority) == np.float32(c.max_priority)
+    g.check()
+    # the same strata through the LDS-top kernel (9 levels staged, the 18 below them walked five per load)
+    g.set_option("sample_path", 2)
+    for beta in (0.4, 1.0):
+        u = rng.random(256).astype(np.float32)
+        assert_sample_equal(g.sample(beta, uniforms=torch.from_numpy(u).cuda()), c.sample(256, beta, u), "LDS-top kernel")
+    g.check()
+    g.destroy()
+
+
 @pytest.mark.parametrize("cap", [1 << 17, 1_000_000])
 def test_config3_atari_shape_properties(mrb, orc, cap):
     """Config 3's rows (u8[84,84,4] + next_idx i64 + action i32 + reward f32 + done bool =
