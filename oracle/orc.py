@@ -186,7 +186,7 @@ class OracleUniform(_Rows):
         lib().orc_urb_seed(self.h, seed)
 
     def __del__(self):
-        if getattr(self, "h", None):
+        if getattr(self, "h", None) and lib is not None:  # at interpreter shutdown the module's names may be gone
             lib().orc_urb_destroy(self.h)
             self.h = None
 
@@ -257,7 +257,7 @@ class OracleReservoir(_Rows):
             raise ValueError("orc_res_create failed")
 
     def __del__(self):
-        if getattr(self, "h", None):
+        if getattr(self, "h", None) and lib is not None:  # at interpreter shutdown the module's names may be gone
             lib().orc_res_destroy(self.h)
             self.h = None
 
@@ -312,7 +312,7 @@ class OraclePER(_Rows):
             raise ValueError("orc_per_create failed")
 
     def __del__(self):
-        if getattr(self, "h", None):
+        if getattr(self, "h", None) and lib is not None:  # at interpreter shutdown the module's names may be gone
             lib().orc_per_destroy(self.h)
             self.h = None
 
