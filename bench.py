@@ -457,7 +457,20 @@ def per_extras(a, torch, r, algo_bytes):
             # sample, then gather at the slots that very sample returned: other rows every call
             extras["sample_plus_next_obs_us"] = timed(
                 lambda i: (r.sample(W + i % K), L.mrb_per_gather(h, nxt.data_ptr(), batch, gptr, sp))) * 1e6
-            del gfields
+            # the same in ONE launch: the sample plus the observation at each sampled row's next_idx
+            # (mrb_per_sample_next: 2 * 28,224 B more per row, the launch and the descent paid once)
+            nobs = torch.empty_like(r.fields[0])
+            def fused(i):
+                rc = L.mrb_per_sample_next(h, batch, float(r.betas[W + i % K]),
+                                           r.uniforms.data_ptr() + (W + i % K) * batch * 4, 1, 0, r.idx.data_ptr(),
+                                           r.wts.data_ptr(), r.fptr, nobs.data_ptr(), sp)
+                if rc:
+                    r._lib.check(rc)
+            us = timed(fused) * 1e6
+            extras["sample_with_next_obs_one_launch_us"] = us
+            extras["sample_with_next_obs_one_launch_frac_of_peak"] = (
+                (algo_bytes + batch * 2 * r.buf._layout.bytes[0]) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS)
+            del gfields, nobs
         # the same calls replayed from one captured HIP graph (a chain: every call ordered after the one before)
         n_g = min(K, 200)
         graph = torch.cuda.CUDAGraph()

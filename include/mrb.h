@@ -169,6 +169,16 @@ int mrb_per_sample(int64_t h, int64_t batch, float beta, const float *uniforms, 
  * update of the priorities (prefetching); one launch then amortises the launch and the tree descent. */
 int mrb_per_sample_many(int64_t h, int64_t nbatch, int64_t batch, float beta, const float *uniforms,
                         int64_t *out_indices, float *out_weights, void *const *out_fields, void *stream);
+/* mrb_per_sample and, in the same launch, field `row_field` of the row whose slot number each sampled row holds
+ * in its field `slot_field` (8 bytes: one int64 per row), written to out_next_rows ([batch, field_bytes[row_field]],
+ * 16-byte aligned): what mrb_per_sample followed by mrb_per_gather at out_fields[slot_field] would leave in that
+ * field's matrix. No counterpart among the reference's primitives: it serves transitions that keep the next
+ * observation as a slot number (frame-shared storage) - a learner needs both observations, and one launch pays
+ * the launch and the tree descent for both. row_field must be a field whose rows are multiples of 16 bytes.
+ * Slot numbers outside [0, size) are clamped and reported by mrb_per_check (MRB_DERR_INDEX). */
+int mrb_per_sample_next(int64_t h, int64_t batch, float beta, const float *uniforms, int slot_field, int row_field,
+                        int64_t *out_indices, float *out_weights, void *const *out_fields, void *out_next_rows,
+                        void *stream);
 /* Replaces PriorityReplayBufferUpdate (priority_replay_buffer.py:71-73,120):
  * leaf[indices[j]] = priorities[j]^alpha for j in order (last write wins on
  * duplicates), every ancestor of a touched leaf recomputed from its final

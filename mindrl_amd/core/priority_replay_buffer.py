@@ -118,6 +118,32 @@ class PriorityReplayBuffer:
         self._keep = u
         return (idx, w) + tuple(fields)
 
+    def sample_with_next(self, beta, slot_field, row_field, uniforms=None):
+        """sample(beta) plus, in the same launch, field `row_field` of the row whose slot number each sampled
+        row holds in its field `slot_field` (an int64[1] field): for transitions that store the next
+        observation as a slot number instead of a copy. Returns sample()'s tuple with one more tensor
+        [B, *shape_row_field] at the end - what `gather(transitions[slot_field])[row_field]` would give, without
+        the second launch and the second tree descent. Fresh output tensors on every call."""
+        n = self._sample_size
+        slot_field, row_field = int(slot_field), int(row_field)
+        if not 0 <= slot_field < len(self._layout) or not 0 <= row_field < len(self._layout):
+            raise ValueError("slot_field and row_field must name fields of the transition")
+        u = None
+        if uniforms is not None:
+            u = flat_on_device(uniforms, torch.float32, self._dev)
+            if u.numel() != n:
+                raise ValueError("uniforms must hold sample_size = %d values" % n)
+        idx = torch.empty(n, dtype=torch.int64, device=self._dev)
+        w = torch.empty(n, dtype=torch.float32, device=self._dev)
+        fields = self._layout.empty(n, self._dev)
+        nxt = torch.empty((n,) + tuple(self._layout.shapes[row_field]), dtype=self._layout.dtypes[row_field],
+                          device=self._dev)
+        _lib.check(_lib.lib().mrb_per_sample_next(self._h, n, float(beta), u.data_ptr() if u is not None else None,
+                                                  slot_field, row_field, idx.data_ptr(), w.data_ptr(),
+                                                  pointers(fields), nxt.data_ptr(), stream_ptr()))
+        self._keep = u
+        return (idx, w) + tuple(fields) + (nxt,)
+
     def sample_many(self, nbatch, beta, uniforms=None):
         """`nbatch` batches in one launch: what `nbatch` successive sample(beta) calls would return on an
         unchanged buffer, stacked: (indices int64[nbatch, B], weights f32[nbatch, B], *transitions

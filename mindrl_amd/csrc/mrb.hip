@@ -203,15 +203,61 @@ void launch_sample_wide_as(dim3 grid, const SampleArgs& a, const WidePlan& plan,
     else one ? launch_sample_wide<kInF, false, true>(grid, a, plan, s) : launch_sample_wide<kInF, false, false>(grid, a, plan, s);
 }
 
-int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, int64_t nbatch, hipStream_t s) {
+// A sample call's optional second layer: field `row_field` of the row whose slot number the sampled row holds
+// in its 8-byte field `slot_field` goes to `out` ([batch, row bytes]).
+struct NextRows {
+    int slot_field = -1, row_field = -1;
+    void* out = nullptr;
+};
+
+template <int kInF, bool kTen, bool kOneWide>
+void launch_sample_next(dim3 grid, const SampleArgs& a, const WidePlan& plan, const NextPlan& nx, hipStream_t s) {
+    const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
+    hipLaunchKernelGGL((k_per_sample_next<kInF, kTen, kOneWide>), grid, dim3(kWideWG), 0, s, a.sum, a.uniforms, a.depth,
+                       pack_groups(a.depth), (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, tail, plan, nx);
+}
+
+template <int kInF>
+void launch_sample_next_as(dim3 grid, const SampleArgs& a, const WidePlan& plan, const NextPlan& nx, hipStream_t s) {
+    const bool ten = a.depth > 0 && a.depth % kGroupMaxLevels == 0;
+    const bool one = plan.nwide == 1;
+    if (ten) one ? launch_sample_next<kInF, true, true>(grid, a, plan, nx, s) : launch_sample_next<kInF, true, false>(grid, a, plan, nx, s);
+    else one ? launch_sample_next<kInF, false, true>(grid, a, plan, nx, s) : launch_sample_next<kInF, false, false>(grid, a, plan, nx, s);
+}
+
+int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, int64_t nbatch, hipStream_t s,
+                const NextRows* next = nullptr) {
     WidePlan plan;
     dim3 grid;
     plan.nbatch = (uint32_t)nbatch;
-    switch (wide_plan(r, t, nbatch * a.batch, plan, grid)) {
-        case 0: return MRB_EINVAL;
-        case 2: launch_sample_wide_as<2>(grid, a, plan, s); break;
-        default: launch_sample_wide_as<8>(grid, a, plan, s); break;
+    const int inflight = wide_plan(r, t, nbatch * a.batch, plan, grid);
+    if (inflight == 0) return MRB_EINVAL;
+    if (next) {
+        // the second layer of workgroups: one wide field, split like a row of its own
+        NextPlan nx{};
+        const int f = next->row_field;
+        nx.slot_field = r.data[next->slot_field];
+        nx.plan.nwide = 1;
+        nx.plan.nbatch = 1;
+        nx.plan.f[0].src = r.data[f];
+        nx.plan.f[0].dst = static_cast<uint8_t*>(next->out);
+        nx.plan.f[0].rb = (uint32_t)r.bytes[f];
+        nx.plan.wide_items = r.units[f];
+        const uint32_t per_wg = (uint32_t)kMaxInFlight * kCopyThreads;
+        const uint32_t split = (nx.plan.wide_items + per_wg - 1) / per_wg;
+        nx.plan.split = (int)split;
+        nx.plan.share = (nx.plan.wide_items + split - 1) / split;
+        if (split > 65535u) return fail(MRB_EINVAL, "field %d is too wide for one launch", f);
+        if (split > grid.y) grid.y = split;
+        grid.z = 2;
+        const uint32_t per_thread = (nx.plan.share + kCopyThreads - 1) / kCopyThreads;
+        if (inflight == 2 && per_thread <= 2) launch_sample_next_as<2>(grid, a, plan, nx, s);
+        else launch_sample_next_as<8>(grid, a, plan, nx, s);
+        LAUNCH_CHECK("k_per_sample_next");
+        return MRB_OK;
     }
+    if (inflight == 2) launch_sample_wide_as<2>(grid, a, plan, s);
+    else launch_sample_wide_as<8>(grid, a, plan, s);
     LAUNCH_CHECK("k_per_sample_wide");
     return MRB_OK;
 }
@@ -1077,7 +1123,8 @@ int mrb_per_update_noalloc(int64_t h, const int64_t* indices, const float* prior
 // `nbatch` batches of `batch` stratified samples each, as nbatch successive mrb_per_sample calls on
 // an unchanged tree would draw them. Outputs hold nbatch * batch rows, batch after batch.
 static int per_sample_impl(Per* b, int64_t nbatch, int64_t batch, float beta, const float* uniforms,
-                           int64_t* out_indices, float* out_weights, void* const* out_fields, hipStream_t s) {
+                           int64_t* out_indices, float* out_weights, void* const* out_fields, hipStream_t s,
+                           const NextRows* next = nullptr) {
     if (batch <= 0 || batch > (1ll << 24)) return fail(MRB_EINVAL, "batch %lld outside [1, 2^24]", (long long)batch);
     if (nbatch <= 0 || nbatch > 4096 || nbatch * batch > (1ll << 24))
         return fail(MRB_EINVAL, "%lld batches of %lld rows exceed one call (at most 4096 batches, 2^24 rows)",
@@ -1120,7 +1167,10 @@ static int per_sample_impl(Per* b, int64_t nbatch, int64_t batch, float beta, co
     const int64_t max_bytes = widest_field(b->rows);
     int path = (int)b->sample_path;
     if (path == 0) path = (batch >= 8192 && max_bytes <= 256) ? 2 : 1;
-    if (path == 1) {
+    if (next) {
+        rc = sample_wide(b->rows, a, t, nbatch, s, next);  // always the wide-row kernel: the gathered field is wide
+        if (rc) return rc;
+    } else if (path == 1) {
         rc = sample_wide(b->rows, a, t, nbatch, s);
         if (rc) return rc;
     } else {
@@ -1161,6 +1211,22 @@ int mrb_per_sample_many(int64_t h, int64_t nbatch, int64_t batch, float beta, co
     GET_PER(b, h);
     return per_sample_impl(b.get(), nbatch, batch, beta, uniforms, out_indices, out_weights, out_fields,
                            static_cast<hipStream_t>(stream));
+}
+
+int mrb_per_sample_next(int64_t h, int64_t batch, float beta, const float* uniforms, int slot_field, int row_field,
+                        int64_t* out_indices, float* out_weights, void* const* out_fields, void* out_next_rows,
+                        void* stream) {
+    GET_PER(b, h);
+    const RowStore& r = b->rows;
+    if (slot_field < 0 || slot_field >= r.nfields || r.bytes[slot_field] != 8)
+        return fail(MRB_EINVAL, "slot_field %d must name a field of 8 bytes (one int64 slot number per row)", slot_field);
+    if (row_field < 0 || row_field >= r.nfields || r.vec_log2[row_field] != 4)
+        return fail(MRB_EINVAL, "row_field %d must name a field whose rows are multiples of 16 bytes", row_field);
+    if (!out_next_rows) return fail(MRB_EINVAL, "out_next_rows is NULL");
+    if (reinterpret_cast<uintptr_t>(out_next_rows) & 15u) return fail(MRB_EINVAL, "out_next_rows %p is not 16-byte aligned", out_next_rows);
+    const NextRows next{slot_field, row_field, out_next_rows};
+    return per_sample_impl(b.get(), 1, batch, beta, uniforms, out_indices, out_weights, out_fields,
+                           static_cast<hipStream_t>(stream), &next);
 }
 
 int mrb_per_gather(int64_t h, const int64_t* indices, int64_t n, void* const* dst_fields, void* stream) {

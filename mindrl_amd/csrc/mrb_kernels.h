@@ -549,16 +549,41 @@ struct CopyWork {
 // `groups` packs the descent plan: bits 0-3 the number of node groups, then 5 bits per group
 // with the levels it takes; bits 20-31 hold the number of batches in the launch minus one. kTen: every group takes 10 levels (trees of 10, 20 or 30 levels); the
 // walk is then compiled for that size, which shortens it by a third.
-template <int kInF, bool kTen, bool kOneWide>
-__global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __restrict__ sum, const float* __restrict__ uniforms,
-                                                             int depth, uint32_t groups, int batch, uint32_t capacity,
-                                                             uint64_t seed, uint64_t calls, SampleTail tail, WidePlan plan) {
+//
+// kNext (k_per_sample_next): the launch has a second layer of workgroups (blockIdx.z == 1) that gathers, for
+// every sampled row, ONE wide field at the slot the row itself names in an 8-byte field - the next observation
+// of a transition that stores a slot number instead of a copy (`nx`). Such a workgroup repeats the walk, reads
+// the slot number from the sampled row, and its copy waves copy that field's row; one launch then pays the
+// launch and the descent for twice the bytes.
+struct NextPlan {
+    const uint8_t* slot_field;  // storage of the 8-byte field that holds the slot number, [capacity, 8]
+    WidePlan plan;              // one wide field: its storage -> the caller's [batch, row_bytes] matrix
+};
+
+struct NoNext {};
+
+template <int kInF, bool kTen, bool kOneWide, bool kNext, typename Next>
+__device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, const float* __restrict__ uniforms,
+                                                 int depth, uint32_t groups, int batch, uint32_t capacity,
+                                                 uint64_t seed, uint64_t calls, const SampleTail& tail,
+                                                 const WidePlan& plan, const Next& nx) {
+    // the next-slot layer's plan and slot field (the row's own plan stands in where there is no such layer)
+    const WidePlan& plan2 = [&]() -> const WidePlan& {
+        if constexpr (kNext) return nx.plan;
+        else return plan;
+    }();
+    const uint8_t* const slot_field = [&]() -> const uint8_t* {
+        if constexpr (kNext) return nx.slot_field;
+        else return nullptr;
+    }();
     __shared__ int64_t s_idx;
     __shared__ float s_picked, s_total, s_pmin;
     __shared__ float s_tot[4];
     __shared__ SampleTail s_tail;
     const int64_t k = blockIdx.x;      // output row
     const uint32_t part = blockIdx.y;  // which of the row's workgroups
+    const bool next_layer = kNext && blockIdx.z == 1;  // this workgroup gathers the row's next-slot field
+    if (kNext && part >= (uint32_t)(next_layer ? plan2.split : plan.split)) return;  // the layers' splits may differ
     // Several batches in one launch (groups >> 20 = their number - 1): output row k is stratum `stratum`
     // of batch `nth`; each batch is stratified on its own and takes the generator's next call counter.
     uint32_t stratum = (uint32_t)k, nth = 0;
@@ -671,11 +696,12 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
     // ---- copy waves, while the walker walks
     CopyWork<kInF, kOneWide> work;
     NarrowWork nw;
-    const bool narrow = wave == 1 && part == 0 && plan.narrow_items;
+    const bool narrow = wave == 1 && part == 0 && plan.narrow_items && !next_layer;
     if (!walker) {
         if (narrow) nw.prepare(plan, k, lane);
-        work.prepare(plan, k, part, ctid);
-        if (part == 0 && wave == 2) {
+        if (next_layer) work.prepare(plan2, k, part, ctid);
+        else work.prepare(plan, k, part, ctid);
+        if ((part == 0 || next_layer) && wave == 2) {
             // what the walker needs after the barrier (member by member: a whole-struct copy would go
             // through private memory)
             if (lane == 0) {
@@ -693,6 +719,24 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
     __syncthreads();
     MRB_TS(ts_past_barrier);
     const int64_t idx = s_idx;
+    if (kNext && next_layer) {
+        // the slot the sampled row names (outside [0, size): clamped and flagged, as mrb_per_gather does)
+        __shared__ int64_t s_next;
+        if (walker && lane == 0) {
+            int64_t size = s_tail.size;
+            if (size < 0) size = counters_behind(s_tail.err)[kCntSize];
+            const int64_t row = idx < (int64_t)capacity ? idx : (int64_t)capacity - 1;
+            int64_t to = *reinterpret_cast<const int64_t*>(slot_field + (uint64_t)row * 8);
+            if (to < 0 || to >= size) {
+                if (part == 0) atomicOr(s_tail.err, MRB_DERR_INDEX);
+                to = to < 0 ? 0 : (size > 0 ? size - 1 : 0);
+            }
+            s_next = to;
+        }
+        __syncthreads();
+        if (!walker) work.run((uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)s_next), plan2, false, nw, lane);
+        return;
+    }
     if (!walker) {
         // the descent can end on an unfilled leaf past the last row (flagged by the walker)
         const uint32_t slot = (uint32_t)(idx < (int64_t)capacity ? idx : (int64_t)capacity - 1);
@@ -732,6 +776,22 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
     MRB_TS_OUT(3, ts_at_barrier);
     MRB_TS_OUT(5, ts_past_barrier);
     MRB_TS_OUT(8, ts_wend);
+}
+
+template <int kInF, bool kTen, bool kOneWide>
+__global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __restrict__ sum, const float* __restrict__ uniforms,
+                                                             int depth, uint32_t groups, int batch, uint32_t capacity,
+                                                             uint64_t seed, uint64_t calls, SampleTail tail, WidePlan plan) {
+    sample_wide_body<kInF, kTen, kOneWide, false>(sum, uniforms, depth, groups, batch, capacity, seed, calls, tail, plan, NoNext{});
+}
+
+// Sample plus, in the same launch, one wide field gathered at the slot each sampled row names (see kNext above).
+template <int kInF, bool kTen, bool kOneWide>
+__global__ __launch_bounds__(kWideWG) void k_per_sample_next(const float* __restrict__ sum, const float* __restrict__ uniforms,
+                                                             int depth, uint32_t groups, int batch, uint32_t capacity,
+                                                             uint64_t seed, uint64_t calls, SampleTail tail, WidePlan plan,
+                                                             NextPlan nx) {
+    sample_wide_body<kInF, kTen, kOneWide, true>(sum, uniforms, depth, groups, batch, capacity, seed, calls, tail, plan, nx);
 }
 
 // Gather of wide rows: io_f[k] = store_f[slot_k], slot_k being `fixed_slot` (mode kFromFixedSlot, a

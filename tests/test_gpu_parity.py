@@ -1275,6 +1275,69 @@ def test_sparse_updates_on_very_large_trees(mrb, orc, cap):
     g.destroy()
 
 
+@pytest.mark.parametrize("cap,obs_shape,extra", [(5000, (84, 84, 4), False), (70_000, (36, 1000), True),
+                                                 (2_500_000, (1024,), False), (300, (16,), True)])
+def test_sample_with_next_equals_sample_then_gather(mrb, orc, cap, obs_shape, extra):
+    """mrb_per_sample_next - the sample and, in the same launch, the observation at the slot each sampled row
+    names - against the oracle's sample plus numpy's take of the observations, and against mrb_per_sample followed by mrb_per_gather:
+    a 28,224-byte image row, a 36,000-byte row (two workgroups per row in the second layer), a 22-level tree
+    (the copy waves share the descent's top group) and 16-byte rows; with a second wide field in the row
+    (`extra`) the general addressing path runs. Slot numbers outside [0, size) are clamped and flagged."""
+    rng = np.random.default_rng(4400 + cap % 1000)
+    shapes = [obs_shape, (1,), (1,)] + ([(8,)] if extra else [])
+    dtypes = [np.uint8, np.int64, np.float32] + ([np.float32] if extra else [])
+    batch = 96
+    g = mrb.PER(0.6, cap, batch, shapes, torch_types(dtypes), seed0=9)
+    c = orc.OraclePER(0.6, cap, shapes, dtypes, seed=9)
+    fill = cap - cap // 7
+    mirror = np.zeros((fill + 4,) + obs_shape, np.uint8)  # the observation field by slot (the ring does not wrap here)
+    for start in range(0, fill, 50_000):
+        m = min(50_000, fill - start)
+        rows = [rng.integers(0, 256, (m,) + obs_shape, dtype=np.uint8),
+                rng.integers(0, fill, (m, 1)).astype(np.int64), rng.normal(size=(m, 1)).astype(np.float32)]
+        if extra:
+            rows.append(rng.normal(size=(m, 8)).astype(np.float32))
+        pr = rng.lognormal(0, 1, m).astype(np.float32)
+        g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda())
+        c.push(rows, m, pr)
+        mirror[start:start + m] = rows[0]
+    for rep in range(3):
+        u = rng.random(batch).astype(np.float32)
+        ud = torch.from_numpy(u).cuda()
+        out = g.sample_with_next(0.5, 1, 0, uniforms=ud)
+        ci, cw, cf = c.sample(batch, 0.5, u)
+        assert_sample_equal(out[:-1], (ci, cw, cf), "sample part, rep %d" % rep)
+        want = np.take(mirror, cf[1].reshape(-1), axis=0)
+        assert np.array_equal(t2n(out[-1]), want), "next rows differ from numpy's take, rep %d" % rep
+        two = g.sample(0.5, uniforms=ud)
+        assert torch.equal(g.gather(two[3].reshape(-1))[0], out[-1])
+        g.check()
+    # slot numbers outside the stored rows: clamped like mrb_per_gather's, and flagged
+    bad = [rng.integers(0, 256, (4,) + obs_shape, dtype=np.uint8), np.array([[-5], [fill + 4], [cap + 9], [3]], np.int64),
+           np.zeros((4, 1), np.float32)] + ([np.zeros((4, 8), np.float32)] if extra else [])
+    huge = np.full(4, 1e9, np.float32)  # the four rows take nearly all of the mass
+    g.insert(*to_dev(bad), priorities=torch.from_numpy(huge).cuda())
+    c.push(bad, 4, huge)
+    mirror[fill:] = bad[0]
+    u = rng.random(batch).astype(np.float32)
+    out = g.sample_with_next(0.5, 1, 0, uniforms=torch.from_numpy(u).cuda())
+    ci, cw, cf = c.sample(batch, 0.5, u)
+    assert_sample_equal(out[:-1], (ci, cw, cf), "sample part with wild slot numbers")
+    slots = cf[1].reshape(-1)
+    assert ((slots < 0) | (slots >= fill + 4)).any()
+    want = np.take(mirror, np.clip(slots, 0, fill + 4 - 1), axis=0)
+    assert np.array_equal(t2n(out[-1]), want)
+    flags = C.c_uint32(0)
+    assert mrb.lib.lib().mrb_per_check(g._h, C.byref(flags), None) == 0
+    assert flags.value == mrb.lib.DERR_INDEX, flags.value
+    # argument checks: the slot field must be 8 bytes wide, the gathered field made of 16-byte granules
+    with pytest.raises(ValueError):
+        g.sample_with_next(0.5, 2, 0)
+    with pytest.raises(ValueError):
+        g.sample_with_next(0.5, 1, 2)
+    g.destroy()
+
+
 def test_tree_of_27_levels(mrb, orc):
     """Capacity 2^26 + 11 (a tree of 27 levels, 2^27 leaves: three node groups of nine levels per descent; deeper
     than the path kernels take, so small updates elect among themselves in the tile kernels): the full ring
