@@ -252,10 +252,14 @@ class PerRun:
         fill_per(self.buf, torch, self.capacity, self.shapes, self.np_dtypes, self.seed, lognormal=not self.loop_step)
         self.fill_s = time.perf_counter() - t0
         self.K, self.W = a.steps, a.warmup
-        n, batch = self.K + self.W, self.batch
+        # draws for the timed steps and, beyond them, for the untimed side figures (which take their own step
+        # counts, so that a short timed run does not make them noisy)
+        n, batch = max(self.K + self.W, 1200), self.batch
+        self.n_draws = n
         self.rng = np.random.default_rng(self.seed + 1)
         self.uniforms = torch.from_numpy(self.rng.random((n, batch)).astype(np.float32)).cuda()
-        self.betas = (np.linspace(0.4, 1.0, n) if a.workload == "c3" else np.full(n, 0.4)).astype(np.float32)
+        self.betas = np.resize((np.linspace(0.4, 1.0, self.K + self.W) if a.workload == "c3"
+                                else np.full(self.K + self.W, 0.4)).astype(np.float32), n)
         self.idx = torch.empty(batch, dtype=torch.int64, device="cuda")
         self.wts = torch.empty(batch, dtype=torch.float32, device="cuda")
         self.fields = self.buf._layout.empty(batch, self.buf._dev)
@@ -401,9 +405,10 @@ def bench_per(a):
 def per_extras(a, torch, r, algo_bytes):
     """Untimed side figures: the other operations of the config's step, the same sample steps replayed from
     a HIP graph, and issued round robin on several streams (independent calls, one output set per stream)."""
-    L, h, sp, K, W, batch = r.L, r.h, r.sp, r.K, r.W, r.batch
+    L, h, sp, W, batch = r.L, r.h, r.sp, r.W, r.batch
+    K = r.n_draws - W  # the side figures run over all the draws there are, whatever the timed run's step count
     extras = {}
-    n_it = max(20, min(300, K))
+    n_it = 300
 
     def timed(fn, n=n_it):
         for i in range(10):
