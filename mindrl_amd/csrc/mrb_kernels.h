@@ -1944,7 +1944,7 @@ __global__ __launch_bounds__(64) void k_tree_paths(UpdateArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// update_priorities of 65 .. 384 entries on a tree of at most 14 levels in ONE launch of ONE workgroup, a
+// update_priorities of at most 384 entries on a tree of at most 14 levels in ONE launch of ONE workgroup, a
 // thread per entry, again along the entries' paths: a call then costs one launch instead of a leaf round and
 // a top that wait for each other. What one wave settles among its lanes in k_tree_paths, the waves of a
 // workgroup settle through LDS:
@@ -1967,11 +1967,13 @@ __global__ __launch_bounds__(64) void k_tree_paths(UpdateArgs a) {
 // memory (sibling and cousins read, own node written, in both trees), and ONE compute unit moves about one
 // such cache line per nanosecond. Measured per call: 10,000 leaves, 128 / 256 / 384 entries: 6.1 / 6.7 / 7.6 us
 // against 8.1-8.3 us for the two launches; 2^17 leaves (six levels below the top): 8.2 / 9.7 / 11.6 us against
-// 7.7; 2^20 leaves, 512 entries: 22 us against 8.7. The kernel itself handles up to 1024 entries and trees
-// of kWgMaxDepth levels.
+// 7.7; 2^20 leaves, 512 entries: 22 us against 8.7. On the small trees it also beats the one-wave kernel above
+// for 64 entries or fewer (10,000 leaves: 5.45 against 5.87 us at 64, 5.15 against 5.82 at 16). The kernel itself
+// handles up to 1024 entries and trees of kWgMaxDepth levels.
 // ---------------------------------------------------------------------------
 constexpr int kWgMaxEntries = 1024;
-constexpr int kWgMinThreads = 512;                // so that two 16-byte pieces per thread stage the top of a tree
+constexpr int kWgMinThreads = 512; // so that kWgPieces 16-byte pieces per thread stage the top of a tree
+constexpr int kWgPieces = 2;
 constexpr int kWgTopLevels = 11;                  // levels 0 .. 11 of both trees live in LDS
 constexpr int kWgTopNodes = 2 << kWgTopLevels;    // 4096 (node 0 does not exist)
 constexpr int kWgSlotsLog2 = 11;
@@ -2035,10 +2037,10 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
         p = a.priorities[tid];
     }
     // the top of both trees, on its way while the entries arrive
-    const uint32_t top_vec = 1u << (T - 1);  // 16-byte pieces per tree: (2 << T) / 4, at most 2 * kWgMinThreads
-    f32x4 st_s[2], st_m[2];
+    const uint32_t top_vec = 1u << (T - 1);  // 16-byte pieces per tree: (2 << T) / 4, at most kWgPieces * kWgMinThreads
+    f32x4 st_s[kWgPieces], st_m[kWgPieces];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < kWgPieces; ++j) {
         const uint32_t i = tid + j * nthreads;
         st_s[j] = 0.0f;
         st_m[j] = 0.0f;
@@ -2095,7 +2097,7 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
     }
     // the staged top goes into LDS (needed only after several more barriers)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < kWgPieces; ++j) {
         const uint32_t i = tid + j * nthreads;
         if (i < top_vec) {
             reinterpret_cast<f32x4*>(top_s)[i] = st_s[j];
@@ -2151,9 +2153,9 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
                 }
             }
             // the table of the step before is free now: empty it for the step after the next
-            if (s >= 1 && tid < kWgSlots / 4) {
+            if (s >= 1) {
                 const f32x4 zero = 0.0f;
-                reinterpret_cast<f32x4*>(&keys[(s + 2) % 3][0])[tid] = zero;
+                for (uint32_t i = tid; i < kWgSlots / 4; i += nthreads) reinterpret_cast<f32x4*>(&keys[(s + 2) % 3][0])[i] = zero;
             }
             if (s + 1 < nh) {  // uniform
                 if (act) {
@@ -2202,7 +2204,7 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
     }
     lds_barrier();
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < kWgPieces; ++j) {
         const uint32_t i = tid + j * nthreads;
         if (i < top_vec) {
             reinterpret_cast<f32x4*>(a.sum)[i] = reinterpret_cast<const f32x4*>(top_s)[i];

@@ -944,7 +944,7 @@ def test_updates_with_invalid_entries_among_many(mrb, orc, cap, n):
 
 @pytest.mark.parametrize("cap", [4, 37, 1000, 2048, 4096, 5000, 10_000, 16_384])
 def test_updates_of_a_few_hundred_entries_on_small_trees(mrb, orc, cap):
-    """update_priorities of 65 .. 384 entries on trees of 2 .. 14 levels (one launch of one workgroup that walks
+    """update_priorities of 1 .. 384 entries on trees of 2 .. 14 levels (one launch of one workgroup that walks
     the entries' paths: the tree's top in LDS, the nodes below it in LDS hash tables, two levels per step): random
     indices, consecutive slots (neighbouring paths meet at every level), a handful of leaves hit by every entry
     (the latest entry wins each) and invalid entries among valid ones - trees, running max and flags as the
@@ -960,8 +960,10 @@ def test_updates_of_a_few_hundred_entries_on_small_trees(mrb, orc, cap):
     g.insert(*to_dev(rows))
     g2.insert(*to_dev(rows))
     c.push(rows, fill)
-    for n in (65, 100, 128, 255, 256, 321, 384):
+    for n in (1, 2, 17, 64, 65, 100, 128, 255, 256, 321, 384):
         for mode in ("random", "consecutive", "crowded", "invalid"):
+            if mode == "invalid" and n < 17:
+                continue
             if mode == "random":
                 idx = rng.integers(0, cap, n)
             elif mode == "consecutive":
