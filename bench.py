@@ -284,10 +284,19 @@ class PerRun:
         base, ip, wp = self.uniforms.data_ptr(), self.idx.data_ptr(), self.wts.data_ptr()
         self._sample_fn = self.L.mrb_per_sample
         self._sample_args = [(self.h, self.batch, float(self.betas[i]), base + i * self.batch * 4, ip, wp, self.fptr, self.sp)
-                             for i in range(self.K + self.W)]
+                             for i in range(self.n_draws)]
+        self._update_fn, self._push_fn = self.L.mrb_per_update, self.L.mrb_per_push
+        self._update_args = [(self.h, ip, self.upr[j].data_ptr(), self.upd, self.sp) for j in range(64)]
+        self._push_args = (self.h, self.sptr, self.ins_n, self.ins_pr, self.sp)
 
     def sample_bound(self, i):
         if self._sample_fn(*self._sample_args[i]):
+            self._lib.check(1)
+
+    def loop_bound(self, i):
+        """One step of the config's loop on the bench's stream: sample, update_priorities at the sampled indices, push."""
+        if (self._sample_fn(*self._sample_args[i]) or self._update_fn(*self._update_args[i % 64])
+                or self._push_fn(*self._push_args)):
             self._lib.check(1)
 
     def sample(self, i, sp=None, out=None):
@@ -313,7 +322,7 @@ def bench_per(a):
     K, W, batch = r.K, r.W, r.batch
     defaults = not (a.capacity or a.row_split or a.sample_path or a.graph)
     r.bind_sample_calls()
-    step = r.loop if r.loop_step else r.sample_bound
+    step = r.loop_bound if r.loop_step else r.sample_bound
     for i in range(W):
         step(i)
     torch.cuda.synchronize()
@@ -424,7 +433,7 @@ def per_extras(a, torch, r, algo_bytes):
     extras["updates_per_s"] = r.upd_n / timed(
         lambda i: L.mrb_per_update(h, uidx[i % 64].data_ptr(), r.upr[i % 64].data_ptr(), r.upd_n, sp))
     extras["inserts_per_s"] = r.ins_n / timed(lambda i: L.mrb_per_push(h, r.sptr, r.ins_n, r.ins_pr, sp))
-    extras["loop_steps_per_s"] = 1.0 / timed(lambda i: r.loop(W + i % K))
+    extras["loop_steps_per_s"] = 1.0 / timed(lambda i: r.loop_bound(W + i % K))
     # the same loop recorded ONCE into a HIP graph (50 steps) with the buffer's counters kept on the device, so
     # that every replay continues where the last one stopped; replayed 10 times
     if r.upd <= 1024:  # device-resident counters take updates of at most 1024 entries
