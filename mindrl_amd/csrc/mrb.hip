@@ -1069,6 +1069,19 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     }
     a.first_slot = b->device_counters ? -1 : first;
     a.n = n;
+    if (b->fused && nrows == 1 && b->depth <= kPushOneMaxDepth) {
+        // one row: one wave walks from its leaf to the root (k_push_one)
+        hipLaunchKernelGGL(k_push_one, dim3(1 + put.blocks), dim3(kWG), 0, s, a.sum, a.mn, a.maxp, a.first_slot, a.capacity,
+                           a.leaves, a.depth, a.alpha, opt_priorities, a.err, put);
+        LAUNCH_CHECK("k_push_one");
+        if (b->device_counters) {
+            rc = counters_advance(*b, nrows, 0, s);
+            if (rc) return rc;
+        }
+        b->pushes += nrows;
+        b->size = b->size + nrows < cap ? b->size + nrows : cap;
+        return MRB_OK;
+    }
     rc = tree_rebuild(*b, a, s, put.blocks ? &put : nullptr);
     if (rc) return rc;
     if (opt_priorities && !fold) {

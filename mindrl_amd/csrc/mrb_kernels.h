@@ -1944,6 +1944,65 @@ __global__ __launch_bounds__(64) void k_tree_paths(UpdateArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// A push of ONE row - the reference's insert() after every environment step - as one launch with one wave on
+// the tree: the row's leaf and the `depth` nodes above it are all the call changes, and the other child of each
+// is as memory holds it, at an address that follows from the slot. Lane L requests the sibling at level L, all
+// at once; the walk from the leaf to the root is then a chain of additions and minima on values read from the
+// lanes (no tile, no barrier, no second launch). The plain leading parameters are preloaded into scalar
+// registers, so the requests go out when the wave starts. The row copy rides along as further workgroups.
+// ---------------------------------------------------------------------------
+constexpr int kPushOneMaxDepth = 30;
+
+__global__ __launch_bounds__(kWG) void k_push_one(float* __restrict__ sum, float* __restrict__ mn, float* maxp,
+                                                  int64_t first_slot, int64_t capacity, int64_t leaves, int depth,
+                                                  float alpha, const float* priority, uint32_t* err, PutArgs put) {
+    if (blockIdx.x >= 1) {
+        rows_put_part(put, blockIdx.x - 1, put.blocks);
+        return;
+    }
+    if (threadIdx.x >= 64) return;
+    const uint32_t lane = threadIdx.x;
+    // negative: the ring position is on the device (see Counters)
+    const int64_t slot = first_slot >= 0 ? first_slot : ring_position(counters_behind(err), capacity);
+    const uint32_t v = (uint32_t)leaves + (uint32_t)slot;
+    float sib_s = 0.0f, sib_m = 0.0f;
+    if (lane >= 1 && lane <= (uint32_t)depth) {
+        const uint32_t node = (v >> ((uint32_t)depth - lane)) ^ 1u;
+        sib_s = sum[node];
+        sib_m = mn[node];
+    }
+    // the leaf: the running max as the call finds it, or the given priority's power (an invalid one is flagged
+    // and the row takes the running max, as a plain push would give it)
+    const float running = *maxp;
+    const float p = priority ? *priority : 0.0f;
+    const bool given = priority != nullptr && valid_priority(p);
+    if (priority != nullptr && !given && lane == 0) atomicOr(err, MRB_DERR_PRIORITY);
+    const float q = given ? powf_det_call(p, alpha) : running;
+    float cs = q, cm = q;
+    uint32_t node = v;
+    if (lane == 0) {
+        sum[node] = cs;
+        mn[node] = cm;
+    }
+#pragma unroll
+    for (int L = kPushOneMaxDepth; L >= 1; --L) {
+        if (L <= depth) {  // wave-uniform
+            const float os = lane_value(sib_s, L), om = lane_value(sib_m, L);
+            const bool right = (node & 1u) != 0;
+            cs = right ? os + cs : cs + os;
+            cm = right ? fminf(om, cm) : fminf(cm, om);
+            node >>= 1;
+            if (lane == 0) {
+                sum[node] = cs;
+                mn[node] = cm;
+            }
+        }
+    }
+    // last: the leaf has read the running max as the call found it
+    if (given && lane == 0 && q > 0.0f) raise_max(maxp, q);
+}
+
+// ---------------------------------------------------------------------------
 // update_priorities of at most 384 entries on a tree of at most 14 levels in ONE launch of ONE workgroup, a
 // thread per entry, again along the entries' paths: a call then costs one launch instead of a leaf round and
 // a top that wait for each other. What one wave settles among its lanes in k_tree_paths, the waves of a
