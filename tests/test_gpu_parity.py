@@ -332,6 +332,71 @@ def test_hip_graph_replays_a_whole_loop_with_device_counters(mrb, orc, cap, path
     g.destroy()
 
 
+@pytest.mark.parametrize("cap", [1, 2, 5, 1000, 70_000, 3_000_000])
+def test_single_row_pushes(mrb, orc, cap):
+    """insert() of one row - one wave's walk from the leaf to the root - on trees of 0 to 22 levels: plain pushes,
+    pushes with a priority (valid, zero, above the running max, invalid: flagged, the row takes the running max),
+    across the ring's wrap, compared with the oracle after every push; then the same recorded ONCE into a HIP graph
+    with the ring position on the device and replayed on new rows and priorities."""
+    rng = np.random.default_rng(9300 + cap % 1000)
+    shapes, dtypes = [(3,), (1,)], [np.float32, np.int32]
+    g, c = make_pair(mrb, orc, 0.6, cap, 4, seed=5, shapes=shapes, dtypes=dtypes)
+    fill = max(0, cap - 7)
+    if fill:
+        rows = random_rows(rng, fill, shapes, dtypes)
+        pr = rng.lognormal(0, 1, fill).astype(np.float32)
+        g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda()), c.push(rows, fill, pr)
+    for step in range(24):
+        row = random_rows(rng, 1, shapes, dtypes)
+        kind = step % 6
+        what = "cap %d step %d kind %d" % (cap, step, kind)
+        if kind in (0, 3):
+            g.insert(*to_dev(row)), c.push(row, 1)
+        else:
+            p = np.array([{1: rng.pareto(1.5) + 1e-6, 2: 0.0, 4: float(c.max_priority) * 3 + 1, 5: np.nan}[kind]], np.float32)
+            g.insert(*to_dev(row), priorities=torch.from_numpy(p).cuda())
+            if kind == 5:
+                c.push(row, 1)  # an invalid priority: the row keeps the running max, the call is flagged
+                with pytest.raises(ValueError):
+                    g.check()
+            else:
+                c.push(row, 1, p)
+        assert_tree_equal(g, c, what)
+        assert bits(np.float32(g.max_priority)) == bits(np.float32(c.max_priority)), what
+        assert g.size() == c.size and g._state()[1] == c.head, what
+    g.check()
+    u = rng.random(4).astype(np.float32)
+    assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(4, 0.5, u), "cap %d" % cap)
+    # recorded once, replayed: the ring position lives on the device
+    g.set_option("device_counters", 1)
+    one = [torch.zeros((1,) + tuple(sh), dtype=t).cuda() for sh, t in zip(shapes, torch_types(dtypes))]
+    two = [torch.zeros((1,) + tuple(sh), dtype=t).cuda() for sh, t in zip(shapes, torch_types(dtypes))]
+    p_dev = torch.ones(1, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        g.insert(*one)
+        g.insert(*two, priorities=p_dev)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for rep in range(10):
+        r1, r2 = random_rows(rng, 1, shapes, dtypes), random_rows(rng, 1, shapes, dtypes)
+        p = (rng.pareto(1.5, 1) + 1e-6).astype(np.float32)
+        for dst, src in zip(one + two, r1 + r2):
+            dst.copy_(torch.from_numpy(src))
+        p_dev.copy_(torch.from_numpy(p))
+        graph.replay()
+        torch.cuda.synchronize()
+        c.push(r1, 1), c.push(r2, 1, p)
+        assert_tree_equal(g, c, "cap %d replay %d" % (cap, rep))
+        assert g.size() == c.size and g._state()[1] == c.head
+    g.set_option("device_counters", 0)
+    del graph
+    g.destroy()
+
+
 def test_sample_output_ring(mrb, orc):
     """sample() hands out preallocated output sets in turn: `output_ring` calls return distinct tensors, the
     next call reuses the first set; output_ring=0 allocates fresh tensors; an explicit out= is written in
