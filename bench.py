@@ -63,6 +63,9 @@ def parse():
     p.add_argument("--sample-path", type=int, default=0, help="0 auto, 1 wide-row kernel, 2 LDS-top kernel")
     p.add_argument("--no-extras", action="store_true",
                    help="skip the untimed side figures (update, insert, loop, graph replay, several streams)")
+    p.add_argument("--settle-ms", type=float, default=300.0,
+                   help="untimed calls of the step for this long before the warm-up steps, so that a short timed "
+                        "region is not measured on a GPU that is still raising its clocks after the host-side set-up")
     return p.parse_args()
 
 
@@ -323,6 +326,15 @@ def bench_per(a):
     defaults = not (a.capacity or a.row_split or a.sample_path or a.graph)
     r.bind_sample_calls()
     step = r.loop_bound if r.loop_step else r.sample_bound
+    settle_calls = 0
+    if a.settle_ms > 0:
+        # not part of the W warm-up steps and not timed: the set-up above leaves the GPU idle for a while
+        t_end = time.perf_counter() + a.settle_ms * 1e-3
+        while time.perf_counter() < t_end:
+            for i in range(100):
+                step(i % r.n_draws)
+            torch.cuda.synchronize()
+            settle_calls += 100
     for i in range(W):
         step(i)
     torch.cuda.synchronize()
@@ -380,7 +392,7 @@ def bench_per(a):
         "config": {"workload": r.desc, "capacity": r.capacity, "batch": batch, "row_bytes": row_bytes, "alpha": 0.6,
                    "beta": "0.4->1.0" if a.workload == "c3" else "0.4",
                    "launch": "hip graph replay" if a.graph else "eager C-ABI calls, one stream, in order",
-                   "prefill_s": round(r.fill_s, 2), "device_flags": flags},
+                   "prefill_s": round(r.fill_s, 2), "settle_calls_before_warmup": settle_calls, "device_flags": flags},
     }
     if r.loop_step:
         # the sample kernel's share of a loop step is timed on its own; the loop itself is launch-bound
@@ -400,6 +412,8 @@ def bench_per(a):
         out["roofline"] = roofline(kernel_name, algo_bytes, dev_s / K, wall / K, a.workload, formula, defaults)
     if not a.no_extras:
         out["extras"] = per_extras(a, torch, r, algo_bytes)
+        if a.workload == "c3":
+            out["roofline"]["floor"] = sample_floor(torch, r, algo_bytes)
     if a.no_cpu_baseline:
         out["cpu_baseline"] = None
     elif r.loop_step:
@@ -409,6 +423,57 @@ def bench_per(a):
     r.buf.destroy()
     print(json.dumps(out))
     return 0
+
+
+def sample_floor(torch, r, algo_bytes):
+    """What this machine charges for the pieces of a config-3 sample call, each timed by HIP events over
+    back-to-back calls on the bench's stream (us per call): a launch of a kernel that does nothing; the runtime's
+    own contiguous device-to-device copy (hipMemcpyDtoDAsync) of as many bytes as a call gathers, from another
+    place of the ring every call (HBM) and from the same place (caches); the gather alone (mrb_per_gather, no
+    tree descent) at given slots that differ from call to call, over the whole ring and confined to its first
+    GiB; and the same slots every call (served by the caches). A sample call is the gather plus a descent that
+    must end before the first row byte can be requested."""
+    L, h, sp, batch = r.L, r.h, r.sp, r.batch
+    n = 400
+
+    def timed(fn):
+        for i in range(20):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = events(torch)
+        e0.record(r.stream)
+        for i in range(n):
+            fn(i)
+        e1.record(r.stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
+    out = {"unit": "us per call, HIP events over %d back-to-back calls" % n}
+    out["empty_launch"] = timed(lambda i: L.mrb_bench_launch(0, None, None, 0, sp))
+    store = r.buf.storage()[0]  # [capacity, 84, 84, 4] u8
+    row = r.buf._layout.bytes[0]
+    dst = r.fields[0]
+    nbytes = batch * row
+    places = max(1, (r.capacity // batch) - 1)
+    base = store.data_ptr()
+    out["d2d_copy_same_bytes_fresh_source"] = timed(
+        lambda i: L.mrb_bench_launch(1, dst.data_ptr(), base + ((i * 37) % places) * nbytes, nbytes, sp))
+    out["d2d_copy_same_bytes_same_source"] = timed(lambda i: L.mrb_bench_launch(1, dst.data_ptr(), base, nbytes, sp))
+    gfields = r.buf._layout.empty(batch, r.buf._dev)
+    gptr = r.pointers(gfields)
+    rng = np.random.default_rng(r.seed + 3)
+    nset = 256
+    for key, window in (("gather_fresh_slots_whole_ring", r.capacity),
+                        ("gather_fresh_slots_first_GiB", min(r.capacity, (1 << 30) // sum(r.buf._layout.bytes)))):
+        idx = torch.from_numpy(rng.integers(0, window, (nset, batch))).cuda()
+        out[key] = timed(lambda i: L.mrb_per_gather(h, idx[i % nset].data_ptr(), batch, gptr, sp))
+    out["gather_same_slots_every_call"] = timed(lambda i: L.mrb_per_gather(h, idx[0].data_ptr(), batch, gptr, sp))
+    out["frac_of_peak_of_d2d_copy_fresh_source"] = (
+        algo_bytes / (out["d2d_copy_same_bytes_fresh_source"] * 1e-6) / 1e9 / HBM_PEAK_GBS)
+    out["frac_of_peak_of_gather_fresh_slots"] = (
+        algo_bytes / (out["gather_fresh_slots_whole_ring"] * 1e-6) / 1e9 / HBM_PEAK_GBS)
+    r.buf.check()
+    return out
 
 
 def per_extras(a, torch, r, algo_bytes):

@@ -73,7 +73,11 @@ extern "C" {
 const char *mrb_last_error(void);
 /* 1 = HIP/gfx950. (There is no CPU backend in this library.) */
 int mrb_backend(void);
-/* ABI version of this header. */
+/* ABI version of this header: the library returns the MRB_ABI_VERSION it was built with; a binding
+ * compares the two before it makes any other call. History: 1 = mrb_set_option(name, value);
+ * 2 = mrb_set_option(handle, name, value), mrb_per_sample_many / _next / _update_noalloc added;
+ * 3 = mrb_per_update_push and mrb_bench_* added, updates of more than 1024 entries refuse stream capture. */
+#define MRB_ABI_VERSION 3
 int mrb_version(void);
 /* Tuning knobs of ONE buffer (any kind of handle); they change how its kernels are launched, never a
  * result. Unknown names return MRB_EINVAL. Set them while no call on the handle is in progress.
@@ -248,6 +252,15 @@ int mrb_res_set_counters(int64_t h, const int64_t *in4);
  * already raised to alpha), every other leaf to empty (sum 0, min FLT_MAX), rebuilds all internal
  * nodes and sets the running max priority. */
 int mrb_per_load_leaves(int64_t h, const float *leaves, int64_t n, float max_priority, void *stream);
+
+/* ---- measurement aids ---------------------------------------------------- */
+
+/* What a machine charges for the steady-state calls above before any of their work: no counterpart in
+ * the reference, no part of any buffer operation. kind 0: one launch of a kernel that does nothing
+ * (calls back to back on one stream give the cost of a launch); kind 1: hipMemcpyDtoDAsync of `bytes`
+ * bytes from src to dst, the runtime's own contiguous device-to-device copy (a gather of the same bytes
+ * is priced against it). Neither waits nor allocates. */
+int mrb_bench_launch(int kind, void *dst, const void *src, int64_t bytes, void *stream);
 
 /* ---- discounted return --------------------------------------------------- */
 

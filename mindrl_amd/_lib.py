@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmrb.so")
 MRB_OK, MRB_EINVAL, MRB_EHANDLE, MRB_EHIP, MRB_ESTATE, MRB_EDEVICE = 0, 1, 2, 3, 4, 5
 DERR_INDEX, DERR_PRIORITY, DERR_TOTAL, DERR_UNFILLED = 1, 2, 4, 8
 MAX_FIELDS = 16
+ABI_VERSION = 3  # MRB_ABI_VERSION of include/mrb.h this binding was written against
 
 _vp, _i64, _u64, _f32, _int = C.c_void_p, C.c_int64, C.c_uint64, C.c_float, C.c_int
 _pvp = C.POINTER(C.c_void_p)
@@ -60,6 +61,7 @@ SIGNATURES = {
     "mrb_res_get_counters": [_i64, _pi64],
     "mrb_res_set_counters": [_i64, _pi64],
     "mrb_per_load_leaves": [_i64, _vp, _i64, _f32, _vp],
+    "mrb_bench_launch": [_int, _vp, _vp, _i64, _vp],
     "mrb_discounted_return": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp],
 }
 
@@ -90,6 +92,9 @@ def lib():
         fn = getattr(L, name)
         fn.restype = C.c_int
         fn.argtypes = args
+    if L.mrb_version() != ABI_VERSION:
+        raise RuntimeError("libmrb.so reports ABI version %d, this binding expects %d: rebuild the library with "
+                           "`python -m mindrl_amd.build`" % (L.mrb_version(), ABI_VERSION))
     _lib = L
     return L
 

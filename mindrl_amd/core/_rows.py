@@ -53,6 +53,18 @@ def view_of(ptr, shape, dtype, owner, dev):
     return torch.as_tensor(_DeviceView(ptr, shape, _TYPESTR[dtype], owner), device=dev)
 
 
+def as_tensor(x):
+    """A torch tensor over `x` without a copy where that is possible: torch tensors as they are, any other
+    object that speaks DLPack (`__dlpack__` / `__dlpack_device__`: arrays of other frameworks, device-resident
+    ones included) through torch.from_dlpack - its memory is shared, nothing passes through the host -, and
+    everything else (numpy arrays, lists, scalars) through numpy."""
+    if isinstance(x, torch.Tensor):
+        return x
+    if hasattr(x, "__dlpack__") and hasattr(x, "__dlpack_device__") and not isinstance(x, np.ndarray):
+        return torch.from_dlpack(x)
+    return torch.as_tensor(np.asarray(x))
+
+
 class FieldLayout:
     """Shapes/dtypes of one buffer element, as given to the reference constructors
     (`shapes`, `types`: mindspore_rl/core/uniform_replay_buffer.py:75)."""
@@ -83,6 +95,8 @@ class FieldLayout:
         for f, numel in zip(fields, self.numel):
             if isinstance(f, torch.Tensor):
                 total = f.numel()
+            elif hasattr(f, "shape") and not isinstance(f, np.ndarray):  # a DLPack producer: no host copy to count
+                total = int(np.prod(tuple(f.shape), dtype=np.int64)) if len(tuple(f.shape)) else 1
             else:
                 total = int(np.prod(tuple(np.shape(f)), dtype=np.int64)) if len(np.shape(f)) else 1
             if total % numel:
@@ -116,8 +130,7 @@ class FieldLayout:
             if isinstance(f, torch.Tensor) and f.is_cuda and f.dtype == d and f.is_contiguous() and f.device == dev:
                 out.append(f)  # the common case: nothing to convert
                 continue
-            t = f if isinstance(f, torch.Tensor) else torch.as_tensor(np.asarray(f))
-            out.append(t.to(device=dev, dtype=d, non_blocking=False).contiguous())
+            out.append(as_tensor(f).to(device=dev, dtype=d, non_blocking=False).contiguous())
         return out
 
     def empty(self, n, dev):
@@ -141,6 +154,8 @@ def flat_on_device(x, dtype, dev):
     on the training path: no conversion, no copy)."""
     if isinstance(x, torch.Tensor) and x.dtype == dtype and x.device == dev and x.is_contiguous():
         return x if x.dim() == 1 else x.reshape(-1)
+    if not isinstance(x, torch.Tensor) and hasattr(x, "__dlpack__") and not isinstance(x, np.ndarray):
+        x = as_tensor(x)
     return torch.as_tensor(x).to(device=dev, dtype=dtype).contiguous().reshape(-1)
 
 

@@ -24,13 +24,14 @@ class PriorityReplayBuffer:
         sample_size (int): rows returned by sample().
         shapes, types: shape / element type of each tensor of an element.
         seed0, seed1 (int): generator seed; seed1 if non-zero, else seed0, else entropy.
-        output_ring (int): sample() hands out its result tensors from this many preallocated sets in
-            turn (default 4), so a call allocates nothing; a returned batch is overwritten by the
-            `output_ring`-th sample() call after it - clone() what must live longer. 0: fresh tensors
-            on every call.
+        output_ring (int): 0 (the default): sample() returns fresh tensors on every call, as the
+            reference does. N > 0 (opt-in, for loops that consume a batch before drawing the N-th next
+            one): sample() hands out its result tensors from N preallocated sets in turn, so a call
+            allocates nothing; a returned batch is then overwritten by the N-th sample() call after
+            it - clone() what must live longer.
     """
 
-    def __init__(self, alpha, capacity, sample_size, shapes, types, seed0=0, seed1=0, output_ring=4):
+    def __init__(self, alpha, capacity, sample_size, shapes, types, seed0=0, seed1=0, output_ring=0):
         self._dev = device()
         self._layout = FieldLayout(shapes, types)
         self._capacity = int(capacity)
@@ -94,8 +95,9 @@ class PriorityReplayBuffer:
         Returns (indices int64[B], weights f32[B], *transitions [B, *shape_i]).
         `uniforms` (f32[B] in [0,1)) replaces the buffer's generator, stratum k
         using uniforms[k]. `out` = (indices, weights, [fields]) writes into the caller's tensors.
-        Without `out` the result comes from the buffer's ring of preallocated output sets (see
-        `output_ring`): it stays valid until `output_ring` further sample() calls have been made."""
+        Without `out` the result is a set of fresh tensors, unless the buffer was built with
+        `output_ring` > 0: then it comes from that ring of preallocated output sets and stays valid
+        until `output_ring` further sample() calls have been made."""
         n = self._sample_size
         u = None
         if uniforms is not None:

@@ -591,6 +591,16 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
     if (b->device_counters && n > kElectMax)
         return fail(MRB_ESTATE, "with device_counters an update takes at most 1024 entries (larger ones elect their "
                                 "entries with tags the host counts, which a graph replay would repeat)");
+    if (n > kElectMax) {
+        // the stamp pass tags leaves with an epoch the HOST counts: a recording would freeze it, and replays would
+        // elect entries against stale tags. Refused while the stream is being captured (a host-side query).
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        HIP_TRY(hipStreamIsCapturing(s, &st));
+        if (st != hipStreamCaptureStatusNone)
+            return fail(MRB_ESTATE, "an update of more than %lld entries cannot be recorded into a HIP graph (its "
+                                    "election tags are counted on the host); split it into calls of at most %lld",
+                        (long long)kElectMax, (long long)kElectMax);
+    }
     int rc = next_epoch(*b, s);
     if (rc) return rc;
     UpdateArgs a = update_args(*b);
@@ -695,7 +705,7 @@ extern "C" {
 
 const char* mrb_last_error(void) { return g_err; }
 int mrb_backend(void) { return 1; }
-int mrb_version(void) { return 1; }
+int mrb_version(void) { return MRB_ABI_VERSION; }
 
 int mrb_set_option(int64_t h, const char* name, int64_t value) {
     if (!name) return fail(MRB_EINVAL, "option name is NULL");
@@ -1480,6 +1490,23 @@ int mrb_per_load_leaves(int64_t h, const float* leaves, int64_t n, float max_pri
     a.first_slot = 0;
     a.n = n;
     return tree_rebuild(*b, a, s);
+}
+
+/* ------------------------------------------------------------ measurement aids */
+
+int mrb_bench_launch(int kind, void* dst, const void* src, int64_t bytes, void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (kind == 0) {
+        hipLaunchKernelGGL(k_nothing, dim3(1), dim3(64), 0, s);
+        LAUNCH_CHECK("k_nothing");
+        return MRB_OK;
+    }
+    if (kind == 1) {
+        if (!dst || !src || bytes <= 0) return fail(MRB_EINVAL, "copy of %lld bytes from %p to %p", (long long)bytes, src, dst);
+        HIP_TRY(hipMemcpyDtoDAsync(dst, const_cast<void*>(src), (size_t)bytes, s));
+        return MRB_OK;
+    }
+    return fail(MRB_EINVAL, "unknown kind %d", kind);
 }
 
 /* ------------------------------------------------------- discounted return */

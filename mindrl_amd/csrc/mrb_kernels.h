@@ -10,17 +10,6 @@
 
 namespace mrb {
 
-// Timestamps inside the kernels, for tuning: compiled in only with -DMRB_PROBE (the library is never
-// built that way; a tuning build includes this file with the macro set and reads g_probe back).
-#ifdef MRB_PROBE
-__device__ uint64_t g_probe[16384 * 16];
-#define MRB_TS(var) const uint64_t var = wall_clock64()
-#define MRB_TS_OUT(slot, var) do { if ((threadIdx.x & 63) == 0 && (threadIdx.x < 64 || (slot) >= 0)) g_probe[(blockIdx.x * 16 + (slot)) & (16384 * 16 - 1)] = (var); } while (0)
-#else
-#define MRB_TS(var) do { } while (0)
-#define MRB_TS_OUT(slot, var) do { } while (0)
-#endif
-
 constexpr int kWG = 256;          // threads per workgroup of the row and sample kernels
 constexpr int kLdsWG = kWG + 64;  // the LDS-top sample kernel: kWG strata and a helper wave
 constexpr int kRoundLevels = 8;   // most tree levels rebuilt by one round of k_tree_update
@@ -530,8 +519,6 @@ struct CopyWork {
             // next to its conditional store, behind the other stores' waits)
 #pragma unroll
             for (int j = 0; j < kInF; ++j) asm volatile("" : "+v"(held[j]));
-            MRB_TS(ts_loaded);
-            MRB_TS_OUT(threadIdx.x < 128 ? 6 : (threadIdx.x < 192 ? 11 : 15), ts_loaded);
 #pragma unroll
             for (int j = 0; j < kInF; ++j) {
                 if (live & (1u << j)) {
@@ -595,7 +582,6 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
     const bool walker = wave == 0;
     const bool deep = depth == 21 || depth == 22;
     const uint32_t ctid = threadIdx.x - 64;  // copy thread number
-    MRB_TS(ts_start);
 
     if (deep) {
         // Trees of 21 and 22 levels would need three dependent node groups of <= 10 levels. Instead
@@ -715,9 +701,7 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
             }
         }
     }
-    MRB_TS(ts_at_barrier);
     __syncthreads();
-    MRB_TS(ts_past_barrier);
     const int64_t idx = s_idx;
     if (kNext && next_layer) {
         // the slot the sampled row names (outside [0, size): clamped and flagged, as mrb_per_gather does)
@@ -741,17 +725,6 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
         // the descent can end on an unfilled leaf past the last row (flagged by the walker)
         const uint32_t slot = (uint32_t)(idx < (int64_t)capacity ? idx : (int64_t)capacity - 1);
         work.run((uint32_t)__builtin_amdgcn_readfirstlane((int)slot), plan, narrow, nw, lane);
-        MRB_TS(ts_end);
-        if (wave == 1) {
-            MRB_TS_OUT(0, ts_start);
-            MRB_TS_OUT(2, ts_at_barrier);
-            MRB_TS_OUT(4, ts_past_barrier);
-            MRB_TS_OUT(7, ts_end);
-        } else if (wave == 2) {
-            MRB_TS_OUT(9, ts_at_barrier);
-            MRB_TS_OUT(10, ts_past_barrier);
-            MRB_TS_OUT(12, ts_end);
-        }
         return;
     }
     // ---- walker of the row's first workgroup: index and importance weight
@@ -771,11 +744,6 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
         if (!(total > 0.0f) || total > 3.0e38f) atomicOr(s_tail.err, MRB_DERR_TOTAL);
         if (idx >= size) atomicOr(s_tail.err, MRB_DERR_UNFILLED);
     }
-    MRB_TS(ts_wend);
-    MRB_TS_OUT(1, ts_start);
-    MRB_TS_OUT(3, ts_at_barrier);
-    MRB_TS_OUT(5, ts_past_barrier);
-    MRB_TS_OUT(8, ts_wend);
 }
 
 template <int kInF, bool kTen, bool kOneWide>
@@ -854,7 +822,6 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
     __shared__ float s_max_w;
     const uint32_t ntop = 2u << lds_levels;
     int64_t* s_slot = reinterpret_cast<int64_t*>(s_top + (ntop < 4 ? 4 : ntop));
-    MRB_TS(ts0);
     const int64_t k0 = (int64_t)blockIdx.x * kWG;
     const int64_t k = k0 + threadIdx.x;
     if (threadIdx.x >= kWG) {
@@ -877,7 +844,6 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
         s_top[threadIdx.x] = sum[threadIdx.x];
     }
     __syncthreads();
-    MRB_TS(ts1);
     constexpr int kOwn = 4;  // leading fields whose row is one granule: every thread copies its own stratum's
     AnyGranule own[kOwn];
     float weight = 0.0f;
@@ -902,10 +868,6 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
         // the additions the tree was built with. The remaining levels are taken five at a time, except
         // that seven are split 4 + 3 (5 + 1 + 1 would be a load more).
         float picked = depth <= lds_levels ? s_top[node] : 0.0f;
-#ifdef MRB_PROBE
-        asm volatile("" ::"v"(node), "v"(mass));
-#endif
-        MRB_TS(ts2);
         while (d < depth) {  // wave-uniform
             const int rest = depth - d;
             const int g = rest >= 5 ? (rest == 7 ? 4 : 5) : rest;
@@ -981,14 +943,6 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
             }
             d += g;
         }
-#ifdef MRB_PROBE
-        asm volatile("" ::"v"(node), "v"(mass));
-#endif
-        MRB_TS(ts3);
-        MRB_TS_OUT(0, ts0);
-        MRB_TS_OUT(1, ts1);
-        MRB_TS_OUT(2, ts2);
-        MRB_TS_OUT(3, ts3);
         const int64_t idx = (int64_t)node - ((int64_t)1 << depth);
         const int64_t slot = idx < a.capacity ? idx : a.capacity - 1;
         // the row's scalar fields are requested now, before the weight's arithmetic and the barrier
@@ -1002,17 +956,8 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
         sample_flags(a, total, idx, size);
         s_slot[threadIdx.x] = slot;
     }
-    MRB_TS(ts4);
     __syncthreads();
-    MRB_TS(ts5);
-    MRB_TS_OUT(4, ts4);
-    MRB_TS_OUT(5, ts5);
     const uint32_t rows = (uint32_t)((batch - k0) < kWG ? (batch - k0) : kWG);
-#ifdef MRB_PROBE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
-    MRB_TS(ts6);
-    MRB_TS_OUT(6, ts6);
     if (k < batch) {
         a.out_w[k] = weight / s_max_w;
 #pragma unroll
@@ -1035,8 +980,6 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
                          as_global(t.store[f]) + (uint64_t)s_slot[r] * t.row_bytes[f] + off, vl);
         }
     }
-    MRB_TS(ts7);
-    MRB_TS_OUT(7, ts7);
 }
 
 // ---------------------------------------------------------------------------
@@ -2541,6 +2484,9 @@ __global__ __launch_bounds__(kWG) void k_fill_uniforms(float* dst, uint64_t seed
 }
 
 // Fills a float array with one value (tree initialisation: sums 0, mins FLT_MAX).
+// A kernel that does nothing: what one launch costs (mrb_bench_launch).
+__global__ void k_nothing() {}
+
 __global__ __launch_bounds__(kWG) void k_fill_f32(float* p, float v, uint64_t n) {
     const uint64_t stride = (uint64_t)gridDim.x * kWG;
     for (uint64_t i = (uint64_t)blockIdx.x * kWG + threadIdx.x; i < n; i += stride) p[i] = v;

@@ -1576,3 +1576,89 @@ def test_random_configurations_and_operation_sequences(mrb, orc, block):
             assert g.size() == c.size and g._state()[1] == c.head, what
             assert np.float32(g.max_priority) == np.float32(c.max_priority), what
         g.destroy()
+
+
+class _Foreign:
+    """An array of another framework as far as this package can tell: it is no torch tensor and no numpy array,
+    it only speaks DLPack (and has a shape). Its memory is a device tensor's."""
+
+    def __init__(self, t):
+        self._t = t
+        self.shape = tuple(t.shape)
+        self.exports = 0
+
+    def __dlpack__(self, *args, **kwargs):
+        self.exports += 1
+        return self._t.__dlpack__(*args, **kwargs)
+
+    def __dlpack_device__(self):
+        return self._t.__dlpack_device__()
+
+
+def test_dlpack_producers_are_taken_without_a_copy(mrb, orc):
+    """insert / update_priorities / sample(uniforms=) accept objects that only speak DLPack; a device-resident
+    producer of the right type is used where it lies (same address, nothing passes through the host), and the
+    results equal the oracle's."""
+    from mindrl_amd.core._rows import as_tensor, flat_on_device
+    rng = np.random.default_rng(21)
+    cap, batch, n = 1000, 32, 300
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=3)
+    rows = id_rows(n)
+    dev_rows = to_dev(rows)
+    foreign = [_Foreign(t) for t in dev_rows]
+    for f, t in zip(foreign, dev_rows):
+        seen = as_tensor(f)
+        assert seen.data_ptr() == t.data_ptr() and seen.is_cuda  # shared memory, no copy
+    lay = g._layout
+    assert lay.batch_of(foreign) == n
+    on_dev = lay.to_device(foreign, g._dev)
+    assert [o.data_ptr() for o in on_dev] == [t.data_ptr() for t in dev_rows]
+    g.insert(*foreign), c.push(rows, n)
+    assert all(f.exports >= 1 for f in foreign)
+    idx = rng.integers(0, n, 50)
+    pr = (rng.pareto(1.5, 50) + 1e-6).astype(np.float32)
+    d_idx, d_pr = torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda()
+    assert flat_on_device(_Foreign(d_pr), torch.float32, g._dev).data_ptr() == d_pr.data_ptr()
+    g.update_priorities(_Foreign(d_idx), _Foreign(d_pr)), c.update(idx, pr)
+    u = rng.random(batch).astype(np.float32)
+    d_u = torch.from_numpy(u).cuda()
+    assert_sample_equal(g.sample(0.5, uniforms=_Foreign(d_u)), c.sample(batch, 0.5, u), "dlpack uniforms")
+    assert_tree_equal(g, c, "dlpack")
+    g.destroy()
+
+
+def test_large_updates_refuse_stream_capture(mrb):
+    """An update of more than 1024 entries elects its entries with tags the host counts; recorded into a HIP graph
+    it would replay against stale tags, so it is refused while the stream is capturing (both entry points), and
+    the capture itself stays usable: a small update recorded right after it replays correctly."""
+    import ctypes as C
+    cap, n = 50_000, 3000
+    shapes, types = [(3,), (1,)], [torch.float32, torch.int32]
+    g = mrb.PER(0.6, cap, 32, shapes, types, seed0=5)
+    g.insert(torch.randn(cap, 3, device="cuda"), torch.arange(cap, dtype=torch.int32, device="cuda").reshape(cap, 1))
+    idx = torch.randint(0, cap, (n,), device="cuda")
+    pr = torch.rand(n, device="cuda") + 0.1
+    L = mrb.lib.lib()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        sp = C.c_void_p(side.cuda_stream)
+        graph.capture_begin()
+        assert L.mrb_per_update(g._h, idx.data_ptr(), pr.data_ptr(), n, sp) == mrb.lib.MRB_ESTATE
+        assert b"1024" in L.mrb_last_error()
+        assert L.mrb_per_update_noalloc(g._h, idx.data_ptr(), pr.data_ptr(), n, sp) == mrb.lib.MRB_ESTATE
+        mrb.lib.check(L.mrb_per_update_noalloc(g._h, idx.data_ptr(), pr.data_ptr(), 1024, sp))  # the limit itself records
+        graph.capture_end()
+    torch.cuda.synchronize()
+    before = g.export_tree()[0].copy()
+    graph.replay()
+    torch.cuda.synchronize()
+    after = g.export_tree()[0]
+    leaves = after.size // 2
+    touched = np.unique(t2n(idx[:1024]))
+    assert np.any(before[leaves + touched] != after[leaves + touched])
+    mrb.lib.check(L.mrb_per_update(g._h, idx.data_ptr(), pr.data_ptr(), n, C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    assert g.check() == 0
+    del graph
+    g.destroy()
