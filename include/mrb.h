@@ -76,7 +76,7 @@ int mrb_backend(void);
 /* ABI version of this header: the library returns the MRB_ABI_VERSION it was built with; a binding
  * compares the two before it makes any other call. History: 1 = mrb_set_option(name, value);
  * 2 = mrb_set_option(handle, name, value), mrb_per_sample_many / _next / _update_noalloc added;
- * 3 = mrb_per_update_push and mrb_bench_* added, updates of more than 1024 entries refuse stream capture. */
+ * 3 = mrb_per_update_push and mrb_bench_launch added, updates of more than 1024 entries refuse stream capture. */
 #define MRB_ABI_VERSION 3
 int mrb_version(void);
 /* Tuning knobs of ONE buffer (any kind of handle); they change how its kernels are launched, never a
@@ -188,6 +188,18 @@ int mrb_per_sample_next(int64_t h, int64_t batch, float beta, const float *unifo
  * duplicates), every ancestor of a touched leaf recomputed from its final
  * children; max priority = max(old, all priorities[j]^alpha). */
 int mrb_per_update(int64_t h, const int64_t *indices, const float *priorities, int64_t n, void *stream);
+/* mrb_per_update(h, indices, priorities, n) followed by mrb_per_push(h, src_fields, nrows, opt_push_priorities),
+ * as ONE call: what a learner does after every step - the new priorities of the batch it has just used
+ * (priority_replay_buffer.py:108-120), then the transitions the actors have produced meanwhile (:78-90); the
+ * reference's training loop issues them back to back (mindspore_rl/algorithm/dqn/dqn_trainer.py:76-87). Same
+ * result, bit for bit, as the two calls (a pushed row without a priority takes the running max AFTER the
+ * update). No counterpart among the reference's primitives: it exists because each of these operations is
+ * bound by kernel launches, and together they need fewer - one launch for up to 384 entries and one row on a
+ * tree of at most 14 levels (or up to 64 entries on one of at most 25), two launches (instead of three) for up
+ * to 1024 entries and a few rows on a tree of 13 to 21 levels; other sizes run as the two calls would. */
+int mrb_per_update_push(int64_t h, const int64_t *indices, const float *priorities, int64_t n,
+                        const void *const *src_fields, int64_t nrows, const float *opt_push_priorities,
+                        void *stream);
 /* mrb_per_update for callers that cannot allocate: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments, same result
  * bit for bit; the scratch that mrb_per_update keeps per buffer (p^alpha of the call's entries) lives

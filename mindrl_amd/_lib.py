@@ -42,6 +42,7 @@ SIGNATURES = {
     "mrb_per_sample_next": [_i64, _i64, _f32, _vp, _int, _int, _vp, _vp, _pvp, _vp, _vp],
     "mrb_per_gather": [_i64, _vp, _i64, _pvp, _vp],
     "mrb_per_update": [_i64, _vp, _vp, _i64, _vp],
+    "mrb_per_update_push": [_i64, _vp, _vp, _i64, _pvp, _i64, _vp, _vp],
     "mrb_per_update_noalloc": [_i64, _vp, _vp, _i64, _vp],
     "mrb_per_export_tree": [_i64, _vp, _vp, _pi64, _vp],
     "mrb_per_state": [_i64, _pi64, _pi64, C.POINTER(C.c_float), _vp],

@@ -177,6 +177,33 @@ class PriorityReplayBuffer:
         self._keep = (idx, pr)
         return self._handle
 
+    def update_priorities_and_insert(self, indices, priorities, *transition, insert_priorities=None):
+        """update_priorities(indices, priorities) followed by insert(*transition, priorities=insert_priorities),
+        as ONE library call (mrb_per_update_push): the result is the two calls', bit for bit, with fewer kernel
+        launches - a learner's step is bound by them (the reference's loop issues the two back to back,
+        mindspore_rl/algorithm/dqn/dqn_trainer.py:76-87). Returns the handle tensor."""
+        idx = flat_on_device(indices, torch.int64, self._dev)
+        pr = flat_on_device(priorities, torch.float32, self._dev)
+        if idx.numel() != pr.numel():
+            raise ValueError("indices and priorities differ in length")
+        if len(transition) == 1 and isinstance(transition[0], (list, tuple)):
+            transition = tuple(transition[0])
+        n = self._layout.rows_if_ready(transition, self._dev)
+        if n is not None:
+            src = transition
+        else:
+            n = self._layout.batch_of(transition)
+            src = self._layout.to_device(transition, self._dev)
+        ipr = None
+        if insert_priorities is not None:
+            ipr = flat_on_device(insert_priorities, torch.float32, self._dev)
+            if ipr.numel() != n:
+                raise ValueError("insert_priorities must hold one value per pushed row")
+        _lib.check(_lib.lib().mrb_per_update_push(self._h, idx.data_ptr(), pr.data_ptr(), idx.numel(), pointers(src), n,
+                                                  ipr.data_ptr() if ipr is not None else None, stream_ptr()))
+        self._keep = (idx, pr, src, ipr)
+        return self._handle
+
     def gather(self, indices, out=None):
         """Rows at the given slots (int64, each in [0, size)): one [n, *shape_i] tensor per field.
         For transitions that store the slot of their successor instead of a copy of it, e.g.

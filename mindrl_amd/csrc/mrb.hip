@@ -1040,11 +1040,18 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     return MRB_OK;
 }
 
-int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const float* opt_priorities, void* stream) {
-    GET_PER(b, h);
+// The push behind mrb_per_push and mrb_per_update_push. `after_update`: an update_priorities of this very call
+// precedes the push on the stream and changed nodes anywhere in the tree, so a one-launch push rebuilds the
+// whole top (see UpdateArgs::full_top); `lead`, if given, is that update's leaf round, still to be launched:
+// the push's row copy rides along in it and the push's own tree work follows as the last launch.
+struct LeadRound {
+    UpdateArgs a;
+};
+
+static int per_push(Per* b, const void* const* src_fields, int64_t nrows, const float* opt_priorities, hipStream_t s,
+                    const LeadRound* lead = nullptr) {
     if (nrows <= 0) return fail(MRB_EINVAL, "nrows %lld must be positive", (long long)nrows);
     if (nrows > 0x7fffffffll) return fail(MRB_EINVAL, "nrows %lld exceeds 2^31 - 1 rows per call", (long long)nrows);
-    hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t cap = b->rows.capacity;
     if (b->device_counters && nrows > cap)
         return fail(MRB_ESTATE, "with device_counters a push takes at most capacity (%lld) rows", (long long)cap);
@@ -1064,9 +1071,17 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
         LAUNCH_CHECK("k_rows_put");
         put.blocks = 0;
     }
+    if (lead) {
+        // the update's leaf round (a wave or two per entry), with this push's row copy as further workgroups
+        const uint32_t waves = (lead->a.n > kPairedAbove ? 2u : 1u) * (uint32_t)lead->a.n;
+        hipLaunchKernelGGL(k_tree_update, dim3((waves + 3) / 4 + put.blocks), dim3(kWG), 0, s, lead->a, 0, 0u, put);
+        LAUNCH_CHECK("k_tree_update");
+        put.blocks = 0;
+    }
     rc = next_epoch(*b, s);
     if (rc) return rc;
     UpdateArgs a = update_args(*b);
+    a.full_top = lead ? 1 : 0;
     // push-then-update: the running max sees every priority of the call, surviving or not, and is
     // raised only after the tree work (a fresh slot with an invalid priority keeps the old running max).
     // Few rows: the top workgroup scans the priorities itself. More: the leaf-level waves, which compute
@@ -1079,7 +1094,7 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     }
     a.first_slot = b->device_counters ? -1 : first;
     a.n = n;
-    if (b->fused && nrows == 1 && b->depth <= kPushOneMaxDepth) {
+    if (!lead && b->fused && nrows == 1 && b->depth <= kPushOneMaxDepth) {
         // one row: one wave walks from its leaf to the root (k_push_one)
         hipLaunchKernelGGL(k_push_one, dim3(1 + put.blocks), dim3(kWG), 0, s, a.sum, a.mn, a.maxp, a.first_slot, a.capacity,
                            a.leaves, a.depth, a.alpha, opt_priorities, a.err, put);
@@ -1107,6 +1122,11 @@ int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const 
     b->pushes += nrows;
     b->size = b->size + nrows < cap ? b->size + nrows : cap;
     return MRB_OK;
+}
+
+int mrb_per_push(int64_t h, const void* const* src_fields, int64_t nrows, const float* opt_priorities, void* stream) {
+    GET_PER(b, h);
+    return per_push(b.get(), src_fields, nrows, opt_priorities, static_cast<hipStream_t>(stream));
 }
 
 int mrb_per_update(int64_t h, const int64_t* indices, const float* priorities, int64_t n, void* stream) {
@@ -1142,6 +1162,85 @@ int mrb_per_update_noalloc(int64_t h, const int64_t* indices, const float* prior
     HIP_TRY(hipGetDevice(&dev));
     if (dev != b->device) return fail(MRB_ESTATE, "the buffer lives on device %d, the current device is %d", b->device, dev);
     return per_update(*b, indices, priorities, n, powered, static_cast<hipStream_t>(stream));
+}
+
+// Leaf tiles a push of n rows can meet when its first slot is known (no wrap) or only known on the device.
+static uint32_t push_tiles(const Per& b, int64_t first, int64_t n) {
+    if (b.device_counters) {
+        UpdateArgs t{};
+        t.capacity = b.rows.capacity;
+        t.n = n;
+        return push_units(t);
+    }
+    if (first + n > b.rows.capacity) return 0xffffffffu;  // wraps: not a single run of tiles
+    return (uint32_t)((first + n - 1) / kBlockNodes) - (uint32_t)(first / kBlockNodes) + 1;
+}
+
+int mrb_per_update_push(int64_t h, const int64_t* indices, const float* priorities, int64_t n,
+                        const void* const* src_fields, int64_t nrows, const float* opt_push_priorities, void* stream) {
+    GET_PER(b, h);
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (n > 0xffffffffll) return fail(MRB_EINVAL, "n %lld exceeds 2^32 - 1 entries per call", (long long)n);
+    if (!indices || !priorities) return fail(MRB_EINVAL, "indices or priorities is NULL");
+    if (nrows <= 0) return fail(MRB_EINVAL, "nrows %lld must be positive", (long long)nrows);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t cap = b->rows.capacity;
+    const bool small_push = nrows <= cap && b->fused;
+    // (1) one launch: the one-workgroup or one-wave update, then the walk of the one pushed row by the same workgroup
+    const bool wg = n <= kWgBestEntries && b->depth >= 2 && b->depth <= kWgMaxDepth;
+    const bool paths = n <= kPathEntries && b->depth <= kPathMaxDepth && b->depth >= 2;
+    if (small_push && nrows == 1 && (wg || paths) && b->depth <= kPushOneMaxDepth) {
+        if (!src_fields) return fail(MRB_EINVAL, "field pointer array is NULL");
+        PutArgs put{};
+        const int64_t first = b->pushes % cap;
+        int rc = put_args(b->rows, src_fields, 0, 1, first, put);
+        if (rc) return rc;
+        if (b->device_counters) {
+            put.first_slot = -1;
+            put.src_first = reinterpret_cast<int64_t>(b->counters);
+        }
+        if (put.blocks <= 2048) {
+            rc = next_epoch(*b, s);
+            if (rc) return rc;
+            UpdateArgs a = update_args(*b);
+            a.indices = indices;
+            a.priorities = priorities;
+            a.n = n;
+            const int64_t slot = b->device_counters ? -1 : first;
+            if (wg) {
+                const uint32_t threads = n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
+                hipLaunchKernelGGL(k_tree_wg_push, dim3(1 + put.blocks), dim3(threads), 0, s, a, slot, opt_push_priorities, put);
+                LAUNCH_CHECK("k_tree_wg_push");
+            } else {
+                hipLaunchKernelGGL(k_tree_paths_push, dim3(1 + put.blocks), dim3(kWG), 0, s, a, slot, opt_push_priorities, put);
+                LAUNCH_CHECK("k_tree_paths_push");
+            }
+            if (b->device_counters) {
+                rc = counters_advance(*b, 1, 0, s);
+                if (rc) return rc;
+            }
+            b->pushes += 1;
+            b->size = b->size + 1 < cap ? b->size + 1 : cap;
+            return MRB_OK;
+        }
+    }
+    // (2) two launches on a tree with one round of levels below its top: the update's leaf round with the push's
+    // row copy riding along, then one workgroup that rebuilds the pushed slots' leaf tiles and the whole top
+    if (small_push && b->nrounds == 1 && n <= kElectMax && n > kFusedWG / 64 && b->depth >= 2 &&
+        push_tiles(*b, b->pushes % cap, nrows) <= (uint32_t)(kFusedWG / 64)) {
+        int rc = next_epoch(*b, s);
+        if (rc) return rc;
+        LeadRound lead{update_args(*b)};
+        lead.a.indices = indices;
+        lead.a.priorities = priorities;
+        lead.a.n = n;
+        lead.a.inline_election = 1;
+        return per_push(b.get(), src_fields, nrows, opt_push_priorities, s, &lead);
+    }
+    // (3) otherwise: the two calls, one after the other
+    int rc = mrb_per_update(h, indices, priorities, n, stream);
+    if (rc) return rc;
+    return per_push(b.get(), src_fields, nrows, opt_push_priorities, s);
 }
 
 // `nbatch` batches of `batch` stratified samples each, as nbatch successive mrb_per_sample calls on

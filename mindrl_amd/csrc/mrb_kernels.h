@@ -1039,6 +1039,8 @@ struct UpdateArgs {
     // sparse updates of very large trees: the lowest sparse_g0 levels are rebuilt per entry
     // (k_tree_sparse) instead of per tile
     int sparse_g0;               // 0 = not used
+    int full_top;                // a push that follows an update in the same call: the top is rebuilt over all its
+                                 // tiles, not only those above the pushed slots (the update changed others)
 };
 
 __device__ __forceinline__ bool valid_priority(float p) { return p >= 0.0f && p <= 3.0e38f; }
@@ -1627,7 +1629,7 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, unsign
     // A push that does not wrap changed the nodes above one run of slots only: above the leaf level, the
     // tiles outside that run hold what they held, and the waves they would occupy stay out of the way.
     uint32_t t_lo = 0, t_hi = tiles - 1;
-    if (!a.indices && top != a.depth && a.first_slot >= 0 && a.first_slot + a.n <= a.capacity) {
+    if (!a.indices && !a.full_top && top != a.depth && a.first_slot >= 0 && a.first_slot + a.n <= a.capacity) {
         t_lo = (uint32_t)(a.first_slot >> (a.depth - top)) / kBlockNodes;
         t_hi = (uint32_t)((a.first_slot + a.n - 1) >> (a.depth - top)) / kBlockNodes;
     }
@@ -1819,7 +1821,7 @@ __device__ __forceinline__ uint32_t bitonic_sort_wave(uint32_t key, uint32_t lan
     return key;
 }
 
-__global__ __launch_bounds__(64) void k_tree_paths(UpdateArgs a) {
+__device__ __forceinline__ void tree_paths_body(const UpdateArgs& a) {
     const uint32_t lane = threadIdx.x;
     // the entries: flags for the invalid ones, keys for the valid ones
     int64_t idx = -1;
@@ -1886,6 +1888,8 @@ __global__ __launch_bounds__(64) void k_tree_paths(UpdateArgs a) {
     }
 }
 
+__global__ __launch_bounds__(64) void k_tree_paths(UpdateArgs a) { tree_paths_body(a); }
+
 // ---------------------------------------------------------------------------
 // A push of ONE row - the reference's insert() after every environment step - as one launch with one wave on
 // the tree: the row's leaf and the `depth` nodes above it are all the call changes, and the other child of each
@@ -1896,15 +1900,13 @@ __global__ __launch_bounds__(64) void k_tree_paths(UpdateArgs a) {
 // ---------------------------------------------------------------------------
 constexpr int kPushOneMaxDepth = 30;
 
-__global__ __launch_bounds__(kWG) void k_push_one(float* __restrict__ sum, float* __restrict__ mn, float* maxp,
-                                                  int64_t first_slot, int64_t capacity, int64_t leaves, int depth,
-                                                  float alpha, const float* priority, uint32_t* err, PutArgs put) {
-    if (blockIdx.x >= 1) {
-        rows_put_part(put, blockIdx.x - 1, put.blocks);
-        return;
-    }
-    if (threadIdx.x >= 64) return;
-    const uint32_t lane = threadIdx.x;
+// The walk of one wave. kAfterUpdate: the walk follows an update_priorities in the same launch (same workgroup),
+// so the running max is read where the update's atomic maxima were performed (past this compute unit's cache),
+// and the siblings are requested only now, after the update's stores.
+template <bool kAfterUpdate>
+__device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp, int64_t first_slot,
+                                              int64_t capacity, int64_t leaves, int depth, float alpha,
+                                              const float* priority, uint32_t* err, uint32_t lane) {
     // negative: the ring position is on the device (see Counters)
     const int64_t slot = first_slot >= 0 ? first_slot : ring_position(counters_behind(err), capacity);
     const uint32_t v = (uint32_t)leaves + (uint32_t)slot;
@@ -1916,7 +1918,9 @@ __global__ __launch_bounds__(kWG) void k_push_one(float* __restrict__ sum, float
     }
     // the leaf: the running max as the call finds it, or the given priority's power (an invalid one is flagged
     // and the row takes the running max, as a plain push would give it)
-    const float running = *maxp;
+    const float running = kAfterUpdate ? __uint_as_float(__hip_atomic_load(reinterpret_cast<unsigned int*>(maxp), __ATOMIC_RELAXED,
+                                                                           __HIP_MEMORY_SCOPE_AGENT))
+                                       : *maxp;
     const float p = priority ? *priority : 0.0f;
     const bool given = priority != nullptr && valid_priority(p);
     if (priority != nullptr && !given && lane == 0) atomicOr(err, MRB_DERR_PRIORITY);
@@ -1943,6 +1947,17 @@ __global__ __launch_bounds__(kWG) void k_push_one(float* __restrict__ sum, float
     }
     // last: the leaf has read the running max as the call found it
     if (given && lane == 0 && q > 0.0f) raise_max(maxp, q);
+}
+
+__global__ __launch_bounds__(kWG) void k_push_one(float* __restrict__ sum, float* __restrict__ mn, float* maxp,
+                                                  int64_t first_slot, int64_t capacity, int64_t leaves, int depth,
+                                                  float alpha, const float* priority, uint32_t* err, PutArgs put) {
+    if (blockIdx.x >= 1) {
+        rows_put_part(put, blockIdx.x - 1, put.blocks);
+        return;
+    }
+    if (threadIdx.x >= 64) return;
+    push_one_walk<false>(sum, mn, maxp, first_slot, capacity, leaves, depth, alpha, priority, err, threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------
@@ -2019,7 +2034,7 @@ __device__ __forceinline__ bool wg_resolve(const uint32_t* keys, const unsigned 
     return true;
 }
 
-__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
+__device__ __forceinline__ void tree_wg_body(const UpdateArgs& a) {
     __shared__ __align__(16) float top_s[kWgTopNodes];
     __shared__ __align__(16) float top_m[kWgTopNodes];
     __shared__ __align__(16) uint32_t keys[3][kWgSlots];
@@ -2213,6 +2228,40 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
             reinterpret_cast<f32x4*>(a.mn)[i] = reinterpret_cast<const f32x4*>(top_m)[i];
         }
     }
+}
+
+__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) { tree_wg_body(a); }
+
+// ---------------------------------------------------------------------------
+// update_priorities followed by a push of ONE row, in ONE launch (mrb_per_update_push: what a learner does after
+// every step - the priorities of the batch it has just used, then the transition the actor has just produced).
+// Workgroup 0 runs the one-workgroup (or one-wave) update above and then, behind a workgroup barrier, the walk
+// of k_push_one: its waves share a compute unit, so the update's stores are what the walk's loads find. The
+// row copy rides along as further workgroups, as in k_push_one.
+//   slot      the pushed row's slot (negative: read from the device, see Counters)
+//   priority  the pushed row's priority (NULL: the running max, which includes this call's update)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
+    if (blockIdx.x >= 1) {
+        rows_put_part(put, blockIdx.x - 1, put.blocks);
+        return;
+    }
+    tree_wg_body(a);
+    __threadfence_block();
+    __syncthreads();
+    if (threadIdx.x < 64)
+        push_one_walk<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x);
+}
+
+__global__ __launch_bounds__(kWG) void k_tree_paths_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
+    if (blockIdx.x >= 1) {
+        rows_put_part(put, blockIdx.x - 1, put.blocks);
+        return;
+    }
+    if (threadIdx.x >= 64) return;
+    tree_paths_body(a);
+    __threadfence_block();
+    push_one_walk<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------

@@ -1662,3 +1662,62 @@ def test_large_updates_refuse_stream_capture(mrb):
     assert g.check() == 0
     del graph
     g.destroy()
+
+
+@pytest.mark.parametrize("cap", [1, 2, 3, 100, 3000, 10_000, 16_384, 20_000, 70_000, 300_000, 1_000_000, 2_200_000, 5_000_000])
+def test_update_push_equals_update_then_push(mrb, orc, cap):
+    """mrb_per_update_push against the oracle's update followed by its push, on trees of 0 to 23 levels: one
+    pushed row or a few, with and without priorities for the pushed rows, duplicate, invalid and out-of-range
+    entries, entries aimed at the very slots the push overwrites, across the ring's wrap; 1 to 1100 entries (the
+    one-workgroup, one-wave, two-launch and two-call paths). Both trees, the running max, size, head, rows and a
+    sample are compared after every call."""
+    rng = np.random.default_rng(cap + 77)
+    batch = 16
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=2)
+    fill = max(1, cap - 7)  # the pushes below run across the end of the ring
+    chunk = 200_000
+    serial = 0
+    while serial < fill:
+        n = min(chunk, fill - serial)
+        rows = id_rows(n, serial)
+        g.insert(*to_dev(rows)), c.push(rows, n)
+        serial += n
+    exp_flags = 0
+    for step, (k, nrows) in enumerate([(1, 1), (64, 1), (17, 1), (300, 1), (512, 4), (40, 3), (1000, 7), (1100, 2),
+                                       (512, 1), (64, 1), (200, 300), (5, 20), (384, 1), (65, 1)]):
+        idx = rng.integers(0, cap, k)
+        if step % 3 == 0 and k > 4:
+            idx[: k // 3] = idx[0]  # duplicates: the last entry wins
+        head = c.head
+        if step % 2 == 1 and k > 2:
+            idx[-1] = head  # the slot the push overwrites next: the push's value must win
+            idx[0] = (head + nrows - 1) % cap
+        pr = (rng.pareto(1.5, k) + 1e-6).astype(np.float32)
+        if step % 4 == 2 and k > 8:
+            pr[3] = -1.0
+            idx[5] = cap + 9
+            exp_flags |= 3
+        if step == 6:
+            pr[k // 2] = np.float32(1e6)  # a new running max that the pushed rows must take
+        rows = id_rows(nrows, serial)
+        serial += nrows
+        ipr = None
+        if step % 5 == 4:
+            ipr = (np.abs(rng.normal(size=nrows)) + 1e-6).astype(np.float32)
+        g.update_priorities_and_insert(torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda(), *to_dev(rows),
+                                       insert_priorities=None if ipr is None else torch.from_numpy(ipr).cuda())
+        ok = (idx >= 0) & (idx < cap) & np.isfinite(pr) & (pr >= 0)  # the device skips and flags the others
+        c.update(idx[ok], pr[ok])
+        c.push(rows, nrows, ipr)
+        what = "cap %d step %d (%d entries, %d rows)" % (cap, step, k, nrows)
+        assert_tree_equal(g, c, what)
+        assert g.size() == c.size and g._state()[1] == c.head, what
+        assert np.float32(g.max_priority) == np.float32(c.max_priority), what
+        u = rng.random(batch).astype(np.float32)
+        assert_sample_equal(g.sample(0.5, uniforms=torch.from_numpy(u).cuda()), c.sample(batch, 0.5, u), what)
+    for f, (a, b) in enumerate(zip(g.storage(), [c.field(0), c.field(1)])):
+        assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8)), f
+    flags = C.c_uint32(0)
+    assert mrb.lib.lib().mrb_per_check(g._h, C.byref(flags), None) == 0
+    assert (flags.value & 3) == exp_flags, flags.value
+    g.destroy()

@@ -24,7 +24,7 @@ def declared_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = declared_symbols()
-    assert len(names) == 44
+    assert len(names) == 45
     L = _lib.lib()
     for n in names:
         assert hasattr(L, n), "libmrb.so does not export %s" % n
@@ -100,7 +100,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
     assert sum("k_per_sample_wide" in k for k in kernels) == 8 and sum("k_rows_gather_wide" in k for k in kernels) == 4
-    assert len(kernels) == 41, sorted(kernels)
+    assert len(kernels) == 43, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)
@@ -127,7 +127,7 @@ def test_only_the_documented_entry_points_wait_or_allocate():
     may_wait = {"mrb_urb_create", "mrb_per_create", "mrb_res_create", "mrb_urb_destroy", "mrb_per_destroy",
                 "mrb_res_destroy", "mrb_per_state", "mrb_per_export_tree", "read_and_clear_flags", "rows_alloc",
                 "counters_to_device", "counters_from_device"}
-    may_alloc = {"mrb_urb_create", "mrb_per_create", "mrb_res_create", "rows_alloc", "mrb_per_update"}
+    may_alloc = {"mrb_urb_create", "mrb_per_create", "mrb_res_create", "rows_alloc", "mrb_per_update"}  # (mrb_per_update_push calls it)
     for name, body in bodies.items():
         if name not in may_wait:
             assert not waits.search(body), "%s waits for the device" % name
