@@ -291,6 +291,9 @@ class PerRun:
         self._update_fn, self._push_fn = self.L.mrb_per_update, self.L.mrb_per_push
         self._update_args = [(self.h, ip, self.upr[j].data_ptr(), self.upd, self.sp) for j in range(64)]
         self._push_args = (self.h, self.sptr, self.ins_n, self.ins_pr, self.sp)
+        self._update_push_fn = self.L.mrb_per_update_push
+        self._update_push_args = [(self.h, ip, self.upr[j].data_ptr(), self.upd, self.sptr, self.ins_n, self.ins_pr, self.sp)
+                                  for j in range(64)]
 
     def sample_bound(self, i):
         if self._sample_fn(*self._sample_args[i]):
@@ -302,6 +305,11 @@ class PerRun:
                 or self._push_fn(*self._push_args)):
             self._lib.check(1)
 
+    def loop_fused_bound(self, i):
+        """The same step with update_priorities and the push as ONE call (mrb_per_update_push)."""
+        if self._sample_fn(*self._sample_args[i]) or self._update_push_fn(*self._update_push_args[i % 64]):
+            self._lib.check(1)
+
     def sample(self, i, sp=None, out=None):
         ip, wp, fptr = out if out else (self.idx.data_ptr(), self.wts.data_ptr(), self.fptr)
         rc = self.L.mrb_per_sample(self.h, self.batch, float(self.betas[i]), self.uniforms.data_ptr() + i * self.batch * 4,
@@ -309,10 +317,14 @@ class PerRun:
         if rc:
             self._lib.check(rc)
 
-    def loop(self, i, sp=None):
+    def loop(self, i, sp=None, fused=False):
         self.sample(i, sp)
-        rc = self.L.mrb_per_update(self.h, self.idx.data_ptr(), self.upr[i % 64].data_ptr(), self.upd, sp or self.sp)
-        rc = rc or self.L.mrb_per_push(self.h, self.sptr, self.ins_n, self.ins_pr, sp or self.sp)
+        if fused:
+            rc = self.L.mrb_per_update_push(self.h, self.idx.data_ptr(), self.upr[i % 64].data_ptr(), self.upd, self.sptr,
+                                            self.ins_n, self.ins_pr, sp or self.sp)
+        else:
+            rc = self.L.mrb_per_update(self.h, self.idx.data_ptr(), self.upr[i % 64].data_ptr(), self.upd, sp or self.sp)
+            rc = rc or self.L.mrb_per_push(self.h, self.sptr, self.ins_n, self.ins_pr, sp or self.sp)
         if rc:
             self._lib.check(rc)
 
@@ -499,28 +511,32 @@ def per_extras(a, torch, r, algo_bytes):
         lambda i: L.mrb_per_update(h, uidx[i % 64].data_ptr(), r.upr[i % 64].data_ptr(), r.upd_n, sp))
     extras["inserts_per_s"] = r.ins_n / timed(lambda i: L.mrb_per_push(h, r.sptr, r.ins_n, r.ins_pr, sp))
     extras["loop_steps_per_s"] = 1.0 / timed(lambda i: r.loop_bound(W + i % K))
+    # the same step with update_priorities and the insert as one call (mrb_per_update_push: fewer launches)
+    extras["update_push_us_per_call"] = timed(lambda i: r._update_push_fn(*r._update_push_args[i % 64])) * 1e6
+    extras["loop_update_push_steps_per_s"] = 1.0 / timed(lambda i: r.loop_fused_bound(W + i % K))
     # the same loop recorded ONCE into a HIP graph (50 steps) with the buffer's counters kept on the device, so
     # that every replay continues where the last one stopped; replayed 10 times
     if r.upd <= 1024:  # device-resident counters take updates of at most 1024 entries
         r.buf.set_option("device_counters", 1)
         n_l = min(K, 50)
-        lgraph = torch.cuda.CUDAGraph()
-        lside = torch.cuda.Stream()
-        with torch.cuda.stream(lside):
-            lsp = C.c_void_p(lside.cuda_stream)
-            lgraph.capture_begin()
-            for i in range(n_l):
-                r.loop(W + i, lsp)
-            lgraph.capture_end()
-        torch.cuda.synchronize()
-        lgraph.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(10):
+        for key, fused in (("loop_graph_replay_steps_per_s", False), ("loop_update_push_graph_replay_steps_per_s", True)):
+            lgraph = torch.cuda.CUDAGraph()
+            lside = torch.cuda.Stream()
+            with torch.cuda.stream(lside):
+                lsp = C.c_void_p(lside.cuda_stream)
+                lgraph.capture_begin()
+                for i in range(n_l):
+                    r.loop(W + i, lsp, fused)
+                lgraph.capture_end()
+            torch.cuda.synchronize()
             lgraph.replay()
-        torch.cuda.synchronize()
-        extras["loop_graph_replay_steps_per_s"] = 10 * n_l / (time.perf_counter() - t0)
-        del lgraph
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(10):
+                lgraph.replay()
+            torch.cuda.synchronize()
+            extras[key] = 10 * n_l / (time.perf_counter() - t0)
+            del lgraph
         r.buf.set_option("device_counters", 0)
     if not r.loop_step:
         extras["sample_us_per_call"] = timed(lambda i: r.sample(W + i % K)) * 1e6

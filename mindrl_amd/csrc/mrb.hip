@@ -497,6 +497,7 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
         if (units > 0 && units <= (uint32_t)(kFusedWG / 64)) {
             PutArgs put = ride ? *ride : none;
             put.blocks = (put.blocks + 3) / 4;  // the ride-along copy was sized for workgroups a quarter as large
+            a.readers = 1 + put.blocks;         // (a.advance != 0: this one launch also moves the device's counters on)
             hipLaunchKernelGGL(k_tree_fused, dim3(1 + put.blocks), dim3(kFusedWG), 0, s, a, tile_base, units, put);
             LAUNCH_CHECK("k_tree_fused");
             return MRB_OK;
@@ -529,6 +530,9 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
         LAUNCH_CHECK("k_tree_update");
     }
     const PutArgs& put = (a.nrounds == 0 && ride) ? *ride : none;
+    // the top is the call's last launch: it moves the device's counters on (a.advance != 0); only when it is also
+    // the first do its workgroups read the ring position
+    a.readers = a.nrounds == 0 ? 1 + put.blocks : 0;
     hipLaunchKernelGGL(k_tree_top, dim3(1 + put.blocks), dim3(kTopWG), 0, s, a, put);
     LAUNCH_CHECK("k_tree_top");
     return MRB_OK;
@@ -1065,8 +1069,10 @@ static int per_push(Per* b, const void* const* src_fields, int64_t nrows, const 
         put.first_slot = -1;
         put.src_first = reinterpret_cast<int64_t>(b->counters);
     }
-    if (put.blocks > 2048) {
-        // a large copy gets its own launch; a small one rides along in the first tree launch
+    // A large copy gets its own launch; a small one rides along in the first tree launch. (With the counters on
+    // the device every workgroup that rides along reports to one counter when it is done - see
+    // counters_push_done -, which is worth it for a few dozen workgroups only.)
+    if (put.blocks > (b->device_counters ? 64u : 2048u)) {
         hipLaunchKernelGGL(k_rows_put, dim3(put.blocks), dim3(kWG), 0, s, put);
         LAUNCH_CHECK("k_rows_put");
         put.blocks = 0;
@@ -1094,30 +1100,24 @@ static int per_push(Per* b, const void* const* src_fields, int64_t nrows, const 
     }
     a.first_slot = b->device_counters ? -1 : first;
     a.n = n;
+    a.advance = b->device_counters ? nrows : 0;  // the call's last launch moves the device's counters on
+    const bool stamp_after = opt_priorities && !fold;
     if (!lead && b->fused && nrows == 1 && b->depth <= kPushOneMaxDepth) {
         // one row: one wave walks from its leaf to the root (k_push_one)
         hipLaunchKernelGGL(k_push_one, dim3(1 + put.blocks), dim3(kWG), 0, s, a.sum, a.mn, a.maxp, a.first_slot, a.capacity,
-                           a.leaves, a.depth, a.alpha, opt_priorities, a.err, put);
+                           a.leaves, a.depth, a.alpha, opt_priorities, a.err, put, a.advance, 1 + put.blocks);
         LAUNCH_CHECK("k_push_one");
-        if (b->device_counters) {
-            rc = counters_advance(*b, nrows, 0, s);
-            if (rc) return rc;
-        }
         b->pushes += nrows;
         b->size = b->size + nrows < cap ? b->size + nrows : cap;
         return MRB_OK;
     }
     rc = tree_rebuild(*b, a, s, put.blocks ? &put : nullptr);
     if (rc) return rc;
-    if (opt_priorities && !fold) {
+    if (stamp_after) {
         a.priorities = opt_priorities;
         a.n = nrows;
         hipLaunchKernelGGL(k_update_stamp, dim3(grid_exact((uint64_t)nrows)), dim3(kWG), 0, s, a);
         LAUNCH_CHECK("k_update_stamp");
-    }
-    if (b->device_counters) {
-        rc = counters_advance(*b, nrows, 0, s);
-        if (rc) return rc;
     }
     b->pushes += nrows;
     b->size = b->size + nrows < cap ? b->size + nrows : cap;
@@ -1199,13 +1199,15 @@ int mrb_per_update_push(int64_t h, const int64_t* indices, const float* prioriti
             put.first_slot = -1;
             put.src_first = reinterpret_cast<int64_t>(b->counters);
         }
-        if (put.blocks <= 2048) {
+        if (put.blocks <= (b->device_counters ? 64u : 2048u)) {
             rc = next_epoch(*b, s);
             if (rc) return rc;
             UpdateArgs a = update_args(*b);
             a.indices = indices;
             a.priorities = priorities;
             a.n = n;
+            a.advance = b->device_counters ? 1 : 0;
+            a.readers = 1 + put.blocks;
             const int64_t slot = b->device_counters ? -1 : first;
             if (wg) {
                 const uint32_t threads = n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
@@ -1214,10 +1216,6 @@ int mrb_per_update_push(int64_t h, const int64_t* indices, const float* prioriti
             } else {
                 hipLaunchKernelGGL(k_tree_paths_push, dim3(1 + put.blocks), dim3(kWG), 0, s, a, slot, opt_push_priorities, put);
                 LAUNCH_CHECK("k_tree_paths_push");
-            }
-            if (b->device_counters) {
-                rc = counters_advance(*b, 1, 0, s);
-                if (rc) return rc;
             }
             b->pushes += 1;
             b->size = b->size + 1 < cap ? b->size + 1 : cap;

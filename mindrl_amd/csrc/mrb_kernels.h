@@ -147,6 +147,26 @@ __device__ __forceinline__ int64_t ring_position(const int64_t* counters, int64_
     return (int64_t)((uint64_t)counters[kCntPushes] % (uint64_t)capacity);
 }
 
+// A push moves the device-resident counters on in its own last launch. Where that launch is also the one whose
+// workgroups read the ring position (`readers` of them: the tree workgroup and the row copy's), every such
+// workgroup reports here when it is done, and the last one to report advances the counters: no workgroup waits
+// for another, and none can read a position already moved on. readers <= 1: the caller is the only reader left.
+// Called by every thread of the workgroup (it contains a barrier); the counters' fourth word counts the reports.
+__device__ __forceinline__ void counters_push_done(uint32_t* err, int64_t pushed, int64_t capacity, uint32_t readers) {
+    if (pushed <= 0) return;  // uniform over the launch
+    __syncthreads();          // every wave's reads of the position are behind it
+    if (threadIdx.x != 0) return;
+    int64_t* counters = reinterpret_cast<int64_t*>(err + 4);
+    if (readers > 1) {
+        unsigned int* arrived = reinterpret_cast<unsigned int*>(counters + 3);
+        if (atomicAdd(arrived, 1u) != readers - 1) return;
+        atomicExch(arrived, 0u);
+    }
+    counters[kCntPushes] += pushed;
+    const int64_t size = counters[kCntSize] + pushed;
+    counters[kCntSize] = size < capacity ? size : capacity;
+}
+
 // The copy itself, by workgroup `block` of `nblocks` (grid-stride over the granules).
 __device__ __forceinline__ void rows_put_part(const PutArgs& p, uint32_t block, uint32_t nblocks) {
     const IoTable& t = p.t;
@@ -1041,6 +1061,10 @@ struct UpdateArgs {
     int sparse_g0;               // 0 = not used
     int full_top;                // a push that follows an update in the same call: the top is rebuilt over all its
                                  // tiles, not only those above the pushed slots (the update changed others)
+    // device-resident counters: rows this launch - the push's last - adds to them when it is done (0: none), and
+    // the workgroups of this launch that read the ring position (see counters_push_done)
+    int64_t advance;
+    uint32_t readers;
 };
 
 __device__ __forceinline__ bool valid_priority(float p) { return p >= 0.0f && p <= 3.0e38f; }
@@ -1712,10 +1736,12 @@ __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) 
     __shared__ unsigned long long s_win[kTopWG / 64][kBlockNodes];
     if (blockIdx.x >= 1) {
         rows_put_part(put, blockIdx.x - 1, put.blocks);
+        counters_push_done(a.err, a.advance, a.capacity, a.readers);
         return;
     }
     top_rebuild(a, a.top_depth, &s_win[0][0]);
     if (a.fold_max) fold_push_max(a);
+    counters_push_done(a.err, a.advance, a.capacity, a.readers);
 }
 
 // ---------------------------------------------------------------------------
@@ -1734,6 +1760,7 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
     __shared__ unsigned long long s_win[kFusedWG / 64][kBlockNodes];
     if (blockIdx.x >= 1) {
         rows_put_part(put, blockIdx.x - 1, put.blocks);
+        counters_push_done(a.err, a.advance, a.capacity, a.readers);
         return;
     }
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1752,6 +1779,7 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
     __syncthreads();
     top_rebuild(a, a.top_depth, &s_win[0][0]);
     if (a.fold_max) fold_push_max(a);
+    counters_push_done(a.err, a.advance, a.capacity, a.readers);
 }
 
 // ---------------------------------------------------------------------------
@@ -1951,13 +1979,16 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
 
 __global__ __launch_bounds__(kWG) void k_push_one(float* __restrict__ sum, float* __restrict__ mn, float* maxp,
                                                   int64_t first_slot, int64_t capacity, int64_t leaves, int depth,
-                                                  float alpha, const float* priority, uint32_t* err, PutArgs put) {
+                                                  float alpha, const float* priority, uint32_t* err, PutArgs put,
+                                                  int64_t advance, uint32_t readers) {
     if (blockIdx.x >= 1) {
         rows_put_part(put, blockIdx.x - 1, put.blocks);
+        counters_push_done(err, advance, capacity, readers);
         return;
     }
-    if (threadIdx.x >= 64) return;
-    push_one_walk<false>(sum, mn, maxp, first_slot, capacity, leaves, depth, alpha, priority, err, threadIdx.x);
+    if (threadIdx.x < 64)
+        push_one_walk<false>(sum, mn, maxp, first_slot, capacity, leaves, depth, alpha, priority, err, threadIdx.x);
+    counters_push_done(err, advance, capacity, readers);
 }
 
 // ---------------------------------------------------------------------------
@@ -2244,6 +2275,7 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) { tree_
 __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
     if (blockIdx.x >= 1) {
         rows_put_part(put, blockIdx.x - 1, put.blocks);
+        counters_push_done(a.err, a.advance, a.capacity, a.readers);
         return;
     }
     tree_wg_body(a);
@@ -2251,17 +2283,21 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(UpdateArgs a, in
     __syncthreads();
     if (threadIdx.x < 64)
         push_one_walk<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x);
+    counters_push_done(a.err, a.advance, a.capacity, a.readers);
 }
 
 __global__ __launch_bounds__(kWG) void k_tree_paths_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
     if (blockIdx.x >= 1) {
         rows_put_part(put, blockIdx.x - 1, put.blocks);
+        counters_push_done(a.err, a.advance, a.capacity, a.readers);
         return;
     }
-    if (threadIdx.x >= 64) return;
-    tree_paths_body(a);
-    __threadfence_block();
-    push_one_walk<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x);
+    if (threadIdx.x < 64) {
+        tree_paths_body(a);
+        __threadfence_block();
+        push_one_walk<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x);
+    }
+    counters_push_done(a.err, a.advance, a.capacity, a.readers);
 }
 
 // ---------------------------------------------------------------------------

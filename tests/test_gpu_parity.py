@@ -1721,3 +1721,63 @@ def test_update_push_equals_update_then_push(mrb, orc, cap):
     assert mrb.lib.lib().mrb_per_check(g._h, C.byref(flags), None) == 0
     assert (flags.value & 3) == exp_flags, flags.value
     g.destroy()
+
+
+@pytest.mark.parametrize("cap,npush,batch", [(3000, 1, 48), (10_000, 1, 64), (70_000, 1, 48), (70_000, 3, 300), (1_000_000, 4, 512),
+                                             (3_000_000, 1, 40), (3_000_000, 2, 100)])
+def test_hip_graph_replays_sample_then_update_push_with_device_counters(mrb, orc, cap, npush, batch):
+    """The learner's step as two calls - a generator-driven sample, then update_priorities of the sampled rows and
+    the push of new ones as ONE call (mrb_per_update_push) - recorded once with device_counters and replayed 10
+    times: the push's own last launch moves the ring position on (no separate launch), the buffer fills, the ring
+    wraps. Every replay equals the oracle's sample, update, push; eager calls in between use the same counters."""
+    rng = np.random.default_rng(cap + npush)
+    shapes, dtypes = ([(300,), (1,), (2,)], [np.float32, np.int32, np.uint8]) if cap < 10 ** 5 else ([(2,), (1,)], [np.float32, np.int32])
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=17, shapes=shapes, dtypes=dtypes)
+    fill = cap - 5 * npush - 2  # not full: the row count changes during the replays, then the ring wraps
+    done = 0
+    while done < fill:
+        n = min(500_000, fill - done)
+        rows = random_rows(rng, n, shapes, dtypes)
+        g.insert(*to_dev(rows)), c.push(rows, n)
+        done += n
+    g.set_option("device_counters", 1)
+    new_rows = [torch.zeros((npush,) + tuple(s), dtype=t).cuda() for s, t in zip(shapes, torch_types(dtypes))]
+    pr_dev = torch.ones(batch, dtype=torch.float32, device="cuda")
+    out = (torch.empty(batch, dtype=torch.int64, device="cuda"), torch.empty(batch, dtype=torch.float32, device="cuda"),
+           g._layout.empty(batch, g._dev))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        g.sample(0.5, out=out)
+        g.update_priorities_and_insert(out[0], pr_dev, *new_rows)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for rep in range(10):
+        fresh = random_rows(rng, npush, shapes, dtypes)
+        pr = (rng.pareto(1.5, batch) + 1e-6).astype(np.float32)
+        for dst, src in zip(new_rows, fresh):
+            dst.copy_(torch.from_numpy(src))
+        pr_dev.copy_(torch.from_numpy(pr))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = c.sample(batch, 0.5)
+        assert_sample_equal((out[0], out[1]) + tuple(out[2]), want, "cap %d replay %d" % (cap, rep))
+        c.update(want[0], pr)
+        c.push(fresh, npush)
+        assert_tree_equal(g, c, "cap %d replay %d" % (cap, rep))
+        assert g.size() == c.size and g._state()[1] == c.head, "cap %d replay %d" % (cap, rep)
+        assert np.float32(g.max_priority) == np.float32(c.max_priority)
+        if rep % 4 == 2:  # eager calls in between
+            extra = random_rows(rng, 3, shapes, dtypes)
+            g.insert(*to_dev(extra)), c.push(extra, 3)
+            one = random_rows(rng, 1, shapes, dtypes)
+            g.insert(*to_dev(one)), c.push(one, 1)
+            assert_sample_equal(g.sample(0.9), c.sample(batch, 0.9), "eager after replay %d" % rep)
+    for f, (a, b) in enumerate(zip(g.storage(), [c.field(i) for i in range(len(shapes))])):
+        assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8)), f
+    g.set_option("device_counters", 0)
+    assert g.size() == c.size
+    del graph
+    g.destroy()
