@@ -1653,9 +1653,13 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, unsign
     // A push that does not wrap changed the nodes above one run of slots only: above the leaf level, the
     // tiles outside that run hold what they held, and the waves they would occupy stay out of the way.
     uint32_t t_lo = 0, t_hi = tiles - 1;
-    if (!a.indices && !a.full_top && top != a.depth && a.first_slot >= 0 && a.first_slot + a.n <= a.capacity) {
-        t_lo = (uint32_t)(a.first_slot >> (a.depth - top)) / kBlockNodes;
-        t_hi = (uint32_t)((a.first_slot + a.n - 1) >> (a.depth - top)) / kBlockNodes;
+    if (!a.indices && !a.full_top && top != a.depth) {
+        // (the slots' start: an argument, or read from the device - the leaf tiles' waves have just read it)
+        const int64_t first_slot = a.first_slot >= 0 ? a.first_slot : ring_position(counters_behind(a.err), a.capacity);
+        if (first_slot + a.n <= a.capacity) {
+            t_lo = (uint32_t)(first_slot >> (a.depth - top)) / kBlockNodes;
+            t_hi = (uint32_t)((first_slot + a.n - 1) >> (a.depth - top)) / kBlockNodes;
+        }
     }
     if (top != a.depth && g1 == kRoundLevels) {
         // full tiles above the leaf level: nothing to elect, no clean blocks - the nodes and their eight levels
