@@ -61,6 +61,9 @@ def parse():
     p.add_argument("--graph", action="store_true", help="replay the timed steps as one captured HIP graph")
     p.add_argument("--row-split", type=int, default=0, help="workgroups per sampled row (0 = library default)")
     p.add_argument("--sample-path", type=int, default=0, help="0 auto, 1 wide-row kernel, 2 LDS-top kernel")
+    p.add_argument("--packed-rows", type=int, default=0,
+                   help="keep rows of at most this many bytes packed in one array (library option packed_rows; 0 = "
+                        "one array per field, the reference's layout)")
     p.add_argument("--no-extras", action="store_true",
                    help="skip the untimed side figures (update, insert, loop, graph replay, several streams)")
     p.add_argument("--settle-ms", type=float, default=300.0,
@@ -248,7 +251,11 @@ class PerRun:
         self.loop_step = a.workload == "c1"  # config 1's step is the whole loop, the others time sample()
         self.seed = 1000 + int(a.workload[1])
         self.buf = PriorityReplayBuffer(0.6, self.capacity, self.batch, self.shapes,
-                                        [getattr(torch, d) for d in self.np_dtypes], seed0=self.seed)
+                                        [getattr(torch, d) for d in self.np_dtypes], seed0=self.seed,
+                                        packed_rows=a.packed_rows)
+        if a.packed_rows:
+            packed = not self.buf.storage()[0].is_contiguous()
+            self.desc += " [rows packed in one array]" if packed else " [packed rows asked for, row too wide]"
         self.buf.set_option("row_split", a.row_split)
         self.buf.set_option("sample_path", a.sample_path)
         t0 = time.perf_counter()
@@ -335,7 +342,7 @@ def bench_per(a):
 
     r = PerRun(a, torch)
     K, W, batch = r.K, r.W, r.batch
-    defaults = not (a.capacity or a.row_split or a.sample_path or a.graph)
+    defaults = not (a.capacity or a.row_split or a.sample_path or a.graph or a.packed_rows)
     r.bind_sample_calls()
     step = r.loop_bound if r.loop_step else r.sample_bound
     settle_calls = 0
@@ -660,7 +667,8 @@ def bench_uniform(a):
 
     capacity, batch = (a.capacity or 1_000_000), 256
     shapes, np_dtypes = [(17,), (6,), (1,), (17,), (1,)], ["float32", "float32", "float32", "float32", "bool"]
-    buf = UniformReplayBuffer(batch, capacity, shapes, [getattr(torch, d) for d in np_dtypes], seed=1002)
+    buf = UniformReplayBuffer(batch, capacity, shapes, [getattr(torch, d) for d in np_dtypes], seed=1002,
+                              packed_rows=a.packed_rows)
     gen = torch.Generator(device="cuda").manual_seed(1002)
     chunk = 1000
     src = [torch.randn((chunk,) + s, device="cuda", generator=gen) if d != "bool"

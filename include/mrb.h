@@ -76,7 +76,8 @@ int mrb_backend(void);
 /* ABI version of this header: the library returns the MRB_ABI_VERSION it was built with; a binding
  * compares the two before it makes any other call. History: 1 = mrb_set_option(name, value);
  * 2 = mrb_set_option(handle, name, value), mrb_per_sample_many / _next / _update_noalloc added;
- * 3 = mrb_per_update_push and mrb_bench_launch added, updates of more than 1024 entries refuse stream capture. */
+ * 3 = mrb_per_update_push, mrb_field_layout and mrb_bench_launch added, library-wide options (handle 0), updates
+ * of more than 1024 entries refuse stream capture. */
 #define MRB_ABI_VERSION 3
 int mrb_version(void);
 /* Tuning knobs of ONE buffer (any kind of handle); they change how its kernels are launched, never a
@@ -101,7 +102,19 @@ int mrb_version(void);
  *   "fused_rebuild" prioritized buffers: 1 (default) = an update of <= 16 entries or a push under <= 16 leaf tiles
  *                  rebuilds the tree in one launch where the tree has one round of levels below its top;
  *                  0 = one launch per round */
+/* Library-wide default, set with handle 0 and taken by buffers created afterwards:
+ *   "packed_rows"  N > 0: a buffer whose packed row - every field at the next multiple of its own copy granule
+ *                  (the largest power of two <= 16 that divides its size), the row padded to the widest granule -
+ *                  takes at most N bytes (N <= 4096) keeps its rows packed in ONE [capacity, packed row] array
+ *                  instead of one [capacity, field_bytes[i]] array per field (the reference's layout,
+ *                  uniform_replay_buffer.py:26-47). A sampled row's fields then share cache lines instead of
+ *                  costing a 128-byte line each; results never differ. 0 (default): one array per field.
+ *                  mrb_field_layout tells where a field lies either way. */
 int mrb_set_option(int64_t h, const char *name, int64_t value);
+/* Where field `field` of buffer `h` (any kind) lies in device memory: row r of the field starts at
+ * *dev_ptr + r * *row_stride (row_stride = field_bytes[field] unless the rows are packed). Backs the `.buffer`
+ * attribute, read directly by callers (mindspore_rl/core/msrl.py:550). Either output may be NULL. */
+int mrb_field_layout(int64_t h, int field, void **dev_ptr, int64_t *row_stride);
 
 /* ---- uniform FIFO ring buffer ----------------------------------------- */
 

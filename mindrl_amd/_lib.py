@@ -23,6 +23,7 @@ SIGNATURES = {
     "mrb_backend": [],
     "mrb_version": [],
     "mrb_set_option": [_i64, C.c_char_p, _i64],
+    "mrb_field_layout": [_i64, _int, _pvp, _pi64],
     "mrb_urb_create": [_i64, _int, _pi64, _pi64],
     "mrb_urb_append": [_i64, _pvp, _i64, _vp],
     "mrb_urb_append_from": [_i64, _i64, _i64, _i64, _vp],

@@ -1,6 +1,7 @@
 """Host-side plumbing shared by both buffer classes: field layout, tensor
 marshalling to device pointers, and views over library-owned storage."""
 import ctypes as C
+import threading
 
 import numpy as np
 import torch
@@ -32,10 +33,10 @@ def stream_ptr():
 class _DeviceView:
     """Exposes library-owned device memory to torch through __cuda_array_interface__."""
 
-    def __init__(self, ptr, shape, typestr, owner):
+    def __init__(self, ptr, shape, typestr, owner, strides=None):
         self.owner = owner  # keeps the buffer object (and so the allocation) alive
         self.__cuda_array_interface__ = {
-            "shape": tuple(shape), "typestr": typestr, "data": (int(ptr), False), "version": 2, "strides": None,
+            "shape": tuple(shape), "typestr": typestr, "data": (int(ptr), False), "version": 2, "strides": strides,
         }
 
 
@@ -45,12 +46,47 @@ _TYPESTR = {
 }
 
 
-def view_of(ptr, shape, dtype, owner, dev):
-    """torch tensor aliasing `ptr` (no copy)."""
+def view_of(ptr, shape, dtype, owner, dev, row_stride=None):
+    """torch tensor aliasing `ptr` (no copy). `row_stride`: bytes from one row (index of the first dimension) to
+    the next, when that is not the row's own size (packed rows: the tensor is then a strided view)."""
+    item = torch.empty((), dtype=dtype).element_size()
+    strides = None
+    if row_stride is not None and row_stride != item * int(np.prod(shape[1:], dtype=np.int64)):
+        inner, acc = [], item
+        for n in reversed(shape[1:]):
+            inner.append(acc)
+            acc *= n
+        strides = (int(row_stride),) + tuple(reversed(inner))
     if dtype == torch.bfloat16:
-        t = torch.as_tensor(_DeviceView(ptr, shape, "<i2", owner), device=dev)
+        t = torch.as_tensor(_DeviceView(ptr, shape, "<i2", owner, strides), device=dev)
         return t.view(torch.bfloat16)
-    return torch.as_tensor(_DeviceView(ptr, shape, _TYPESTR[dtype], owner), device=dev)
+    return torch.as_tensor(_DeviceView(ptr, shape, _TYPESTR[dtype], owner, strides), device=dev)
+
+
+_create_lock = threading.Lock()
+
+
+def create_with_layout(packed_rows, create):
+    """Runs `create()` (a libmrb *_create call) with the library-wide option "packed_rows" set for its duration:
+    False / 0 = every field an array of its own (the reference's layout), True = rows of at most 64 bytes are
+    kept packed, an int = rows of at most that many bytes."""
+    limit = 64 if packed_rows is True else int(packed_rows or 0)
+    with _create_lock:
+        _lib.set_option(0, "packed_rows", limit)
+        try:
+            return create()
+        finally:
+            _lib.set_option(0, "packed_rows", 0)
+
+
+def storage_views(handle, layout, capacity, owner, dev):
+    """One [capacity, *shape_i] tensor per field over the buffer's own memory (strided when rows are packed)."""
+    views = []
+    for i, (s, d) in enumerate(zip(layout.shapes, layout.dtypes)):
+        p, stride = C.c_void_p(), C.c_int64(0)
+        _lib.check(_lib.lib().mrb_field_layout(handle, i, C.byref(p), C.byref(stride)))
+        views.append(view_of(p.value, (capacity,) + s, d, owner, dev, stride.value))
+    return tuple(views)
 
 
 def as_tensor(x):

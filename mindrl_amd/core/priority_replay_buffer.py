@@ -7,8 +7,8 @@ import numpy as np
 import torch
 
 from .. import _lib
-from ._rows import (FieldLayout, device, flat_on_device, get_counters, load_fields, pointers, save_fields,
-                    set_counters, stream_ptr, view_of)
+from ._rows import (FieldLayout, create_with_layout, device, flat_on_device, get_counters, load_fields, pointers,
+                    save_fields, set_counters, storage_views, stream_ptr)
 
 
 class PriorityReplayBuffer:
@@ -29,9 +29,13 @@ class PriorityReplayBuffer:
             one): sample() hands out its result tensors from N preallocated sets in turn, so a call
             allocates nothing; a returned batch is then overwritten by the N-th sample() call after
             it - clone() what must live longer.
+        packed_rows (bool or int): False (default): every field is a [capacity, *shape_i] array of its own, the
+            reference's layout. True (or a byte limit): rows of at most 64 (that many) bytes are kept packed in
+            one array, so that a sampled row's fields share cache lines; storage() then returns strided views.
+            Results never differ.
     """
 
-    def __init__(self, alpha, capacity, sample_size, shapes, types, seed0=0, seed1=0, output_ring=0):
+    def __init__(self, alpha, capacity, sample_size, shapes, types, seed0=0, seed1=0, output_ring=0, packed_rows=False):
         self._dev = device()
         self._layout = FieldLayout(shapes, types)
         self._capacity = int(capacity)
@@ -39,8 +43,8 @@ class PriorityReplayBuffer:
         self._alpha = float(alpha)
         seed = int(seed1) or int(seed0) or int.from_bytes(os.urandom(8), "little")
         h = C.c_int64(0)
-        _lib.check(_lib.lib().mrb_per_create(self._capacity, self._alpha, len(self._layout), self._layout.c_bytes,
-                                             seed & (2**64 - 1), C.byref(h)))
+        create_with_layout(packed_rows, lambda: _lib.check(_lib.lib().mrb_per_create(
+            self._capacity, self._alpha, len(self._layout), self._layout.c_bytes, seed & (2**64 - 1), C.byref(h))))
         self._h = h.value
         self._handle = torch.tensor([self._h], dtype=torch.int64)
         self._keep = None
@@ -264,12 +268,7 @@ class PriorityReplayBuffer:
 
     def storage(self):
         """Views of the row storage, one [capacity, *shape_i] tensor per field."""
-        views = []
-        for i, (s, d) in enumerate(zip(self._layout.shapes, self._layout.dtypes)):
-            p = C.c_void_p()
-            _lib.check(_lib.lib().mrb_per_field_ptr(self._h, i, C.byref(p)))
-            views.append(view_of(p.value, (self._capacity,) + s, d, self, self._dev))
-        return tuple(views)
+        return storage_views(self._h, self._layout, self._capacity, self, self._dev)
 
     def state_dict(self):
         """Everything needed to rebuild this buffer: rows, the leaves of the sum tree (internal nodes

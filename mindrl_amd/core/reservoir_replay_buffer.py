@@ -6,8 +6,8 @@ import os
 import torch
 
 from .. import _lib
-from ._rows import (FieldLayout, device, get_counters, load_fields, pointers, save_fields, set_counters, stream_ptr,
-                    view_of)
+from ._rows import (FieldLayout, create_with_layout, device, get_counters, load_fields, pointers, save_fields,
+                    set_counters, storage_views, stream_ptr)
 
 
 class ReservoirReplayBuffer:
@@ -24,15 +24,16 @@ class ReservoirReplayBuffer:
         seed0, seed1 (int): generator seed; seed1 if non-zero, else seed0, else entropy.
     """
 
-    def __init__(self, capacity, sample_size, shapes, dtypes, seed0=0, seed1=0):
+    def __init__(self, capacity, sample_size, shapes, dtypes, seed0=0, seed1=0, packed_rows=False):
         self._dev = device()
         self._layout = FieldLayout(shapes, dtypes)
         self._capacity = int(capacity)
         self._sample_size = int(sample_size)
         seed = int(seed1) or int(seed0) or int.from_bytes(os.urandom(8), "little")
         h = C.c_int64(0)
-        _lib.check(_lib.lib().mrb_res_create(self._capacity, len(self._layout), self._layout.c_bytes,
-                                             seed & (2**64 - 1), C.byref(h)))
+        # packed_rows: as in UniformReplayBuffer (rows of at most 64 bytes, or the given limit, in one array)
+        create_with_layout(packed_rows, lambda: _lib.check(_lib.lib().mrb_res_create(
+            self._capacity, len(self._layout), self._layout.c_bytes, seed & (2**64 - 1), C.byref(h))))
         self._h = h.value
         self._handle = torch.tensor([self._h], dtype=torch.int64)
         self._keep = None
@@ -95,12 +96,7 @@ class ReservoirReplayBuffer:
 
     def storage(self):
         """Views of the row storage, one [capacity, *shape_i] tensor per field."""
-        views = []
-        for i, (s, d) in enumerate(zip(self._layout.shapes, self._layout.dtypes)):
-            p = C.c_void_p()
-            _lib.check(_lib.lib().mrb_res_field_ptr(self._h, i, C.byref(p)))
-            views.append(view_of(p.value, (self._capacity,) + s, d, self, self._dev))
-        return tuple(views)
+        return storage_views(self._h, self._layout, self._capacity, self, self._dev)
 
     def set_option(self, name, value):
         """Sets a launch option of this buffer ("row_split"; prioritized buffers also "sample_path",

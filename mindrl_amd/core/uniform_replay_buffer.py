@@ -6,8 +6,8 @@ import numpy as np
 import torch
 
 from .. import _lib
-from ._rows import (FieldLayout, device, get_counters, load_fields, pointers, save_fields, set_counters, stream_ptr,
-                    view_of)
+from ._rows import (FieldLayout, create_with_layout, device, get_counters, load_fields, pointers, save_fields,
+                    set_counters, storage_views, stream_ptr)
 
 
 class _BufferAppend:
@@ -58,23 +58,22 @@ class UniformReplayBuffer:
         capacity (int): number of rows kept; the oldest row is overwritten when full.
         shapes (list[tuple]): shape of each tensor of an element.
         types (list): element type of each tensor (torch / numpy dtype or name).
+        packed_rows (bool or int): False (default): every field is a [capacity, *shape_i] array of its own, the
+            reference's layout. True (or a byte limit): rows of at most 64 (that many) bytes are kept packed in
+            one array; `.buffer` then holds strided views of the same shapes. Results never differ.
     """
 
-    def __init__(self, sample_size, capacity, shapes, types, seed=0):
+    def __init__(self, sample_size, capacity, shapes, types, seed=0, packed_rows=False):
         self._dev = device()
         self._layout = FieldLayout(shapes, types)
         self._capacity = int(capacity)
         self._sample_size = int(sample_size)
         h = C.c_int64(0)
-        _lib.check(_lib.lib().mrb_urb_create(self._capacity, len(self._layout), self._layout.c_bytes, C.byref(h)))
+        create_with_layout(packed_rows, lambda: _lib.check(_lib.lib().mrb_urb_create(
+            self._capacity, len(self._layout), self._layout.c_bytes, C.byref(h))))
         self._h = h.value
         _lib.check(_lib.lib().mrb_urb_seed(self._h, int(seed) & (2**64 - 1)))
-        views = []
-        for i, (s, d) in enumerate(zip(self._layout.shapes, self._layout.dtypes)):
-            p = C.c_void_p()
-            _lib.check(_lib.lib().mrb_urb_field_ptr(self._h, i, C.byref(p)))
-            views.append(view_of(p.value, (self._capacity,) + s, d, self, self._dev))
-        self.buffer = tuple(views)
+        self.buffer = storage_views(self._h, self._layout, self._capacity, self, self._dev)
         # Attributes that subclasses and callers of the reference class reach into: the append and sample
         # primitives (mindspore_rl/algorithm/mappo/mappo_replaybuffer.py:43 calls
         # `self.buffer_append(self.buffer, exp, self.count, self.head)`;

@@ -4,6 +4,7 @@
 // entry point that touches a buffer fails with MRB_EHIP.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cfloat>
 #include <cstdarg>
 #include <cstdio>
@@ -41,22 +42,35 @@ int fail(int code, const char* fmt, ...) {
         if (e_ != hipSuccess) return fail(MRB_EHIP, "launch %s: %s", name, hipGetErrorString(e_)); \
     } while (0)
 
-// Row storage: structure of arrays, field i = [capacity, bytes_i]
-// (reference layout: mindspore_rl/core/uniform_replay_buffer.py:26-47).
+// Row storage. By default a structure of arrays, field i = [capacity, bytes_i] (reference layout:
+// mindspore_rl/core/uniform_replay_buffer.py:26-47). With the library option "packed_rows" narrow rows are kept
+// packed instead: one [capacity, row_stride] allocation, field i at byte offset_i of every row (each field
+// aligned to its own copy granule), so that a sampled row's fields share cache lines instead of costing one
+// 128-byte line per field. Either way row r of field i starts at data[i] + r * stride[i].
 struct RowStore {
     int64_t capacity = 0;
     int nfields = 0;
     int64_t bytes[MRB_MAX_FIELDS] = {};
+    int64_t stride[MRB_MAX_FIELDS] = {};
     uint8_t* data[MRB_MAX_FIELDS] = {};
+    uint8_t* packed_base = nullptr;  // packed rows: the one allocation (data[i] point into it)
     uint32_t vec_log2[MRB_MAX_FIELDS] = {};
     uint32_t units[MRB_MAX_FIELDS] = {};
     int64_t row_split = 0;  // option "row_split": least number of workgroups per row in the wide-row kernel (0 = auto)
 
     ~RowStore() {
+        if (packed_base) {
+            (void)hipFree(packed_base);
+            return;
+        }
         for (int i = 0; i < nfields; ++i)
             if (data[i]) (void)hipFree(data[i]);
     }
 };
+
+// Library-wide default of the option "packed_rows" (mrb_set_option with handle 0): buffers created afterwards
+// keep their rows packed when a packed row takes at most this many bytes; 0 = every field an array of its own.
+std::atomic<int64_t> g_packed_rows{0};
 
 int rows_alloc(RowStore& r, int64_t capacity, int nfields, const int64_t* field_bytes) {
     if (capacity <= 0 || capacity > (1ll << 30)) return fail(MRB_EINVAL, "capacity %lld outside [1, 2^30]", (long long)capacity);
@@ -66,15 +80,36 @@ int rows_alloc(RowStore& r, int64_t capacity, int nfields, const int64_t* field_
         if (field_bytes[i] <= 0 || field_bytes[i] > (1ll << 30))
             return fail(MRB_EINVAL, "field_bytes[%d] = %lld outside [1, 2^30]", i, (long long)field_bytes[i]);
     r.capacity = capacity;
+    int64_t offset[MRB_MAX_FIELDS], end = 0, widest = 1;
     for (int i = 0; i < nfields; ++i) {
         r.bytes[i] = field_bytes[i];
         uint32_t vl = 4;
         while (vl > 0 && (field_bytes[i] & ((1ll << vl) - 1))) --vl;
         r.vec_log2[i] = vl;
         r.units[i] = (uint32_t)(field_bytes[i] >> vl);
+        // where the field would lie in a packed row: at the next multiple of its own copy granule
+        const int64_t g = 1ll << vl;
+        offset[i] = (end + g - 1) / g * g;
+        end = offset[i] + field_bytes[i];
+        if (g > widest) widest = g;
+    }
+    const int64_t packed_row = (end + widest - 1) / widest * widest;  // rows start at multiples of the widest granule
+    if (nfields > 1 && packed_row <= g_packed_rows.load()) {
+        const size_t total = (size_t)capacity * (size_t)packed_row;
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&r.packed_base), total));
+        HIP_TRY(hipMemset(r.packed_base, 0, total));
+        for (int i = 0; i < nfields; ++i) {
+            r.data[i] = r.packed_base + offset[i];
+            r.stride[i] = packed_row;
+        }
+        r.nfields = nfields;
+        return MRB_OK;
+    }
+    for (int i = 0; i < nfields; ++i) {
         const size_t total = (size_t)capacity * (size_t)field_bytes[i];
         HIP_TRY(hipMalloc(reinterpret_cast<void**>(&r.data[i]), total));
         r.nfields = i + 1;  // so the destructor frees what exists
+        r.stride[i] = field_bytes[i];
         HIP_TRY(hipMemset(r.data[i], 0, total));
     }
     return MRB_OK;
@@ -92,6 +127,7 @@ int make_table(const RowStore& r, const void* const* io, int64_t n, IoTable& t) 
         t.store[i] = r.data[i];
         t.io[i] = const_cast<uint8_t*>(static_cast<const uint8_t*>(io[i]));
         t.row_bytes[i] = (uint32_t)r.bytes[i];
+        t.stride[i] = (uint32_t)r.stride[i];
         t.units[i] = r.units[i];
         t.vec_log2[i] = r.vec_log2[i];
         t.prefix[i + 1] = t.prefix[i] + (uint64_t)n * r.units[i];
@@ -159,6 +195,7 @@ int wide_plan(const RowStore& r, const IoTable& t, int64_t n, WidePlan& plan, di
         plan.f[q].src = t.store[i];
         plan.f[q].dst = t.io[i];
         plan.f[q].rb = t.row_bytes[i];
+        plan.f[q].ss = t.stride[i];
         uint32_t& items = wide ? plan.wide_items : plan.narrow_items;
         plan.f[q].first = items;
         items += wide ? r.units[i] : t.row_bytes[i];
@@ -242,6 +279,8 @@ int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, int64_
         nx.plan.f[0].src = r.data[f];
         nx.plan.f[0].dst = static_cast<uint8_t*>(next->out);
         nx.plan.f[0].rb = (uint32_t)r.bytes[f];
+        nx.plan.f[0].ss = (uint32_t)r.stride[f];
+        nx.slot_stride = (uint32_t)r.stride[next->slot_field];
         nx.plan.wide_items = r.units[f];
         const uint32_t per_wg = (uint32_t)kMaxInFlight * kCopyThreads;
         const uint32_t split = (nx.plan.wide_items + per_wg - 1) / per_wg;
@@ -713,6 +752,13 @@ int mrb_version(void) { return MRB_ABI_VERSION; }
 
 int mrb_set_option(int64_t h, const char* name, int64_t value) {
     if (!name) return fail(MRB_EINVAL, "option name is NULL");
+    if (h == 0) {
+        // library-wide defaults, taken by buffers created afterwards
+        if (strcmp(name, "packed_rows")) return fail(MRB_EINVAL, "'%s' is not a library-wide option (handle 0)", name);
+        if (value < 0 || value > 4096) return fail(MRB_EINVAL, "packed_rows must be in [0, 4096] bytes");
+        g_packed_rows.store(value);
+        return MRB_OK;
+    }
     RowStore* rows = nullptr;
     std::shared_ptr<Per> per = find_per(h);
     std::shared_ptr<Urb> urb = per ? nullptr : find_urb(h);
@@ -752,6 +798,21 @@ int mrb_set_option(int64_t h, const char* name, int64_t value) {
     } else {
         return fail(MRB_EINVAL, "unknown option '%s'", name);
     }
+    return MRB_OK;
+}
+
+int mrb_field_layout(int64_t h, int field, void** dev_ptr, int64_t* row_stride) {
+    const RowStore* rows = nullptr;
+    std::shared_ptr<Per> per = find_per(h);
+    std::shared_ptr<Urb> urb = per ? nullptr : find_urb(h);
+    std::shared_ptr<Res> res = (per || urb) ? nullptr : find_res(h);
+    if (per) rows = &per->rows;
+    if (urb) rows = &urb->rows;
+    if (res) rows = &res->rows;
+    if (!rows) return fail(MRB_EHANDLE, "unknown buffer handle %lld", (long long)h);
+    if (field < 0 || field >= rows->nfields) return fail(MRB_EINVAL, "bad field %d", field);
+    if (dev_ptr) *dev_ptr = rows->data[field];
+    if (row_stride) *row_stride = rows->stride[field];
     return MRB_OK;
 }
 
@@ -820,7 +881,8 @@ int mrb_urb_append_from(int64_t h, int64_t src, int64_t first_logical, int64_t n
                     (long long)(first_logical + n), (long long)from->count);
     if (from->rows.nfields != b->rows.nfields) return fail(MRB_EINVAL, "buffers differ in their fields");
     for (int i = 0; i < b->rows.nfields; ++i)
-        if (from->rows.bytes[i] != b->rows.bytes[i]) return fail(MRB_EINVAL, "buffers differ in field %d", i);
+        if (from->rows.bytes[i] != b->rows.bytes[i] || from->rows.stride[i] != b->rows.stride[i])
+            return fail(MRB_EINVAL, "buffers differ in field %d (size or row layout)", i);
     const int64_t cap = b->rows.capacity;
     // source slot of the first row: logical -> physical as in get_item
     const int64_t t0 = from->count - from->head;

@@ -17,13 +17,16 @@ constexpr int kBlockNodes = 256;  // nodes per wave tile in k_tree_update (float
 constexpr int kTopMaxDepth = 12;  // deepest level k_tree_top normally starts from (4096 nodes)
 
 // Per-call table of the fields of a row, passed to kernels by value.
-// `store` is the buffer's [capacity, row_bytes] matrix, `io` the caller's
-// contiguous [n, row_bytes] matrix (source of an append, destination of a gather).
+// `store` is the field's place in the buffer - row r of the field at store + r * stride: a [capacity, row_bytes]
+// matrix of its own, or a column of the packed rows -, `io` the caller's contiguous [n, row_bytes] matrix
+// (source of an append, destination of a gather).
 struct IoTable {
     int nfields;
     uint8_t* store[MRB_MAX_FIELDS];
     uint8_t* io[MRB_MAX_FIELDS];
     uint32_t row_bytes[MRB_MAX_FIELDS];
+    uint32_t stride[MRB_MAX_FIELDS];    // bytes from one row of the field to the next in `store`: row_bytes when every
+                                        // field has an array of its own, the packed row's size when rows are packed
     uint32_t units[MRB_MAX_FIELDS];     // row_bytes >> vec_log2
     uint32_t vec_log2[MRB_MAX_FIELDS];  // copy granule: 16, 8, 4, 2 or 1 bytes
     uint64_t prefix[MRB_MAX_FIELDS + 1];  // running sum of n * units over fields
@@ -189,8 +192,9 @@ __device__ __forceinline__ void rows_put_part(const PutArgs& p, uint32_t block, 
         }
         const uint32_t vl = t.vec_log2[f];
         const uint64_t off = (uint64_t)unit << vl;
-        copy_granule(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f] + off,
-                     as_global(t.io[f]) + src_row * t.row_bytes[f] + off, vl);
+        // (a source that is itself a ring is another buffer's storage, laid out like this one's)
+        copy_granule(as_global(t.store[f]) + (uint64_t)slot * t.stride[f] + off,
+                     as_global(t.io[f]) + src_row * (p.src_capacity > 0 ? t.stride[f] : t.row_bytes[f]) + off, vl);
     }
 }
 
@@ -224,7 +228,7 @@ __global__ __launch_bounds__(kWG) void k_rows_gather(IoTable t, int64_t capacity
         if (out_indices && f == 0 && unit == 0) out_indices[row] = slot;
         const uint32_t vl = t.vec_log2[f];
         const uint64_t off = (uint64_t)unit << vl;
-        copy_granule(as_global(t.io[f]) + row * t.row_bytes[f] + off, as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f] + off, vl);
+        copy_granule(as_global(t.io[f]) + row * t.row_bytes[f] + off, as_global(t.store[f]) + (uint64_t)slot * t.stride[f] + off, vl);
     }
 }
 
@@ -266,7 +270,7 @@ __global__ __launch_bounds__(kWG) void k_res_put(IoTable t, const unsigned long 
         if (stamp && stamp[slot] != (((unsigned long long)epoch << 32) | row)) continue;
         const uint32_t vl = t.vec_log2[f];
         const uint64_t off = (uint64_t)unit << vl;
-        copy_granule(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f] + off,
+        copy_granule(as_global(t.store[f]) + (uint64_t)slot * t.stride[f] + off,
                      as_global(t.io[f]) + row * t.row_bytes[f] + off, vl);
     }
 }
@@ -345,11 +349,12 @@ __device__ __forceinline__ void sample_flags(const SampleArgs& a, float total, i
 // what the caller reads next).
 // ---------------------------------------------------------------------------
 struct WideField {  // one table entry, 32 bytes
-    const uint8_t* src;  // storage [capacity, row_bytes]
+    const uint8_t* src;  // the field's place in the buffer: row r at src + r * ss
     uint8_t* dst;        // the caller's [batch, row_bytes] matrix
     uint32_t rb;         // row_bytes
     uint32_t first;      // wide field: number of its first granule among the wide ones; narrow: of its first byte
-    uint32_t pad[2];
+    uint32_t ss;         // bytes from one row to the next in the buffer (row_bytes, or the packed row's size)
+    uint32_t pad;
 };
 struct WidePlan {
     int split;              // workgroups per row
@@ -397,11 +402,11 @@ __device__ __forceinline__ uint64_t lane_u64(uint64_t x, int src_lane) {
 struct NarrowWork {
     const gbyte* base[kNarrowInF];
     gbyte* dst[kNarrowInF];
-    uint32_t rb[kNarrowInF];
+    uint32_t rb[kNarrowInF];  // the byte's field: bytes from one row to the next in the buffer
     uint32_t live;  // bit j: position j holds a byte
     // the table entry of field `lane` (lanes 0 .. MRB_MAX_FIELDS - 1), kept for bytes past the first ones
     uint64_t e_src, e_dst;
-    uint32_t e_rb, e_first;
+    uint32_t e_rb, e_first, e_ss;
 
     // Lane q fetches table entry q, needed or not: the address depends on nothing loaded, so the
     // table costs one round trip. Each lane then finds its bytes' fields from the entries held by
@@ -412,6 +417,7 @@ struct NarrowWork {
         e_dst = (uint64_t)e.dst + (uint64_t)k * e.rb;
         e_rb = e.rb;
         e_first = e.first;
+        e_ss = e.ss;
         live = 0;
 #pragma unroll
         for (int j = 0; j < kNarrowInF; ++j) {
@@ -422,14 +428,14 @@ struct NarrowWork {
         }
         for (int q = plan.nwide; q < plan.nwide + plan.nnarrow; ++q) {
             const uint64_t src_q = lane_u64(e_src, q), dst_q = lane_u64(e_dst, q);
-            const uint32_t rb_q = lane_u32(e_rb, q), first_q = lane_u32(e_first, q);
+            const uint32_t rb_q = lane_u32(e_rb, q), first_q = lane_u32(e_first, q), ss_q = lane_u32(e_ss, q);
 #pragma unroll
             for (int j = 0; j < kNarrowInF; ++j) {
                 const uint32_t rel = ((live >> j) & 1u ? lane + 64 * j : 0u) - first_q;  // wraps for bytes of earlier fields
                 if (rel < rb_q) {
                     base[j] = (const gbyte*)(src_q + rel);
                     dst[j] = (gbyte*)(dst_q + rel);
-                    rb[j] = rb_q;
+                    rb[j] = ss_q;
                 }
             }
         }
@@ -444,7 +450,7 @@ struct NarrowWork {
             if (live & (1u << j)) *dst[j] = held[j];
         if (plan.narrow_items > 64u * kNarrowInF) {  // wave-uniform; rows with many narrow bytes
             for (int q = plan.nwide; q < plan.nwide + plan.nnarrow; ++q) {
-                const uint64_t src_q = lane_u64(e_src, q) + (uint64_t)slot * lane_u32(e_rb, q), dst_q = lane_u64(e_dst, q);
+                const uint64_t src_q = lane_u64(e_src, q) + (uint64_t)slot * lane_u32(e_ss, q), dst_q = lane_u64(e_dst, q);
                 const uint32_t rb_q = lane_u32(e_rb, q), first_q = lane_u32(e_first, q);
                 // bytes of this field numbered 64 * kNarrowInF or more among the narrow bytes
                 uint32_t rel = (first_q >= 64u * kNarrowInF ? 0u : 64u * kNarrowInF - first_q) + lane;
@@ -465,9 +471,9 @@ template <int kInF, bool kOneWide>
 struct CopyWork {
     const gbyte* base[kOneWide ? 1 : kInF];  // general: field storage + offset of the granule within a row
     g16* dst[kOneWide ? 1 : kInF];
-    uint32_t rb[kOneWide ? 1 : kInF];
+    uint32_t rb[kOneWide ? 1 : kInF];        // general: bytes from one row to the next in the buffer
     uint32_t off[kOneWide ? kInF : 1];       // one wide field: byte offset of the granule within a row
-    const uint8_t* src0;                     // one wide field: storage, destination row, row size (wave-uniform)
+    const uint8_t* src0;                     // one wide field: storage, destination row, storage row stride (wave-uniform)
     uint8_t* dst0;
     uint32_t rb0;
     uint32_t live;  // bit j: position j holds a granule of this workgroup
@@ -487,7 +493,7 @@ struct CopyWork {
         if (kOneWide) {
             const WideField e = plan.f[0];
             src0 = e.src;
-            rb0 = e.rb;
+            rb0 = e.ss;
             dst0 = e.dst + (uint64_t)k * e.rb;
 #pragma unroll
             for (int j = 0; j < kInF; ++j) off[j] = it[j] << 4;
@@ -510,7 +516,7 @@ struct CopyWork {
                 if (rel < units) {
                     base[j] = s + ((uint64_t)rel << 4);
                     dst[j] = (g16*)(d + ((uint64_t)rel << 4));
-                    rb[j] = e.rb;
+                    rb[j] = e.ss;
                 }
             }
         };
@@ -563,7 +569,8 @@ struct CopyWork {
 // the slot number from the sampled row, and its copy waves copy that field's row; one launch then pays the
 // launch and the descent for twice the bytes.
 struct NextPlan {
-    const uint8_t* slot_field;  // storage of the 8-byte field that holds the slot number, [capacity, 8]
+    const uint8_t* slot_field;  // the 8-byte field that holds the slot number: row r at slot_field + r * slot_stride
+    uint32_t slot_stride;
     WidePlan plan;              // one wide field: its storage -> the caller's [batch, row_bytes] matrix
 };
 
@@ -582,6 +589,10 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
     const uint8_t* const slot_field = [&]() -> const uint8_t* {
         if constexpr (kNext) return nx.slot_field;
         else return nullptr;
+    }();
+    const uint32_t slot_stride = [&]() -> uint32_t {
+        if constexpr (kNext) return nx.slot_stride;
+        else return 8u;
     }();
     __shared__ int64_t s_idx;
     __shared__ float s_picked, s_total, s_pmin;
@@ -730,7 +741,7 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
             int64_t size = s_tail.size;
             if (size < 0) size = counters_behind(s_tail.err)[kCntSize];
             const int64_t row = idx < (int64_t)capacity ? idx : (int64_t)capacity - 1;
-            int64_t to = *reinterpret_cast<const int64_t*>(slot_field + (uint64_t)row * 8);
+            int64_t to = *reinterpret_cast<const int64_t*>(slot_field + (uint64_t)row * slot_stride);
             if (to < 0 || to >= size) {
                 if (part == 0) atomicOr(s_tail.err, MRB_DERR_INDEX);
                 to = to < 0 ? 0 : (size > 0 ? size - 1 : 0);
@@ -969,7 +980,7 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
 #pragma unroll
         for (int f = 0; f < kOwn; ++f)
             if (f < t.nfields && t.units[f] == 1)
-                own[f].load(as_global(t.store[f]) + (uint64_t)slot * t.row_bytes[f], t.vec_log2[f]);
+                own[f].load(as_global(t.store[f]) + (uint64_t)slot * t.stride[f], t.vec_log2[f]);
         a.out_idx[k] = idx;
         const int64_t size = s_slot[kWG];  // left there by the helper wave before the first barrier
         weight = powf_det(picked / total * (float)size, -beta);
@@ -997,7 +1008,7 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
             split_work(w, units, r, u);
             const uint64_t off = (uint64_t)u << vl;
             copy_granule(as_global(t.io[f]) + (uint64_t)(k0 + (int64_t)r) * t.row_bytes[f] + off,
-                         as_global(t.store[f]) + (uint64_t)s_slot[r] * t.row_bytes[f] + off, vl);
+                         as_global(t.store[f]) + (uint64_t)s_slot[r] * t.stride[f] + off, vl);
         }
     }
 }

@@ -1140,10 +1140,10 @@ def test_randomised_differential(mrb, orc, seed):
 
 
 @pytest.mark.parametrize("path", [1, 2])
-def test_sixteen_fields_of_odd_sizes(mrb, orc, path):
+def test_sixteen_fields_of_odd_sizes(mrb, orc, path, sizes=(1, 2, 3, 4, 6, 8, 12, 16, 20, 24, 48, 100, 1000, 4096, 4100, 7)):
     """The maximum of 16 fields, row sizes 1..4100 bytes covering every copy granule (1, 2, 4, 8,
     16 bytes) and rows that need several passes per workgroup; all three buffer kinds."""
-    sizes = [1, 2, 3, 4, 6, 8, 12, 16, 20, 24, 48, 100, 1000, 4096, 4100, 7]
+    sizes = list(sizes)
     shapes, dtypes = [(n,) for n in sizes], [np.uint8] * len(sizes)
     shapes[7], dtypes[7] = (4,), np.float32   # 16 bytes
     shapes[9], dtypes[9] = (3,), np.int64     # 24 bytes

@@ -24,7 +24,7 @@ def declared_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = declared_symbols()
-    assert len(names) == 45
+    assert len(names) == 46
     L = _lib.lib()
     for n in names:
         assert hasattr(L, n), "libmrb.so does not export %s" % n
