@@ -72,16 +72,30 @@ def parse():
     return p.parse_args()
 
 
+def kernel_sources_sha16():
+    """First 16 hex digits of the SHA-256 of the library's kernel sources: names the build a profile was taken of."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in ("mrb_device.h", "mrb_kernels.h", "mrb.hip"):
+        with open(os.path.join(ROOT, "mindrl_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def profile_figures(workload):
-    """Figures of the committed rocprofv3 summary of this workload's dominant kernel (lines `key: number`
-    in its "figures" block), or {} if the summary is not there."""
+    """Figures of the committed rocprofv3 summary of this workload's dominant kernel (lines `key: value`
+    in its "figures" block), or {} if the summary is not there or was taken of other kernel sources than the
+    ones in this tree (its `kernel_sources_sha16` line): a stale profile prices nothing."""
     name = PROFILE_OF.get(workload)
     path = os.path.join(ROOT, "profiles", name) if name else None
     if not path or not os.path.exists(path):
         return {}, name
+    text = open(path).read()
+    sha = re.search(r"^\s*kernel_sources_sha16:\s*([0-9a-f]{16})\s*$", text, re.M)
+    if not sha or sha.group(1) != kernel_sources_sha16():
+        return {"stale": True}, name
     out = {}
-    for key, val in re.findall(r"^\s*(rocprof_avg_ns|traffic_bytes_per_launch):\s*([0-9.eE+]+)\s*$",
-                               open(path).read(), re.M):
+    for key, val in re.findall(r"^\s*(rocprof_avg_ns|traffic_bytes_per_launch):\s*([0-9.eE+]+)\s*$", text, re.M):
         out[key] = float(val)
     return out, name
 
@@ -97,6 +111,8 @@ def roofline(kernel, algo_bytes, kern_s, wall_s_per_step, workload, formula, def
          "traffic": fig.get("traffic_bytes_per_launch"), "kernel": kernel, "algorithmic_bytes_per_launch": algo_bytes,
          "algorithmic_bytes": formula, "avg_launch_us": kern_s * 1e6,
          "frac_wall": algo_bytes / wall_s_per_step / 1e9 / HBM_PEAK_GBS, "profile": name}
+    if fig.get("stale"):
+        r["profile_note"] = "the committed profile was taken of other kernel sources: traffic and profiler figures left out"
     if "rocprof_avg_ns" in fig:
         r["rocprof_avg_us"] = fig["rocprof_avg_ns"] * 1e-3
         r["frac_kernel_rocprof"] = algo_bytes / (fig["rocprof_avg_ns"] * 1e-9) / 1e9 / HBM_PEAK_GBS

@@ -224,10 +224,13 @@ uint32_t pack_groups(int depth) {
     return packed;
 }
 
+// Threads of a wide-row workgroup: the walker wave, the copy waves and, where rows have narrow fields, their wave.
+inline uint32_t wide_threads(const WidePlan& plan) { return plan.narrow_items ? (uint32_t)kWideWG : (uint32_t)kWideWG - 64u; }
+
 template <int kInF, bool kTen, bool kOneWide>
 void launch_sample_wide(dim3 grid, const SampleArgs& a, const WidePlan& plan, hipStream_t s) {
     const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
-    hipLaunchKernelGGL((k_per_sample_wide<kInF, kTen, kOneWide>), grid, dim3(kWideWG), 0, s, a.sum, a.uniforms, a.depth,
+    hipLaunchKernelGGL((k_per_sample_wide<kInF, kTen, kOneWide>), grid, dim3(wide_threads(plan)), 0, s, a.sum, a.uniforms, a.depth,
                        pack_groups(a.depth) | ((plan.nbatch - 1) << 20), (int)a.batch, (uint32_t)a.capacity, a.seed,
                        a.calls, tail, plan);
 }
@@ -250,7 +253,7 @@ struct NextRows {
 template <int kInF, bool kTen, bool kOneWide>
 void launch_sample_next(dim3 grid, const SampleArgs& a, const WidePlan& plan, const NextPlan& nx, hipStream_t s) {
     const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
-    hipLaunchKernelGGL((k_per_sample_next<kInF, kTen, kOneWide>), grid, dim3(kWideWG), 0, s, a.sum, a.uniforms, a.depth,
+    hipLaunchKernelGGL((k_per_sample_next<kInF, kTen, kOneWide>), grid, dim3(wide_threads(plan)), 0, s, a.sum, a.uniforms, a.depth,
                        pack_groups(a.depth), (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, tail, plan, nx);
 }
 
@@ -305,10 +308,10 @@ template <int kInF>
 void launch_gather_wide(dim3 grid, const int64_t* indices, int mode, int64_t count, int64_t fixed_slot, uint64_t seed,
                         uint64_t calls, int64_t* out_indices, uint32_t* err, const WidePlan& plan, hipStream_t s) {
     if (plan.nwide == 1)
-        hipLaunchKernelGGL((k_rows_gather_wide<kInF, true>), grid, dim3(kWideWG), 0, s, indices, mode, count, fixed_slot, seed,
+        hipLaunchKernelGGL((k_rows_gather_wide<kInF, true>), grid, dim3(wide_threads(plan)), 0, s, indices, mode, count, fixed_slot, seed,
                            calls, out_indices, err, plan);
     else
-        hipLaunchKernelGGL((k_rows_gather_wide<kInF, false>), grid, dim3(kWideWG), 0, s, indices, mode, count, fixed_slot, seed,
+        hipLaunchKernelGGL((k_rows_gather_wide<kInF, false>), grid, dim3(wide_threads(plan)), 0, s, indices, mode, count, fixed_slot, seed,
                            calls, out_indices, err, plan);
 }
 

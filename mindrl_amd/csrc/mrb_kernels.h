@@ -379,7 +379,8 @@ struct SampleTail {
 
 constexpr int kCopyWaves = 4;
 constexpr int kCopyThreads = 64 * kCopyWaves;
-constexpr int kWideWG = 64 + kCopyThreads;  // the walker wave, then four copy waves
+constexpr int kWideWG = 64 + kCopyThreads + 64;  // the walker wave, four copy waves and, for rows with narrow
+                                                  // fields, a wave that carries those (launched only then)
 constexpr int kMaxInFlight = 8;             // most granules a copy thread holds between its loads and its stores
 constexpr int kFastWide = 2;                // wide fields whose table entries are fetched unconditionally, in one round
 
@@ -394,10 +395,10 @@ __device__ __forceinline__ uint64_t lane_u64(uint64_t x, int src_lane) {
     return ((uint64_t)lane_u32((uint32_t)(x >> 32), src_lane) << 32) | lane_u32((uint32_t)x, src_lane);
 }
 
-// The narrow fields of a row, copied byte by byte by the first copy wave of the row's first
-// workgroup: lane l takes bytes l, l + 64, ... of the narrow fields' bytes, numbered consecutively
-// over the fields; the first kNarrowInF of them are loaded ahead of the wave's wide granules and
-// stored after them. Narrow fields are small (scalars such as action, reward, done); byte
+// The narrow fields of a row, copied byte by byte by a wave of their own in the row's first
+// workgroup (the sixth; a copy wave that also carried them would hold its wide stores back until
+// the narrow loads have arrived: 0.06 us per launch of 512 Atari-shaped rows): lane l takes bytes l,
+// l + 64, ... of the narrow fields' bytes, numbered consecutively over the fields. Narrow fields are small (scalars such as action, reward, done); byte
 // granularity keeps their copy free of branches on a granule size.
 struct NarrowWork {
     const gbyte* base[kNarrowInF];
@@ -489,7 +490,7 @@ struct CopyWork {
             if (it[j] < hi) live |= 1u << j;
             else it[j] = lo;
         }
-        if (lo >= hi) live = 0;
+        if (lo >= hi || tid >= (uint32_t)kCopyThreads) live = 0;  // (a wave past the copy waves carries narrow fields only)
         if (kOneWide) {
             const WideField e = plan.f[0];
             src0 = e.src;
@@ -526,11 +527,11 @@ struct CopyWork {
         for (int q = kFastWide; q < plan.nwide; ++q) take(q);
     }
 
-    // `narrow`: this thread also carries narrow bytes (first copy wave of the row's first workgroup)
+    // `narrow`: this thread carries narrow bytes (the wave after the copy waves, in the row's first workgroup)
     __device__ __forceinline__ void run(uint32_t slot, const WidePlan& plan, bool narrow, const NarrowWork& nw, uint32_t lane) const {
         uint8_t nheld[kNarrowInF];
         granule_t held[kInF];
-        if (narrow) nw.load(slot, nheld);  // ahead of the wide loads in the memory pipeline
+        if (narrow) nw.load(slot, nheld);
         if (live) {
             if (kOneWide) {
                 const gbyte* row = as_global(src0) + (uint64_t)slot * rb0;  // wave-uniform
@@ -713,7 +714,7 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
     // ---- copy waves, while the walker walks
     CopyWork<kInF, kOneWide> work;
     NarrowWork nw;
-    const bool narrow = wave == 1 && part == 0 && plan.narrow_items && !next_layer;
+    const bool narrow = wave == 1 + kCopyWaves && part == 0 && plan.narrow_items && !next_layer;
     if (!walker) {
         if (narrow) nw.prepare(plan, k, lane);
         if (next_layer) work.prepare(plan2, k, part, ctid);
@@ -812,7 +813,7 @@ __global__ __launch_bounds__(kWideWG) void k_rows_gather_wide(const int64_t* __r
     const uint32_t ctid = threadIdx.x - 64;
     CopyWork<kInF, kOneWide> work;
     NarrowWork nw;
-    const bool narrow = wave == 1 && part == 0 && plan.narrow_items;
+    const bool narrow = wave == 1 + kCopyWaves && part == 0 && plan.narrow_items;
     if (walker) {
         if (lane == 0) {
             // out-of-range slots are clamped and flagged (a fixed slot was range-checked by the host
