@@ -518,6 +518,19 @@ uint32_t push_units(const UpdateArgs& a) {
     return (uint32_t)(units < ring_tiles ? units : ring_tiles);
 }
 
+// A push whose tree work is ONE launch and that also moves the device's counters on (a.advance != 0): every
+// workgroup that rides along reports to one counter when it has read the ring position (see counters_push_done),
+// which is worth it for a few dozen workgroups only - a larger copy then gets a launch of its own, ahead.
+constexpr uint32_t kRideWithCounters = 64;
+int ride_alone_if_large(const UpdateArgs& a, PutArgs& put, hipStream_t s) {
+    if (a.advance && put.blocks > kRideWithCounters) {
+        hipLaunchKernelGGL(k_rows_put, dim3(put.blocks), dim3(kWG), 0, s, put);
+        LAUNCH_CHECK("k_rows_put");
+        put.blocks = 0;
+    }
+    return MRB_OK;
+}
+
 // Rebuilds the tree above the leaves that `a` writes: one launch per round, then the top. A push hands
 // its row copy over (`ride`): it is done by extra workgroups of the first launch.
 int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = nullptr) {
@@ -538,6 +551,7 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
         }
         if (units > 0 && units <= (uint32_t)(kFusedWG / 64)) {
             PutArgs put = ride ? *ride : none;
+            if (int rc = ride_alone_if_large(a, put, s)) return rc;
             put.blocks = (put.blocks + 3) / 4;  // the ride-along copy was sized for workgroups a quarter as large
             a.readers = 1 + put.blocks;         // (a.advance != 0: this one launch also moves the device's counters on)
             hipLaunchKernelGGL(k_tree_fused, dim3(1 + put.blocks), dim3(kFusedWG), 0, s, a, tile_base, units, put);
@@ -571,7 +585,8 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
         hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4 + put.blocks), dim3(kWG), 0, s, a, r, tile_base, put);
         LAUNCH_CHECK("k_tree_update");
     }
-    const PutArgs& put = (a.nrounds == 0 && ride) ? *ride : none;
+    PutArgs put = (a.nrounds == 0 && ride) ? *ride : none;
+    if (int rc = ride_alone_if_large(a, put, s)) return rc;
     // the top is the call's last launch: it moves the device's counters on (a.advance != 0); only when it is also
     // the first do its workgroups read the ring position
     a.readers = a.nrounds == 0 ? 1 + put.blocks : 0;
@@ -1134,10 +1149,8 @@ static int per_push(Per* b, const void* const* src_fields, int64_t nrows, const 
         put.first_slot = -1;
         put.src_first = reinterpret_cast<int64_t>(b->counters);
     }
-    // A large copy gets its own launch; a small one rides along in the first tree launch. (With the counters on
-    // the device every workgroup that rides along reports to one counter when it is done - see
-    // counters_push_done -, which is worth it for a few dozen workgroups only.)
-    if (put.blocks > (b->device_counters ? 64u : 2048u)) {
+    // A large copy gets its own launch; a small one rides along in the first tree launch.
+    if (put.blocks > 2048u) {
         hipLaunchKernelGGL(k_rows_put, dim3(put.blocks), dim3(kWG), 0, s, put);
         LAUNCH_CHECK("k_rows_put");
         put.blocks = 0;
@@ -1169,6 +1182,8 @@ static int per_push(Per* b, const void* const* src_fields, int64_t nrows, const 
     const bool stamp_after = opt_priorities && !fold;
     if (!lead && b->fused && nrows == 1 && b->depth <= kPushOneMaxDepth) {
         // one row: one wave walks from its leaf to the root (k_push_one)
+        rc = ride_alone_if_large(a, put, s);
+        if (rc) return rc;
         hipLaunchKernelGGL(k_push_one, dim3(1 + put.blocks), dim3(kWG), 0, s, a.sum, a.mn, a.maxp, a.first_slot, a.capacity,
                            a.leaves, a.depth, a.alpha, opt_priorities, a.err, put, a.advance, 1 + put.blocks);
         LAUNCH_CHECK("k_push_one");
@@ -1264,7 +1279,7 @@ int mrb_per_update_push(int64_t h, const int64_t* indices, const float* prioriti
             put.first_slot = -1;
             put.src_first = reinterpret_cast<int64_t>(b->counters);
         }
-        if (put.blocks <= (b->device_counters ? 64u : 2048u)) {
+        if (put.blocks <= (b->device_counters ? kRideWithCounters : 2048u)) {
             rc = next_epoch(*b, s);
             if (rc) return rc;
             UpdateArgs a = update_args(*b);

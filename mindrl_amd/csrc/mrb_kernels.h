@@ -1180,8 +1180,10 @@ __device__ __forceinline__ void parents_step(const UpdateArgs& a, int g, uint32_
     }
 }
 
+// root_s / root_m (optional): the node eight levels above a full tile, as computed here (what is stored when g >= 8).
 __device__ __forceinline__ void tile_parents(const UpdateArgs& a, int g, uint32_t first, uint32_t lane, bool active,
-                                             const float4& vs, const float4& vm) {
+                                             const float4& vs, const float4& vm, float* root_s = nullptr,
+                                             float* root_m = nullptr) {
     // one level up: two nodes per lane; two levels up: one node per lane
     const float s0 = vs.x + vs.y, s1 = vs.z + vs.w;
     const float m0 = fminf(vm.x, vm.y), m1 = fminf(vm.z, vm.w);
@@ -1210,11 +1212,16 @@ __device__ __forceinline__ void tile_parents(const UpdateArgs& a, int g, uint32_
         a.sum[first >> 8] = s_lo + s_hi;
         a.mn[first >> 8] = fminf(m_lo, m_hi);
     }
+    if (root_s) *root_s = s_lo + s_hi;
+    if (root_m) *root_m = fminf(m_lo, m_hi);
 }
 
+// root_s / root_m / rebuilt (optional, full tiles with g = 8): the tile's root as stored, and whether the tile
+// was rebuilt at all (its one block was dirty).
 __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, uint32_t tile, bool sparse,
                                            const uint32_t* __restrict__ dirty_in, uint32_t* __restrict__ dirty_out,
-                                           int g_next, uint32_t lane, unsigned long long* win = nullptr) {
+                                           int g_next, uint32_t lane, unsigned long long* win = nullptr,
+                                           float* root_s = nullptr, float* root_m = nullptr, bool* rebuilt = nullptr) {
     const uint32_t level_nodes = 1u << lo;
     const bool leaf_level = lo == a.depth;
     // where a push's slots start (a.first_slot, or read from the device)
@@ -1357,7 +1364,8 @@ __device__ __forceinline__ void tile_round(const UpdateArgs& a, int lo, int g, u
         q = wave_max(q);
         if (lane == 0 && q > 0.0f) raise_max(a.maxp_next, q);
     }
-    tile_parents(a, g, first, lane, active, vs, vm);
+    tile_parents(a, g, first, lane, active, vs, vm, root_s, root_m);
+    if (rebuilt) *rebuilt = __any(active);
 }
 
 // ---------------------------------------------------------------------------
@@ -1780,6 +1788,69 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
         return;
     }
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int top = a.top_depth;
+    if (!a.inline_election && a.lo[0] == a.depth && a.g[0] == kRoundLevels && top >= kRoundLevels &&
+        (1u << top) / kBlockNodes <= (uint32_t)(kFusedWG / 64)) {
+        // A push: the top's tiles (one per wave) are requested BEFORE the leaf tiles are rebuilt - of all their
+        // nodes only the leaf tiles' roots change, and those reach the waves that hold them through LDS - so the
+        // call has two dependent trips to memory on its path (leaf tiles and top tiles together, then the last
+        // tile) instead of three.
+        __shared__ uint32_t s_root_tile[kFusedWG / 64];
+        __shared__ float s_root_s[kFusedWG / 64], s_root_m[kFusedWG / 64];
+        const uint32_t tiles = (1u << top) / kBlockNodes;
+        uint32_t t_lo = 0, t_hi = tiles - 1;
+        const int64_t first_slot = a.first_slot >= 0 ? a.first_slot : ring_position(counters_behind(a.err), a.capacity);
+        if (!a.full_top && first_slot + a.n <= a.capacity) {
+            t_lo = (uint32_t)(first_slot >> (a.depth - top)) / kBlockNodes;
+            t_hi = (uint32_t)((first_slot + a.n - 1) >> (a.depth - top)) / kBlockNodes;
+        }
+        const bool mine = wave >= t_lo && wave <= t_hi;  // this wave rebuilds the top's tile number `wave`
+        const uint32_t top_first = (1u << top) + wave * kBlockNodes;
+        float4 tvs = make_float4(0.f, 0.f, 0.f, 0.f), tvm = tvs;
+        if (mine) {
+            tvs = *reinterpret_cast<const float4*>(a.sum + top_first + 4 * lane);
+            tvm = *reinterpret_cast<const float4*>(a.mn + top_first + 4 * lane);
+        }
+        uint32_t leaf_tile = 0xffffffffu;
+        float rs = 0.0f, rm = 0.0f;
+        if (wave < units) {
+            const uint32_t ring_tiles = (uint32_t)((a.capacity + kBlockNodes - 1) / kBlockNodes);  // the ring ends at `capacity`
+            const uint32_t tile = a.first_slot >= 0 ? tile_base + wave
+                                                    : ((uint32_t)(first_slot / kBlockNodes) + wave) % ring_tiles;
+            bool rebuilt = false;
+            tile_round(a, a.depth, kRoundLevels, tile, true, nullptr, nullptr, 0, lane, nullptr, &rs, &rm, &rebuilt);
+            if (rebuilt) leaf_tile = tile;
+        }
+        if (lane == 0) {
+            s_root_tile[wave] = leaf_tile;
+            s_root_s[wave] = rs;
+            s_root_m[wave] = rm;
+        }
+        lds_barrier();
+        if (mine) {
+            for (uint32_t u = 0; u < units; ++u) {  // uniform
+                const uint32_t lt = s_root_tile[u];  // the leaf tile's number = its root's place in the top's level
+                if (lt != 0xffffffffu && lt / kBlockNodes == wave && (lt % kBlockNodes) / 4 == lane) {
+                    const float ps = s_root_s[u], pm = s_root_m[u];
+                    switch (lt & 3u) {
+                        case 0: tvs.x = ps, tvm.x = pm; break;
+                        case 1: tvs.y = ps, tvm.y = pm; break;
+                        case 2: tvs.z = ps, tvm.z = pm; break;
+                        default: tvs.w = ps, tvm.w = pm; break;
+                    }
+                }
+            }
+            tile_parents(a, kRoundLevels, top_first, lane, true, tvs, tvm);
+        }
+        if (top > kRoundLevels) {
+            __threadfence_block();  // the tiles' parents, written by other waves of this workgroup, are read below
+            __syncthreads();
+            if (wave == 0) tile_round(a, top - kRoundLevels, top - kRoundLevels, 0, false, nullptr, nullptr, 0, lane);
+        }
+        if (a.fold_max) fold_push_max(a);
+        counters_push_done(a.err, a.advance, a.capacity, a.readers);
+        return;
+    }
     if (const uint32_t unit = wave; unit < units) {
         if (a.inline_election) {
             entry_tile(a, a.g[0], unit, lane, s_win[wave], nullptr, 0);
