@@ -409,16 +409,26 @@ struct NarrowWork {
     uint64_t e_src, e_dst;
     uint32_t e_rb, e_first, e_ss;
 
-    // Lane q fetches table entry q, needed or not: the address depends on nothing loaded, so the
-    // table costs one round trip. Each lane then finds its bytes' fields from the entries held by
-    // the other lanes (the loops are wave-uniform).
+    // Each lane finds the fields of its bytes from the table's entries. Up to kNarrowFast narrow fields (the
+    // usual few scalars) are read with wave-uniform indices - scalar loads, issued together, from lines of the
+    // kernel-argument segment that the copy waves' own reads bring into the scalar cache. More fields than that:
+    // lane q fetches entry q with one vector load (a round trip of its own through memory, which holds back the
+    // workgroup's barrier when nothing else, such as a tree descent, takes as long) and the entries are read from
+    // the lanes. Rows with more than 64 * kNarrowInF narrow bytes keep the per-lane copy for store().
+    static constexpr int kNarrowFast = 4;
+    __device__ __forceinline__ void take(const WidePlan& plan, int64_t k, uint32_t lane, uint64_t src_q, uint64_t dst_q,
+                                         uint32_t rb_q, uint32_t first_q, uint32_t ss_q) {
+#pragma unroll
+        for (int j = 0; j < kNarrowInF; ++j) {
+            const uint32_t rel = ((live >> j) & 1u ? lane + 64 * j : 0u) - first_q;  // wraps for bytes of earlier fields
+            if (rel < rb_q) {
+                base[j] = (const gbyte*)(src_q + rel);
+                dst[j] = (gbyte*)(dst_q + rel);
+                rb[j] = ss_q;
+            }
+        }
+    }
     __device__ __forceinline__ void prepare(const WidePlan& plan, int64_t k, uint32_t lane) {
-        const WideField e = plan.f[lane < MRB_MAX_FIELDS ? lane : 0];
-        e_src = (uint64_t)e.src;
-        e_dst = (uint64_t)e.dst + (uint64_t)k * e.rb;
-        e_rb = e.rb;
-        e_first = e.first;
-        e_ss = e.ss;
         live = 0;
 #pragma unroll
         for (int j = 0; j < kNarrowInF; ++j) {
@@ -427,19 +437,26 @@ struct NarrowWork {
             rb[j] = 0;
             if (lane + 64 * j < plan.narrow_items) live |= 1u << j;
         }
-        for (int q = plan.nwide; q < plan.nwide + plan.nnarrow; ++q) {
-            const uint64_t src_q = lane_u64(e_src, q), dst_q = lane_u64(e_dst, q);
-            const uint32_t rb_q = lane_u32(e_rb, q), first_q = lane_u32(e_first, q), ss_q = lane_u32(e_ss, q);
+        e_src = e_dst = 0;
+        e_rb = e_first = e_ss = 0;
+        if (plan.nnarrow <= kNarrowFast && plan.narrow_items <= 64u * kNarrowInF) {  // wave-uniform
+            WideField e[kNarrowFast];
 #pragma unroll
-            for (int j = 0; j < kNarrowInF; ++j) {
-                const uint32_t rel = ((live >> j) & 1u ? lane + 64 * j : 0u) - first_q;  // wraps for bytes of earlier fields
-                if (rel < rb_q) {
-                    base[j] = (const gbyte*)(src_q + rel);
-                    dst[j] = (gbyte*)(dst_q + rel);
-                    rb[j] = ss_q;
-                }
-            }
+            for (int i = 0; i < kNarrowFast; ++i) e[i] = plan.f[plan.nwide + (i < plan.nnarrow ? i : 0)];
+#pragma unroll
+            for (int i = 0; i < kNarrowFast; ++i)
+                if (i < plan.nnarrow)
+                    take(plan, k, lane, (uint64_t)e[i].src, (uint64_t)e[i].dst + (uint64_t)k * e[i].rb, e[i].rb, e[i].first, e[i].ss);
+            return;
         }
+        const WideField e = plan.f[lane < MRB_MAX_FIELDS ? lane : 0];
+        e_src = (uint64_t)e.src;
+        e_dst = (uint64_t)e.dst + (uint64_t)k * e.rb;
+        e_rb = e.rb;
+        e_first = e.first;
+        e_ss = e.ss;
+        for (int q = plan.nwide; q < plan.nwide + plan.nnarrow; ++q)
+            take(plan, k, lane, lane_u64(e_src, q), lane_u64(e_dst, q), lane_u32(e_rb, q), lane_u32(e_first, q), lane_u32(e_ss, q));
     }
     __device__ __forceinline__ void load(uint32_t slot, uint8_t (&held)[kNarrowInF]) const {
 #pragma unroll
