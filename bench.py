@@ -462,6 +462,9 @@ def bench_per(a):
         out["extras"] = per_extras(a, torch, r, algo_bytes)
         if a.workload == "c3":
             out["roofline"]["floor"] = sample_floor(torch, r, algo_bytes)
+            # the same kernel with several batches per launch (mrb_per_sample_many): where the 60 % of peak lie
+            many = out["extras"].get("sample_many_batches_per_launch", {})
+            out["roofline"]["frac_with_batches_per_launch"] = {k: round(v["frac_of_peak"], 4) for k, v in many.items()}
     if a.no_cpu_baseline:
         out["cpu_baseline"] = None
     elif r.loop_step:
