@@ -83,6 +83,8 @@ int mrb_version(void);
 /* Tuning knobs of ONE buffer (any kind of handle); they change how its kernels are launched, never a
  * result. Unknown names return MRB_EINVAL. Set them while no call on the handle is in progress.
  *   "row_split"    least number of workgroups per row in the wide-row kernel (0 = auto, max 64)
+ *   "row_wave"     prioritized buffers: the wave-per-row sample kernel (rows of at most 4 KB in 16-byte fields and 256
+ *                  narrow bytes) is taken 0 = for launches of at least 2048 rows, 1 = whenever the rows fit it, 2 = never
  *   "sample_path"  prioritized buffers: 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
  *   "lds_levels"   prioritized buffers: tree levels staged in LDS by the LDS-top kernel (0 = auto, max 12)
  *   "device_counters" prioritized and uniform buffers: 1 = the ring position, the number of stored rows and the generator's

@@ -316,7 +316,7 @@ class PriorityReplayBuffer:
         return f
 
     def set_option(self, name, value):
-        """Sets a launch option of this buffer ("row_split"; prioritized buffers also "sample_path",
+        """Sets a launch option of this buffer ("row_split"; prioritized buffers also "sample_path", "row_wave",
         "lds_levels", "fused_rebuild", "device_counters"). Options change how kernels are launched, never a
         result."""
         _lib.set_option(self._h, name, value)

@@ -57,6 +57,8 @@ struct RowStore {
     uint32_t vec_log2[MRB_MAX_FIELDS] = {};
     uint32_t units[MRB_MAX_FIELDS] = {};
     int64_t row_split = 0;  // option "row_split": least number of workgroups per row in the wide-row kernel (0 = auto)
+    int64_t row_wave = 0;   // option "row_wave": the wave-per-row sample kernel, 0 = for launches of many rows, 1 = whenever
+                            // the rows fit it, 2 = never
 
     ~RowStore() {
         if (packed_base) {
@@ -250,6 +252,8 @@ struct NextRows {
     void* out = nullptr;
 };
 
+constexpr int64_t kRowWaveMinRows = 2048;  // fewest rows of a launch that go to the wave-per-row sample kernel
+
 template <int kInF, bool kTen, bool kOneWide>
 void launch_sample_next(dim3 grid, const SampleArgs& a, const WidePlan& plan, const NextPlan& nx, hipStream_t s) {
     const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
@@ -296,6 +300,26 @@ int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, int64_
         if (inflight == 2 && per_thread <= 2) launch_sample_next_as<2>(grid, a, plan, nx, s);
         else launch_sample_next_as<8>(grid, a, plan, nx, s);
         LAUNCH_CHECK("k_per_sample_next");
+        return MRB_OK;
+    }
+    // Many rows of up to 4 KB in 16-byte fields and a handful of narrow bytes: a wave per row (k_per_sample_rows)
+    // instead of a workgroup per row. One wave does in a row what six do side by side, so a launch of few rows
+    // takes longer that way (config 4, 1024 rows of 521 B: 6.4 us against 5.5) and a launch of many less (4096
+    // rows: 9.2 us against 15.6; 16,384: 26 against 54): a sixth of the waves to dispatch. (`row_split` asks for
+    // the workgroup kernel.)
+    const int64_t nrows = nbatch * a.batch;
+    if (r.row_split == 0 && r.row_wave != 2 && plan.split == 1 && plan.wide_items <= (uint32_t)kRowWaveInF * 64u &&
+        plan.narrow_items <= 256u && (nrows >= kRowWaveMinRows || r.row_wave == 1)) {
+        const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
+        const uint32_t blocks = (uint32_t)((nrows + kRowWaveWG / 64 - 1) / (kRowWaveWG / 64));
+        const uint32_t packed = pack_groups(a.depth) | ((plan.nbatch - 1) << 20);
+        if (a.depth > 0 && a.depth % kGroupMaxLevels == 0)
+            hipLaunchKernelGGL((k_per_sample_rows<true>), dim3(blocks), dim3(kRowWaveWG), 0, s, a.sum, a.uniforms, a.depth, packed,
+                               (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, nrows, tail, plan);
+        else
+            hipLaunchKernelGGL((k_per_sample_rows<false>), dim3(blocks), dim3(kRowWaveWG), 0, s, a.sum, a.uniforms, a.depth, packed,
+                               (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, nrows, tail, plan);
+        LAUNCH_CHECK("k_per_sample_rows");
         return MRB_OK;
     }
     if (inflight == 2) launch_sample_wide_as<2>(grid, a, plan, s);
@@ -788,6 +812,9 @@ int mrb_set_option(int64_t h, const char* name, int64_t value) {
     if (!strcmp(name, "row_split")) {
         if (value < 0 || value > 64) return fail(MRB_EINVAL, "row_split must be in [0, 64]");
         rows->row_split = value;
+    } else if (!strcmp(name, "row_wave")) {
+        if (value < 0 || value > 2) return fail(MRB_EINVAL, "row_wave must be 0, 1 or 2");
+        rows->row_wave = value;
     } else if (!strcmp(name, "sample_path")) {
         if (!per) return fail(MRB_EINVAL, "sample_path is an option of prioritized buffers");
         if (value < 0 || value > 2) return fail(MRB_EINVAL, "sample_path must be 0, 1 or 2");

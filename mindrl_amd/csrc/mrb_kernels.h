@@ -485,7 +485,8 @@ struct NarrowWork {
 // addresses are then a wave-uniform row base plus a 32-bit offset, which costs a tenth of the
 // general path's address arithmetic - work that would otherwise compete with the walker for
 // the SIMD's issue slots.
-template <int kInF, bool kOneWide>
+// kThreads: the threads that share a workgroup's granules (the four copy waves; one wave in k_per_sample_rows).
+template <int kInF, bool kOneWide, int kThreads = kCopyThreads>
 struct CopyWork {
     const gbyte* base[kOneWide ? 1 : kInF];  // general: field storage + offset of the granule within a row
     g16* dst[kOneWide ? 1 : kInF];
@@ -503,11 +504,11 @@ struct CopyWork {
         live = 0;
 #pragma unroll
         for (int j = 0; j < kInF; ++j) {
-            it[j] = lo + j * kCopyThreads + tid;
+            it[j] = lo + j * kThreads + tid;
             if (it[j] < hi) live |= 1u << j;
             else it[j] = lo;
         }
-        if (lo >= hi || tid >= (uint32_t)kCopyThreads) live = 0;  // (a wave past the copy waves carries narrow fields only)
+        if (lo >= hi || tid >= (uint32_t)kThreads) live = 0;  // (a wave past the copy waves carries narrow fields only)
         if (kOneWide) {
             const WideField e = plan.f[0];
             src0 = e.src;
@@ -809,6 +810,101 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_next(const float* __rest
                                                              uint64_t seed, uint64_t calls, SampleTail tail, WidePlan plan,
                                                              NextPlan nx) {
     sample_wide_body<kInF, kTen, kOneWide, true>(sum, uniforms, depth, groups, batch, capacity, seed, calls, tail, plan, nx);
+}
+
+// ---------------------------------------------------------------------------
+// PER sample of rows of up to a few kilobytes (a CartPole or MuJoCo transition, an Ape-X row of 521 bytes): ONE
+// WAVE per sampled row instead of a workgroup of five or six - the wave walks the tree, requests its row, takes
+// the importance weight while the row is on its way, and stores. No LDS, no barrier, a sixth of the waves to
+// dispatch. The walk's first node group is requested before anything else; the field table (kernel arguments,
+// a trip to memory of their own when a kernel starts) is read while that group is on its way. Same outputs,
+// bit for bit, as k_per_sample_wide. Rows of at most kRowWaveInF * 64 wide granules (4 KB in 16-byte fields).
+// ---------------------------------------------------------------------------
+constexpr int kRowWaveInF = 4;
+constexpr int kRowWaveWG = 256;  // four rows per workgroup
+
+template <bool kTen>
+__global__ __launch_bounds__(kRowWaveWG) void k_per_sample_rows(const float* __restrict__ sum, const float* __restrict__ uniforms,
+                                                                int depth, uint32_t groups, int batch, uint32_t capacity,
+                                                                uint64_t seed, uint64_t calls, int64_t nrows, SampleTail tail,
+                                                                WidePlan plan) {
+    const int lane = threadIdx.x & 63;
+    const int64_t k = (int64_t)blockIdx.x * (kRowWaveWG / 64) + (threadIdx.x >> 6);  // output row
+    if (k >= nrows) return;  // wave-uniform
+    uint32_t stratum = (uint32_t)k, nth = 0;
+    if (groups >> 20) {  // several batches in the launch, each stratified on its own
+        nth = (uint32_t)k / (uint32_t)batch;
+        stratum = (uint32_t)k - nth * (uint32_t)batch;
+    }
+    CopyWork<kRowWaveInF, false, 64> work;
+    NarrowWork nw;
+    const bool narrow = plan.narrow_items != 0;
+    const int ngroups = (int)(groups & 15u);
+    uint32_t node = 1;
+    float picked, mass = 0.0f, total;
+    if (depth >= 2) {
+        uint32_t packed = (groups >> 4) & 0x7fffu;
+        int g = kTen ? kGroupMaxLevels : (int)(packed & 31u);
+        f32x4 r0, r1, r2, r3;
+        group_request(sum, 1u, g, lane, r0, r1, r2, r3);
+        total = sum[1];
+        const float u_given = *(uniforms ? uniforms + k : sum + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        // the field table, while the first group is on its way
+        work.prepare(plan, k, 0, (uint32_t)lane);
+        if (narrow) nw.prepare(plan, k, (uint32_t)lane);
+        const float u = uniforms ? u_given : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+        mass = (u + (float)stratum) * (total / (float)batch);  // each operation rounded once
+        node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
+#pragma nounroll
+        for (int i = 1; i < ngroups; ++i) {
+            packed >>= 5;
+            g = kTen ? kGroupMaxLevels : (int)(packed & 31u);
+            group_request(sum, node, g, lane, r0, r1, r2, r3);
+            __builtin_amdgcn_sched_barrier(0);
+            node = (node << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
+        }
+    } else {
+        total = sum[1];
+        const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+        work.prepare(plan, k, 0, (uint32_t)lane);
+        if (narrow) nw.prepare(plan, k, (uint32_t)lane);
+        mass = (u + (float)stratum) * (total / (float)batch);
+        picked = total;
+        node = (1u << depth) + (depth ? group_walk(group_load_tiny(sum, 1u, depth, lane), depth, lane, mass, picked) : 0u);
+    }
+    const int64_t idx = (int64_t)node - ((int64_t)1 << depth);
+    // the descent can end on an unfilled leaf past the last row (flagged below); the copy stays inside the storage
+    const uint32_t slot = (uint32_t)(idx < (int64_t)capacity ? idx : (int64_t)capacity - 1);
+    // the row: every load before the weight's arithmetic, every store after it
+    uint8_t nheld[kNarrowInF];
+    granule_t held[kRowWaveInF];
+    if (narrow) nw.load(slot, nheld);
+    if (work.live) {
+#pragma unroll
+        for (int j = 0; j < kRowWaveInF; ++j) held[j] = __builtin_nontemporal_load((const g16*)(work.base[j] + (uint64_t)slot * work.rb[j]));
+    }
+    int64_t size = tail.size;
+    if (size < 0) size = counters_behind(tail.err)[kCntSize];  // device-resident counters (see Counters)
+    const float fsize = (float)size;
+    const float x = lane == 0 ? picked : tail.mn[1];
+    float r = 0.0f;
+    if (lane < 2) r = powf_det_call(x / total * fsize, -tail.beta);  // lane 0: the row's power, lane 1: the minimum's
+    const float max_w = __shfl(r, 1);
+    if (lane == 0) {
+        tail.out_idx[k] = idx;
+        tail.out_w[k] = r / max_w;
+        if (!(total > 0.0f) || total > 3.0e38f) atomicOr(tail.err, MRB_DERR_TOTAL);
+        if (idx >= size) atomicOr(tail.err, MRB_DERR_UNFILLED);
+    }
+    if (work.live) {
+#pragma unroll
+        for (int j = 0; j < kRowWaveInF; ++j) asm volatile("" : "+v"(held[j]));
+#pragma unroll
+        for (int j = 0; j < kRowWaveInF; ++j)
+            if (work.live & (1u << j)) *work.dst[j] = held[j];
+    }
+    if (narrow) nw.store(slot, nheld, plan, (uint32_t)lane);
 }
 
 // Gather of wide rows: io_f[k] = store_f[slot_k], slot_k being `fixed_slot` (mode kFromFixedSlot, a
