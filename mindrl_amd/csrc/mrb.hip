@@ -322,6 +322,21 @@ int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, int64_
         LAUNCH_CHECK("k_per_sample_rows");
         return MRB_OK;
     }
+    // Fewer rows of that size: the workgroup kernel with two copy waves instead of four (k_per_sample_light).
+    if (r.row_split == 0 && plan.split == 1 && plan.wide_items <= 2u * 64u * kLightCopyWaves && a.depth != 22) {
+        const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
+        const uint32_t packed = pack_groups(a.depth) | ((plan.nbatch - 1) << 20);
+        const dim3 threads(plan.narrow_items ? (uint32_t)kLightWG : (uint32_t)kLightWG - 64u);
+        const bool ten = a.depth > 0 && a.depth % kGroupMaxLevels == 0, one = plan.nwide == 1;
+#define MRB_LAUNCH_LIGHT(T, O)                                                                                         \
+    hipLaunchKernelGGL((k_per_sample_light<T, O>), grid, threads, 0, s, a.sum, a.uniforms, a.depth, packed, (int)a.batch, \
+                       (uint32_t)a.capacity, a.seed, a.calls, tail, plan)
+        if (ten) { if (one) MRB_LAUNCH_LIGHT(true, true); else MRB_LAUNCH_LIGHT(true, false); }
+        else { if (one) MRB_LAUNCH_LIGHT(false, true); else MRB_LAUNCH_LIGHT(false, false); }
+#undef MRB_LAUNCH_LIGHT
+        LAUNCH_CHECK("k_per_sample_light");
+        return MRB_OK;
+    }
     if (inflight == 2) launch_sample_wide_as<2>(grid, a, plan, s);
     else launch_sample_wide_as<8>(grid, a, plan, s);
     LAUNCH_CHECK("k_per_sample_wide");

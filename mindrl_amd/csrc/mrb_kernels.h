@@ -595,7 +595,8 @@ struct NextPlan {
 
 struct NoNext {};
 
-template <int kInF, bool kTen, bool kOneWide, bool kNext, typename Next>
+// kCW: copy waves of a workgroup (four; two in k_per_sample_light, for rows of at most 4 KB).
+template <int kInF, bool kTen, bool kOneWide, bool kNext, typename Next, int kCW = kCopyWaves>
 __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, const float* __restrict__ uniforms,
                                                  int depth, uint32_t groups, int batch, uint32_t capacity,
                                                  uint64_t seed, uint64_t calls, const SampleTail& tail,
@@ -730,9 +731,9 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
         __builtin_amdgcn_s_setprio(0);
     }
     // ---- copy waves, while the walker walks
-    CopyWork<kInF, kOneWide> work;
+    CopyWork<kInF, kOneWide, 64 * kCW> work;
     NarrowWork nw;
-    const bool narrow = wave == 1 + kCopyWaves && part == 0 && plan.narrow_items && !next_layer;
+    const bool narrow = wave == 1 + kCW && part == 0 && plan.narrow_items && !next_layer;
     if (!walker) {
         if (narrow) nw.prepare(plan, k, lane);
         if (next_layer) work.prepare(plan2, k, part, ctid);
@@ -801,6 +802,20 @@ __global__ __launch_bounds__(kWideWG) void k_per_sample_wide(const float* __rest
                                                              int depth, uint32_t groups, int batch, uint32_t capacity,
                                                              uint64_t seed, uint64_t calls, SampleTail tail, WidePlan plan) {
     sample_wide_body<kInF, kTen, kOneWide, false>(sum, uniforms, depth, groups, batch, capacity, seed, calls, tail, plan, NoNext{});
+}
+
+// The same kernel with two copy waves instead of four, for rows of at most 4 KB in 16-byte fields (two granules per
+// copy thread): a workgroup of three or four waves per row instead of five or six. Rows that small leave most of
+// four copy waves idle, and a launch of a thousand of them is bound by the number of waves to dispatch (config 4,
+// 1024 rows of 521 B). Trees of 22 levels, whose walk four copy waves share, keep the full kernel.
+constexpr int kLightCopyWaves = 2;
+constexpr int kLightWG = 64 + 64 * kLightCopyWaves + 64;
+template <bool kTen, bool kOneWide>
+__global__ __launch_bounds__(kLightWG) void k_per_sample_light(const float* __restrict__ sum, const float* __restrict__ uniforms,
+                                                               int depth, uint32_t groups, int batch, uint32_t capacity,
+                                                               uint64_t seed, uint64_t calls, SampleTail tail, WidePlan plan) {
+    sample_wide_body<2, kTen, kOneWide, false, NoNext, kLightCopyWaves>(sum, uniforms, depth, groups, batch, capacity, seed, calls,
+                                                                       tail, plan, NoNext{});
 }
 
 // Sample plus, in the same launch, one wide field gathered at the slot each sampled row names (see kNext above).
