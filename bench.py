@@ -419,7 +419,18 @@ def bench_per(a):
     levels = max(1, (r.capacity - 1).bit_length())
     # the library's own choice (mrb_per_sample): the LDS-top kernel for many narrow rows, else the wide-row kernel
     lds_path = a.sample_path == 2 or (a.sample_path == 0 and batch >= 8192 and max(r.buf._layout.bytes) <= 256)
-    kernel_name = "k_per_sample_lds" if lds_path else "k_per_sample_wide"
+    # (rows of at most 4 KB in 16-byte fields: the workgroup kernel with two copy waves, or, for launches of at least
+    # 2048 rows, the wave-per-row kernel)
+    wide_granules = sum(b // 16 for b in r.buf._layout.bytes if b % 16 == 0)
+    narrow_bytes = sum(b for b in r.buf._layout.bytes if b % 16)
+    if lds_path:
+        kernel_name = "k_per_sample_lds"
+    elif wide_granules <= 256 and narrow_bytes <= 256 and batch >= 2048 and not a.row_split:
+        kernel_name = "k_per_sample_rows"
+    elif wide_granules <= 256 and levels != 22 and not a.row_split:
+        kernel_name = "k_per_sample_light"
+    else:
+        kernel_name = "k_per_sample_wide"
     if a.workload == "c3":
         # rows read + rows written + index (8) + weight (4): the gather-bound headline figure
         algo_bytes, formula = batch * (2 * row_bytes + 12), "batch * (2 * row_bytes + 12)"
