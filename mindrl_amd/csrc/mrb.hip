@@ -762,13 +762,13 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
 // Device-resident counters: host -> device (when the option is switched on, after a load) and back (state
 // queries, when it is switched off). Both wait for the device.
 int counters_to_device(Per& b) {
-    const int64_t v[4] = {b.pushes, b.size, (int64_t)b.calls, 0};
+    const int64_t v[kCntWords] = {b.pushes, b.size, (int64_t)b.calls, 0, b.pushes % b.rows.capacity};
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(b.counters, v, sizeof(v), hipMemcpyHostToDevice));
     return MRB_OK;
 }
 int counters_from_device(Per& b) {
-    int64_t v[4];
+    int64_t v[kCntWords];
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(v, b.counters, sizeof(v), hipMemcpyDeviceToHost));
     b.pushes = v[kCntPushes], b.size = v[kCntSize], b.calls = (uint64_t)v[kCntCalls];
@@ -776,13 +776,13 @@ int counters_from_device(Per& b) {
 }
 int counters_to_device(Urb& b) {
     const int64_t cap = b.rows.capacity;
-    const int64_t v[4] = {b.count < cap && b.head == 0 ? b.count : b.head, b.count, (int64_t)b.calls, b.head};
+    const int64_t v[kCntWords] = {0, b.count, (int64_t)b.calls, b.head, b.count < cap && b.head == 0 ? b.count : b.head};
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(b.counters, v, sizeof(v), hipMemcpyHostToDevice));
     return MRB_OK;
 }
 int counters_from_device(Urb& b) {
-    int64_t v[4];
+    int64_t v[kCntWords];
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(v, b.counters, sizeof(v), hipMemcpyDeviceToHost));
     b.count = v[kUrbCount], b.head = v[kUrbHead], b.calls = (uint64_t)v[kUrbCalls];
@@ -884,8 +884,8 @@ int mrb_urb_create(int64_t capacity, int nfields, const int64_t* field_bytes, in
     auto b = std::make_shared<Urb>();
     int rc = rows_alloc(b->rows, capacity, nfields, field_bytes);
     if (rc) return rc;
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16 + 4 * sizeof(int64_t)));
-    HIP_TRY(hipMemset(b->err, 0, 16 + 4 * sizeof(int64_t)));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16 + kCntWords * sizeof(int64_t)));
+    HIP_TRY(hipMemset(b->err, 0, 16 + kCntWords * sizeof(int64_t)));
     b->counters = reinterpret_cast<int64_t*>(b->err + 4);
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->slots), kUrbDrawMax * sizeof(int64_t)));
     HIP_TRY(hipDeviceSynchronize());  // the zero-fills ran on the null stream; the caller's stream may not wait for it
@@ -1121,9 +1121,9 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->stamp), (size_t)b->leaves * sizeof(unsigned long long)));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->maxp), 16));
     // one allocation: the error word (16 bytes), then the device copy of the counters (kernels find them there)
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16 + 4 * sizeof(int64_t)));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16 + kCntWords * sizeof(int64_t)));
     b->counters = reinterpret_cast<int64_t*>(b->err + 4);
-    HIP_TRY(hipMemset(b->counters, 0, 4 * sizeof(int64_t)));
+    HIP_TRY(hipMemset(b->counters, 0, kCntWords * sizeof(int64_t)));
     // update_priorities scratch, sized once: a call rarely names more entries than there are rows
     b->powered_cap = capacity < 4096 ? 4096 : (capacity > (1ll << 20) ? (1ll << 20) : capacity);
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->powered), (size_t)b->powered_cap * sizeof(float)));
@@ -1226,8 +1226,9 @@ static int per_push(Per* b, const void* const* src_fields, int64_t nrows, const 
         // one row: one wave walks from its leaf to the root (k_push_one)
         rc = ride_alone_if_large(a, put, s);
         if (rc) return rc;
-        hipLaunchKernelGGL(k_push_one, dim3(1 + put.blocks), dim3(kWG), 0, s, a.sum, a.mn, a.maxp, a.first_slot, a.capacity,
-                           a.leaves, a.depth, a.alpha, opt_priorities, a.err, put, a.advance, 1 + put.blocks);
+        hipLaunchKernelGGL(b->device_counters ? k_push_one<true> : k_push_one<false>, dim3(1 + put.blocks), dim3(kWG), 0, s,
+                           a.sum, a.mn, a.maxp, a.first_slot, a.capacity, a.leaves, a.depth, a.alpha, opt_priorities, a.err, put,
+                           a.advance, 1 + put.blocks * (kWG / 64));
         LAUNCH_CHECK("k_push_one");
         b->pushes += nrows;
         b->size = b->size + nrows < cap ? b->size + nrows : cap;
@@ -1329,14 +1330,18 @@ int mrb_per_update_push(int64_t h, const int64_t* indices, const float* prioriti
             a.priorities = priorities;
             a.n = n;
             a.advance = b->device_counters ? 1 : 0;
-            a.readers = 1 + put.blocks;
             const int64_t slot = b->device_counters ? -1 : first;
+            // (readers: the waves that read the device's counters - the tree wave and every wave of the row copy)
             if (wg) {
                 const uint32_t threads = n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
-                hipLaunchKernelGGL(k_tree_wg_push, dim3(1 + put.blocks), dim3(threads), 0, s, a, slot, opt_push_priorities, put);
+                a.readers = 1 + put.blocks * (threads / 64);
+                hipLaunchKernelGGL(b->device_counters ? k_tree_wg_push<true> : k_tree_wg_push<false>, dim3(1 + put.blocks),
+                                   dim3(threads), 0, s, a, slot, opt_push_priorities, put);
                 LAUNCH_CHECK("k_tree_wg_push");
             } else {
-                hipLaunchKernelGGL(k_tree_paths_push, dim3(1 + put.blocks), dim3(kWG), 0, s, a, slot, opt_push_priorities, put);
+                a.readers = 1 + put.blocks * (kWG / 64);
+                hipLaunchKernelGGL(b->device_counters ? k_tree_paths_push<true> : k_tree_paths_push<false>, dim3(1 + put.blocks),
+                                   dim3(kWG), 0, s, a, slot, opt_push_priorities, put);
                 LAUNCH_CHECK("k_tree_paths_push");
             }
             b->pushes += 1;

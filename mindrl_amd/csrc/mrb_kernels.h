@@ -141,23 +141,56 @@ struct PutArgs {
 // Kernels are told through a negative first slot / row count in their arguments and find the counters
 // behind the buffer's error word (one allocation: 16 bytes of flags, then the counters), so that the
 // arguments of the ordinary case are what they were.
-constexpr int kCntPushes = 0, kCntSize = 1, kCntCalls = 2;
+// ([3] counts the reports of a launch that moves the counters on; [4] is the ring position, pushes mod capacity, kept
+// beside the count so that no kernel divides)
+constexpr int kCntPushes = 0, kCntSize = 1, kCntCalls = 2, kCntPos = 4, kCntWords = 5;
 
 __device__ __forceinline__ const int64_t* counters_behind(const uint32_t* err) {
     return reinterpret_cast<const int64_t*>(err + 4);
 }
 __device__ __forceinline__ int64_t ring_position(const int64_t* counters, int64_t capacity) {
-    return (int64_t)((uint64_t)counters[kCntPushes] % (uint64_t)capacity);
+    return counters[kCntPos];
 }
+// The counters after a push of `pushed` rows (at most `capacity`), stored.
+__device__ __forceinline__ void counters_store_advanced(int64_t* counters, int64_t pushes, int64_t size, int64_t pos,
+                                                        int64_t pushed, int64_t capacity) {
+    counters[kCntPushes] = pushes + pushed;
+    size += pushed;
+    counters[kCntSize] = size < capacity ? size : capacity;
+    pos += pushed;
+    counters[kCntPos] = pos < capacity ? pos : pos - capacity;
+}
+
+// The counters as a wave found them, and what its report returned (see counters_report).
+struct CounterTicket {
+    int64_t pushes, size, pos;
+    uint32_t before;  // reports ahead of this wave's
+};
+// (atomic loads: vector loads past the compute unit's caches, which wait for nothing but themselves)
+__device__ __forceinline__ CounterTicket counters_take(const uint32_t* err) {
+    const int64_t* counters = counters_behind(err);
+    CounterTicket t;
+    t.pushes = __hip_atomic_load(counters + kCntPushes, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    t.size = __hip_atomic_load(counters + kCntSize, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    t.pos = __hip_atomic_load(counters + kCntPos, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    t.before = 0;
+    return t;
+}
+__device__ __forceinline__ int64_t ticket_position(const CounterTicket& t, int64_t capacity) { return t.pos; }
 
 // A push moves the device-resident counters on in its own last launch. Where that launch is also the one whose
 // workgroups read the ring position (`readers` of them: the tree workgroup and the row copy's), every such
 // workgroup reports here when it is done, and the last one to report advances the counters: no workgroup waits
 // for another, and none can read a position already moved on. readers <= 1: the caller is the only reader left.
 // Called by every thread of the workgroup (it contains a barrier); the counters' fourth word counts the reports.
-__device__ __forceinline__ void counters_push_done(uint32_t* err, int64_t pushed, int64_t capacity, uint32_t readers) {
+// `known`: the counters as thread 0 took them when the kernel started (nobody changes them before this advance);
+// without it thread 0 requests them here, ahead of the barrier and the report.
+__device__ __forceinline__ void counters_push_done(uint32_t* err, int64_t pushed, int64_t capacity, uint32_t readers,
+                                                   const CounterTicket* known = nullptr) {
     if (pushed <= 0) return;  // uniform over the launch
-    __syncthreads();          // every wave's reads of the position are behind it
+    CounterTicket t{};
+    if (threadIdx.x == 0) t = known ? *known : counters_take(err);
+    __syncthreads();  // every wave's reads of the position are behind it
     if (threadIdx.x != 0) return;
     int64_t* counters = reinterpret_cast<int64_t*>(err + 4);
     if (readers > 1) {
@@ -165,18 +198,52 @@ __device__ __forceinline__ void counters_push_done(uint32_t* err, int64_t pushed
         if (atomicAdd(arrived, 1u) != readers - 1) return;
         atomicExch(arrived, 0u);
     }
-    counters[kCntPushes] += pushed;
-    const int64_t size = counters[kCntSize] + pushed;
-    counters[kCntSize] = size < capacity ? size : capacity;
+    counters_store_advanced(counters, t.pushes, t.size, t.pos, pushed, capacity);
 }
 
-// The copy itself, by workgroup `block` of `nblocks` (grid-stride over the granules).
-__device__ __forceinline__ void rows_put_part(const PutArgs& p, uint32_t block, uint32_t nblocks) {
+// The same for the one-launch pushes whose tree work is a single wave (k_push_one, k_tree_wg_push,
+// k_tree_paths_push), wave by wave and EARLY: what must precede the advance is every wave's READ of the
+// counters, not its work. A wave takes the counters (counters_take: loads only), reports as soon as the values
+// are there (counters_report: one atomic whose operand depends on the loaded values, so that it cannot be issued
+// before they arrive; its result is not awaited here) and goes on with its work; when that is done it looks at
+// what the atomic returned (counters_settle) and, if it was the last of the `readers` waves to report, stores the
+// advanced counters, computed from the values it took - no load, and no round trip to L2 at the kernel's end.
+// All three are called by whole waves; lane 0 acts. readers <= 1: the calling wave is the only reader.
+__device__ __forceinline__ void counters_report(CounterTicket& t, uint32_t* err, uint32_t readers, uint32_t lane) {
+    if (readers <= 1 || lane != 0) return;
+    unsigned int* arrived = reinterpret_cast<unsigned int*>(reinterpret_cast<int64_t*>(err + 4) + 3);
+    // (both counters are non-negative: the operand is 1)
+    t.before = atomicAdd(arrived, 1u + (unsigned int)((uint64_t)(t.pushes | t.size | t.pos) >> 63));
+}
+__device__ __forceinline__ void counters_settle(const CounterTicket& t, uint32_t* err, int64_t pushed, int64_t capacity,
+                                                uint32_t readers, uint32_t lane) {
+    if (lane != 0) return;
+    int64_t* counters = reinterpret_cast<int64_t*>(err + 4);
+    if (readers > 1) {
+        if (t.before != readers - 1) return;
+        atomicExch(reinterpret_cast<unsigned int*>(counters + 3), 0u);
+    }
+    counters_store_advanced(counters, t.pushes, t.size, t.pos, pushed, capacity);
+}
+
+// How a workgroup that carries a row copy in another kernel's launch ends. The compiler lays such a kernel out as
+// if the tree workgroup's code could follow the copy, and without the explicit wait it makes the tree workgroup
+// wait, early on, for loads that only the copy ever issues (its first requests then go out one after the other
+// instead of together: a third of a microsecond on a one-workgroup call).
+__device__ __forceinline__ void rider_ends() {
+    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_endpgm();
+}
+
+// The copy itself, by workgroup `block` of `nblocks` (grid-stride over the granules). known_first >= 0: the
+// first slot, already read from the device's counters by the caller.
+__device__ __forceinline__ void rows_put_part(const PutArgs& p, uint32_t block, uint32_t nblocks, int64_t known_first = -1) {
     const IoTable& t = p.t;
     const uint64_t total = t.prefix[t.nfields];
     const uint64_t stride = (uint64_t)nblocks * blockDim.x;
-    const int64_t first_slot =
-        p.first_slot >= 0 ? p.first_slot : ring_position(reinterpret_cast<const int64_t*>(p.src_first), p.capacity);
+    const int64_t first_slot = known_first >= 0  ? known_first
+                               : p.first_slot >= 0 ? p.first_slot
+                                                   : ring_position(reinterpret_cast<const int64_t*>(p.src_first), p.capacity);
     for (uint64_t w = (uint64_t)block * blockDim.x + threadIdx.x; w < total; w += stride) {
         const int f = field_of(t, w);
         uint64_t row;
@@ -745,7 +812,8 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
                 s_tail.out_idx = tail.out_idx;
                 s_tail.out_w = tail.out_w;
                 s_tail.err = tail.err;
-                s_tail.size = tail.size;
+                // (device-resident counters, see Counters: the number of stored rows is fetched here, beside the walk)
+                s_tail.size = tail.size >= 0 ? tail.size : counters_behind(tail.err)[kCntSize];
                 s_tail.beta = tail.beta;
             } else if (lane == 1) {
                 s_pmin = tail.mn[1];
@@ -758,8 +826,7 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
         // the slot the sampled row names (outside [0, size): clamped and flagged, as mrb_per_gather does)
         __shared__ int64_t s_next;
         if (walker && lane == 0) {
-            int64_t size = s_tail.size;
-            if (size < 0) size = counters_behind(s_tail.err)[kCntSize];
+            const int64_t size = s_tail.size;
             const int64_t row = idx < (int64_t)capacity ? idx : (int64_t)capacity - 1;
             int64_t to = *reinterpret_cast<const int64_t*>(slot_field + (uint64_t)row * slot_stride);
             if (to < 0 || to >= size) {
@@ -782,8 +849,7 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
     if (part != 0) return;
     // lane 0: (p / total * size)^-beta, lane 1: (pmin / total * size)^-beta
     const float total = s_total;
-    int64_t size = s_tail.size;
-    if (size < 0) size = counters_behind(s_tail.err)[kCntSize];  // device-resident counters (see Counters)
+    const int64_t size = s_tail.size;
     const float fsize = (float)size;
     const float x = lane == 0 ? s_picked : s_pmin;
     float r = 0.0f;
@@ -1838,7 +1904,7 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
     const uint32_t tile_blocks = gridDim.x - put.blocks;
     if (blockIdx.x >= tile_blocks) {
         rows_put_part(put, blockIdx.x - tile_blocks, put.blocks);
-        return;
+        rider_ends();
     }
     const uint32_t lane = threadIdx.x & 63;
     const int lo = a.lo[round], g = a.g[round];
@@ -1886,14 +1952,17 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
 constexpr int kTopWG = 1024;
 __global__ __launch_bounds__(kTopWG) void k_tree_top(UpdateArgs a, PutArgs put) {
     __shared__ unsigned long long s_win[kTopWG / 64][kBlockNodes];
-    if (blockIdx.x >= 1) {
+    if (__builtin_expect(blockIdx.x >= 1, 0)) {  // (the tree workgroup's code comes first: it is the one the call waits for)
         rows_put_part(put, blockIdx.x - 1, put.blocks);
         counters_push_done(a.err, a.advance, a.capacity, a.readers);
-        return;
+        rider_ends();
     }
+    // (a launch that moves the device's counters on: thread 0 takes them now, for the advance at the end)
+    CounterTicket ticket{};
+    if (a.advance > 0 && threadIdx.x == 0) ticket = counters_take(a.err);
     top_rebuild(a, a.top_depth, &s_win[0][0]);
     if (a.fold_max) fold_push_max(a);
-    counters_push_done(a.err, a.advance, a.capacity, a.readers);
+    counters_push_done(a.err, a.advance, a.capacity, a.readers, &ticket);
 }
 
 // ---------------------------------------------------------------------------
@@ -1910,13 +1979,16 @@ constexpr int kFusedWG = 1024;
 
 __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t tile_base, uint32_t units, PutArgs put) {
     __shared__ unsigned long long s_win[kFusedWG / 64][kBlockNodes];
-    if (blockIdx.x >= 1) {
+    if (__builtin_expect(blockIdx.x >= 1, 0)) {  // (the tree workgroup's code comes first: it is the one the call waits for)
         rows_put_part(put, blockIdx.x - 1, put.blocks);
         counters_push_done(a.err, a.advance, a.capacity, a.readers);
-        return;
+        rider_ends();
     }
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int top = a.top_depth;
+    // (a launch that moves the device's counters on: thread 0 takes them now, for the advance at the end)
+    CounterTicket ticket{};
+    if (a.advance > 0 && threadIdx.x == 0) ticket = counters_take(a.err);
     if (!a.inline_election && a.lo[0] == a.depth && a.g[0] == kRoundLevels && top >= kRoundLevels &&
         (1u << top) / kBlockNodes <= (uint32_t)(kFusedWG / 64)) {
         // A push: the top's tiles (one per wave) are requested BEFORE the leaf tiles are rebuilt - of all their
@@ -1976,7 +2048,7 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
             if (wave == 0) tile_round(a, top - kRoundLevels, top - kRoundLevels, 0, false, nullptr, nullptr, 0, lane);
         }
         if (a.fold_max) fold_push_max(a);
-        counters_push_done(a.err, a.advance, a.capacity, a.readers);
+        counters_push_done(a.err, a.advance, a.capacity, a.readers, &ticket);
         return;
     }
     if (const uint32_t unit = wave; unit < units) {
@@ -1994,7 +2066,7 @@ __global__ __launch_bounds__(kFusedWG) void k_tree_fused(UpdateArgs a, uint32_t 
     __syncthreads();
     top_rebuild(a, a.top_depth, &s_win[0][0]);
     if (a.fold_max) fold_push_max(a);
-    counters_push_done(a.err, a.advance, a.capacity, a.readers);
+    counters_push_done(a.err, a.advance, a.capacity, a.readers, &ticket);
 }
 
 // ---------------------------------------------------------------------------
@@ -2146,12 +2218,18 @@ constexpr int kPushOneMaxDepth = 30;
 // The walk of one wave. kAfterUpdate: the walk follows an update_priorities in the same launch (same workgroup),
 // so the running max is read where the update's atomic maxima were performed (past this compute unit's cache),
 // and the siblings are requested only now, after the update's stores.
+// `taken`: this launch moves the device's counters on, `ticket` holds them as the caller took them - the position is theirs,
+// and, unless the caller has reported already (`report`), the wave's report (see counters_report) goes out behind the
+// walk's own requests, so that nothing the walk waits for queues up behind the atomic.
 template <bool kAfterUpdate>
 __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp, int64_t first_slot,
                                               int64_t capacity, int64_t leaves, int depth, float alpha,
-                                              const float* priority, uint32_t* err, uint32_t lane) {
+                                              const float* priority, uint32_t* err, uint32_t lane,
+                                              CounterTicket& ticket, bool taken, bool report, uint32_t readers) {
     // negative: the ring position is on the device (see Counters)
-    const int64_t slot = first_slot >= 0 ? first_slot : ring_position(counters_behind(err), capacity);
+    const int64_t slot = taken             ? ticket_position(ticket, capacity)
+                         : first_slot >= 0 ? first_slot
+                                           : ring_position(counters_behind(err), capacity);
     const uint32_t v = (uint32_t)leaves + (uint32_t)slot;
     float sib_s = 0.0f, sib_m = 0.0f;
     if (lane >= 1 && lane <= (uint32_t)depth) {
@@ -2165,6 +2243,7 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
                                                                            __HIP_MEMORY_SCOPE_AGENT))
                                        : *maxp;
     const float p = priority ? *priority : 0.0f;
+    if (report) counters_report(ticket, err, readers, lane);
     const bool given = priority != nullptr && valid_priority(p);
     if (priority != nullptr && !given && lane == 0) atomicOr(err, MRB_DERR_PRIORITY);
     const float q = given ? powf_det_call(p, alpha) : running;
@@ -2192,18 +2271,48 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
     if (given && lane == 0 && q > 0.0f) raise_max(maxp, q);
 }
 
+// A workgroup of the row copy that rides along in such a launch. advance != 0: this launch moves the device's
+// counters on, every wave reports its read of them (see counters_report).
+__device__ __forceinline__ void push_rider(const PutArgs& put, uint32_t block, uint32_t* err, int64_t advance,
+                                           int64_t capacity, uint32_t readers) {
+    if (advance <= 0) {  // uniform over the launch
+        rows_put_part(put, block, put.blocks);
+        return;
+    }
+    const uint32_t lane = threadIdx.x & 63u;
+    CounterTicket t = counters_take(err);
+    counters_report(t, err, readers, lane);
+    rows_put_part(put, block, put.blocks, ticket_position(t, capacity));
+    counters_settle(t, err, advance, capacity, readers, lane);
+}
+
+// The tree wave of such a launch: the walk of push_one_walk, reporting its read of the device's counters (taken
+// by the caller as `t` when advance != 0) beside the walk's own requests.
+template <bool kAfterUpdate>
+__device__ __forceinline__ void push_one_wave(float* sum, float* mn, float* maxp, int64_t first_slot, int64_t capacity,
+                                              int64_t leaves, int depth, float alpha, const float* priority,
+                                              uint32_t* err, uint32_t lane, CounterTicket& t, int64_t advance,
+                                              uint32_t readers) {
+    push_one_walk<kAfterUpdate>(sum, mn, maxp, first_slot, capacity, leaves, depth, alpha, priority, err, lane, t,
+                                advance > 0, advance > 0, readers);
+    if (advance > 0) counters_settle(t, err, advance, capacity, readers, lane);
+}
+
+template <bool kDev>
 __global__ __launch_bounds__(kWG) void k_push_one(float* __restrict__ sum, float* __restrict__ mn, float* maxp,
                                                   int64_t first_slot, int64_t capacity, int64_t leaves, int depth,
                                                   float alpha, const float* priority, uint32_t* err, PutArgs put,
                                                   int64_t advance, uint32_t readers) {
-    if (blockIdx.x >= 1) {
-        rows_put_part(put, blockIdx.x - 1, put.blocks);
-        counters_push_done(err, advance, capacity, readers);
-        return;
+    if (__builtin_expect(blockIdx.x >= 1, 0)) {  // (the tree workgroup's code comes first: it is the one the call waits for)
+        if (kDev) push_rider(put, blockIdx.x - 1, err, advance, capacity, readers);
+        else rows_put_part(put, blockIdx.x - 1, put.blocks);
+        rider_ends();
     }
-    if (threadIdx.x < 64)
-        push_one_walk<false>(sum, mn, maxp, first_slot, capacity, leaves, depth, alpha, priority, err, threadIdx.x);
-    counters_push_done(err, advance, capacity, readers);
+    if (threadIdx.x >= 64) return;
+    CounterTicket t{};
+    if (kDev) t = counters_take(err);
+    push_one_wave<false>(sum, mn, maxp, first_slot, capacity, leaves, depth, alpha, priority, err, threadIdx.x, t,
+                         kDev ? advance : 0, readers);
 }
 
 // ---------------------------------------------------------------------------
@@ -2280,7 +2389,12 @@ __device__ __forceinline__ bool wg_resolve(const uint32_t* keys, const unsigned 
     return true;
 }
 
-__device__ __forceinline__ void tree_wg_body(const UpdateArgs& a) {
+// kTake: a push follows in the same kernel and moves the device's counters on: the workgroup's LAST wave - a call
+// of a few dozen entries leaves it little else to do, while the first waves carry the entries - leaves them in
+// `ticket` (requested behind the body's own first requests, see counters_take) and reports its read once the
+// election is over, so that the report has long returned when the push looks at it (see counters_report).
+template <bool kTake>
+__device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket& ticket) {
     __shared__ __align__(16) float top_s[kWgTopNodes];
     __shared__ __align__(16) float top_m[kWgTopNodes];
     __shared__ __align__(16) uint32_t keys[3][kWgSlots];
@@ -2347,6 +2461,7 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a) {
             }
         }
     }
+    if (kTake && tid >= nthreads - 64) ticket = counters_take(a.err);
     // the power, while all of that is on its way; every valid entry's counts for the running max, also that
     // of an entry that loses its leaf
     const float q = valid ? powf_det(p, a.alpha) : 0.0f;
@@ -2368,6 +2483,7 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a) {
         }
     }
     lds_barrier();
+    if (kTake && tid >= nthreads - 64) counters_report(ticket, a.err, a.readers, lane);
     bool act = valid && (uint32_t)(vals[0][slot] >> 32) == tid;
     uint32_t v = leaf_node;
     float cs = q, cm = q;
@@ -2476,7 +2592,10 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a) {
     }
 }
 
-__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) { tree_wg_body(a); }
+__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
+    CounterTicket none{};
+    tree_wg_body<false>(a, none);
+}
 
 // ---------------------------------------------------------------------------
 // update_priorities followed by a push of ONE row, in ONE launch (mrb_per_update_push: what a learner does after
@@ -2487,32 +2606,51 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) { tree_
 //   slot      the pushed row's slot (negative: read from the device, see Counters)
 //   priority  the pushed row's priority (NULL: the running max, which includes this call's update)
 // ---------------------------------------------------------------------------
+// kDev: the buffer's counters live on the device and this launch moves them on (see Counters); the other
+// instantiation carries none of that.
+template <bool kDev>
 __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
-    if (blockIdx.x >= 1) {
-        rows_put_part(put, blockIdx.x - 1, put.blocks);
-        counters_push_done(a.err, a.advance, a.capacity, a.readers);
-        return;
+    if (__builtin_expect(blockIdx.x >= 1, 0)) {  // (the tree workgroup's code comes first: it is the one the call waits for)
+        if (kDev) push_rider(put, blockIdx.x - 1, a.err, a.advance, a.capacity, a.readers);
+        else rows_put_part(put, blockIdx.x - 1, put.blocks);
+        rider_ends();
     }
-    tree_wg_body(a);
+    // The device's counters are the last wave's business: it requests them among the update's first requests, hands
+    // the position to the walking wave through LDS and moves the counters on while that wave walks.
+    __shared__ int64_t s_position;
+    const bool keeper = kDev && threadIdx.x >= blockDim.x - 64;
+    CounterTicket t{};
+    tree_wg_body<kDev>(a, t);
+    if (keeper && (threadIdx.x & 63u) == 0) s_position = ticket_position(t, a.capacity);
     __threadfence_block();
     __syncthreads();
-    if (threadIdx.x < 64)
-        push_one_walk<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x);
-    counters_push_done(a.err, a.advance, a.capacity, a.readers);
-}
-
-__global__ __launch_bounds__(kWG) void k_tree_paths_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
-    if (blockIdx.x >= 1) {
-        rows_put_part(put, blockIdx.x - 1, put.blocks);
-        counters_push_done(a.err, a.advance, a.capacity, a.readers);
-        return;
-    }
     if (threadIdx.x < 64) {
-        tree_paths_body(a);
-        __threadfence_block();
-        push_one_walk<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x);
+        CounterTicket none{};
+        if (kDev) {  // (the slot stays in scalar registers either way)
+            const int64_t at = s_position;
+            slot = ((int64_t)__builtin_amdgcn_readfirstlane((int)(at >> 32)) << 32) |
+                   (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+        }
+        push_one_walk<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x,
+                            none, false, false, 0);
+    } else if (keeper) {
+        counters_settle(t, a.err, a.advance, a.capacity, a.readers, threadIdx.x & 63u);
     }
-    counters_push_done(a.err, a.advance, a.capacity, a.readers);
+}
+template <bool kDev>
+__global__ __launch_bounds__(kWG) void k_tree_paths_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
+    if (__builtin_expect(blockIdx.x >= 1, 0)) {  // (the tree workgroup's code comes first: it is the one the call waits for)
+        if (kDev) push_rider(put, blockIdx.x - 1, a.err, a.advance, a.capacity, a.readers);
+        else rows_put_part(put, blockIdx.x - 1, put.blocks);
+        rider_ends();
+    }
+    if (threadIdx.x >= 64) return;
+    CounterTicket t{};
+    if (kDev) t = counters_take(a.err);
+    tree_paths_body(a);
+    __threadfence_block();
+    push_one_wave<true>(a.sum, a.mn, a.maxp, slot, a.capacity, a.leaves, a.depth, a.alpha, priority, a.err, threadIdx.x, t,
+                        kDev ? a.advance : 0, a.readers);
 }
 
 // ---------------------------------------------------------------------------
@@ -2711,18 +2849,14 @@ __global__ __launch_bounds__(kDrWG) void k_discounted_return_tiled(const float* 
 // Device-resident counters (see Counters): after a push, and after a sample that used the generator.
 __global__ void k_counters_advance(int64_t* counters, int64_t pushed, int64_t capacity, int64_t calls) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
-        if (pushed) {
-            counters[kCntPushes] += pushed;
-            const int64_t size = counters[kCntSize] + pushed;
-            counters[kCntSize] = size < capacity ? size : capacity;
-        }
+        if (pushed) counters_store_advanced(counters, counters[kCntPushes], counters[kCntSize], counters[kCntPos], pushed, capacity);
         counters[kCntCalls] += calls;
     }
 }
 
-// The uniform buffer's device-resident counters: [0] the next write position, [1] count, [2] the generator's
-// call counter, [3] head. kUrb* name them; the row copy finds its position at [0] like a prioritized push.
-constexpr int kUrbWrite = 0, kUrbCount = 1, kUrbCalls = 2, kUrbHead = 3;
+// The uniform buffer's device-resident counters: [1] count, [2] the generator's call counter, [3] head, [4] the
+// next write position. kUrb* name them; the row copy finds its position where a prioritized push finds it.
+constexpr int kUrbWrite = kCntPos, kUrbCount = 1, kUrbCalls = 2, kUrbHead = 3;
 constexpr int64_t kUrbDrawMax = 1 << 16;  // most rows a sample draws through the device-side index array
 
 // count / head after an append of n rows (n <= capacity; the write position is chosen once per call: `count`

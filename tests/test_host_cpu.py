@@ -100,7 +100,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
     assert sum("k_per_sample_wide" in k for k in kernels) == 8 and sum("k_rows_gather_wide" in k for k in kernels) == 4
-    assert len(kernels) == 49, sorted(kernels)
+    assert len(kernels) == 52, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)
@@ -109,7 +109,8 @@ def test_kernels_use_no_scratch_memory(tmp_path):
         if "k_tree_update" in name:
             assert lds == 8192, (name, lds)  # the election words (256 x 8 B per wave) and nothing else
         if "k_tree_wg" in name:
-            assert lds == 2 * 4096 * 4 + 3 * 2048 * 12, (name, lds)  # the staged top of both trees, three hash tables
+            # the staged top of both trees, three hash tables (+ the position word of the device-counter variant)
+            assert lds == 2 * 4096 * 4 + 3 * 2048 * 12 + (8 if "pushILb1E" in name else 0), (name, lds)
 
 
 def test_only_the_documented_entry_points_wait_or_allocate():
