@@ -1030,6 +1030,34 @@ __global__ __launch_bounds__(kWideWG) void k_rows_gather_wide(const int64_t* __r
     if (!walker) work.run((uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)s_idx), plan, narrow, nw, lane);
 }
 
+// Three levels of the descent from the eight nodes three levels under a node (lo: the first four, hi: the last
+// four): which of them the mass falls into, what is left of the mass inside it, and its value. The sums of the
+// two levels between are the single additions the tree was built with.
+__device__ __forceinline__ uint32_t walk8(const float4 lo, const float4 hi, float& mass, float& picked) {
+    const float a0 = lo.x + lo.y, a1 = lo.z + lo.w, a2 = hi.x + hi.y;
+    const float b0 = a0 + a1;
+    uint32_t p = 0;
+    if (!(mass <= b0)) {
+        mass -= b0;
+        p = 4;
+    }
+    const float left1 = p ? a2 : a0;
+    if (!(mass <= left1)) {
+        mass -= left1;
+        p += 2;
+    }
+    const float n0 = p == 0 ? lo.x : p == 2 ? lo.z : p == 4 ? hi.x : hi.z;
+    const float n1 = p == 0 ? lo.y : p == 2 ? lo.w : p == 4 ? hi.y : hi.w;
+    if (!(mass <= n0)) {
+        mass -= n0;
+        p += 1;
+        picked = n1;
+    } else {
+        picked = n0;
+    }
+    return p;
+}
+
 // ---------------------------------------------------------------------------
 // PER sample, many narrow rows: one workgroup per 256 strata. The top
 // `lds_levels` levels of the sum tree (nodes [1, 2 << lds_levels)) are staged
@@ -1079,6 +1107,15 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
         float mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
         uint32_t node = 1;
         int d = 0;
+        // through the staged levels three at a time: the eight descendants of `node` three levels down are 32
+        // contiguous, aligned bytes of LDS - one read instead of three dependent ones -, the two levels between
+        // are rebuilt with the additions the tree was built with
+        for (; d + 3 <= lds_levels; d += 3) {
+            const float4 lo = *reinterpret_cast<const float4*>(s_top + ((size_t)node << 3));
+            const float4 hi = *reinterpret_cast<const float4*>(s_top + ((size_t)node << 3) + 4);
+            float unused;
+            node = (node << 3) + walk8(lo, hi, mass, unused);
+        }
         for (; d < lds_levels; ++d) {
             const float left = s_top[2 * node];
             if (mass <= left) {
@@ -1117,28 +1154,7 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
             } else if (g == 3) {
                 const float4* src = reinterpret_cast<const float4*>(sum + ((uint64_t)node << 3));
                 const float4 lo = src[0], hi = src[1];
-                const float a0 = lo.x + lo.y, a1 = lo.z + lo.w, a2 = hi.x + hi.y;
-                const float b0 = a0 + a1;
-                uint32_t p = 0;
-                if (!(mass <= b0)) {
-                    mass -= b0;
-                    p = 4;
-                }
-                const float left1 = p ? a2 : a0;
-                if (!(mass <= left1)) {
-                    mass -= left1;
-                    p += 2;
-                }
-                const float n0 = p == 0 ? lo.x : p == 2 ? lo.z : p == 4 ? hi.x : hi.z;
-                const float n1 = p == 0 ? lo.y : p == 2 ? lo.w : p == 4 ? hi.y : hi.w;
-                if (!(mass <= n0)) {
-                    mass -= n0;
-                    p += 1;
-                    picked = n1;
-                } else {
-                    picked = n0;
-                }
-                node = (node << 3) + p;
+                node = (node << 3) + walk8(lo, hi, mass, picked);
             } else if (g == 2) {
                 const float4 v = *reinterpret_cast<const float4*>(sum + ((uint64_t)node << 2));
                 const float left = v.x + v.y;
