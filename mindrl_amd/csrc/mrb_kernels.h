@@ -2714,151 +2714,158 @@ __global__ __launch_bounds__(kWG) void k_discounted_return(const float* __restri
 // system idle: a workgroup takes 64 columns and walks the time axis backwards in chunks of
 // kDrChunk steps through three LDS buffers, as a pipeline whose stages run at the same time on
 // consecutive chunks:
-//   request  waves 1..15 (the movers) request chunk s+1's rewards and done flags into registers
-//            (independent, coalesced loads); they arrive during the stage ...
-//   deposit  ... the movers put chunk s, requested a stage ago, into its LDS buffer ...
-//   recur    ... wave 0 runs the recurrence over chunk s-1 out of LDS (lane = column) ...
-//   drain    ... and the movers write chunk s-2's results from LDS to memory.
+//   deposit  waves 1..15 (the movers) put chunk s, requested a stage ago, into its LDS buffer ...
+//   request  ... request chunk s+1's rewards and done flags into the registers just emptied
+//            (independent, coalesced loads; they arrive during the next stage) ...
+//   drain    ... and write chunk s-2's results from LDS to memory, while ...
+//   recur    ... wave 0 runs the recurrence over chunk s-1 out of LDS (lane = column).
 // One barrier per stage; no wave waits for a load it has just issued. The memory system so sees
 // loads and stores all the time, instead of a load phase, a phase without traffic and a store
 // phase per chunk. The arithmetic and its order are those of k_discounted_return.
+// Every mover issues the SAME number of loads and stores in every stage, without a branch around any of them: a
+// row past the end of a short chunk is replaced by the chunk's last row (loaded twice, stored twice with the same
+// value), a chunk past the end of the time axis by one row that is already cached, a column past the last one
+// by the workgroup's first column. Only so can the compiler count what is in flight: with a branch per element
+// it waited for EVERYTHING before each deposit - also for the next chunk's loads, issued a moment before -
+// and every stage paid a full trip to memory (0.6 us per stage, a quarter of the kernel's time).
 // (lds_barrier: here the next chunk's requests and the last chunk's results stay in flight across it.)
 
-constexpr int kDrChunk = 128;
 constexpr int kDrCols = 64;
 constexpr int kDrWG = 1024;
-constexpr int kDrMovers = kDrWG - 64;                         // threads of waves 1..15
-constexpr int kDrSweep = kDrMovers / kDrCols;                 // rows the movers cover at once
-constexpr int kDrPer = (kDrChunk + kDrSweep - 1) / kDrSweep;  // elements a mover carries per chunk
+constexpr int kDrMovers = kDrWG - 64;          // threads of waves 1..15
+constexpr int kDrSweep = kDrMovers / kDrCols;  // rows the movers cover at once
+constexpr int kDrPer = 4;                      // elements a mover carries per chunk
+constexpr int kDrChunk = kDrPer * kDrSweep;    // 60 steps; three buffers of 60 x 64 x 8 B are 92 KB of LDS
+constexpr int kDrAhead = 3;                    // chunks on their way from memory at any time
 __global__ __launch_bounds__(kDrWG) void k_discounted_return_tiled(const float* __restrict__ reward,
                                                                  const uint8_t* __restrict__ done,
                                                                  const float* __restrict__ last_value,
                                                                  float* __restrict__ out, int64_t timesteps,
                                                                  int64_t batch, int64_t inner, float gamma) {
-    __shared__ float s_val[3][kDrChunk * kDrCols];    // rewards in, returns out
-    __shared__ uint8_t s_done[3][kDrChunk * kDrCols];
+    // per element: .x the reward in, the return out; .y the factor (1 - done) * gamma, put there by the mover that
+    // holds the done flag, so that a step of the recurrence is one LDS read, one multiply-add, one LDS write
+    __shared__ float2 s_val[3][kDrChunk * kDrCols];
     const int64_t cols = batch * inner;
-    const int64_t c0 = (int64_t)blockIdx.x * kDrCols;
+    // Workgroups are dealt to the chip's eight dies in turn, and each die has its own L2. A workgroup's 64 done flags
+    // of a time step are half a cache line, the neighbouring columns' workgroup reads the other half: with
+    // neighbours on different dies every such line is fetched from memory twice (measured: 98.5 MB fetched per
+    // launch for 81.9 MB of input at [1000, 16384]). So neighbouring column groups go to the SAME die: workgroup b
+    // takes group (b mod 8) * (n / 8) + b / 8 when the grid divides by eight.
+    uint32_t group = blockIdx.x;
+    if ((gridDim.x & 7u) == 0) group = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int64_t c0 = (int64_t)group * kDrCols;
     const int ncols = (int)(cols - c0 < kDrCols ? cols - c0 : kDrCols);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const bool mover = wave != 0;
     // a mover's elements of a chunk: column m % 64 of the rows m / 64, m / 64 + 15, ... (960 movers = 15 rows
-    // of 64 columns per sweep), so its addresses differ by a constant from one element to the next
+    // of 64 columns per sweep)
     const int m = (int)threadIdx.x - 64;
-    const int mrow = m / kDrCols;
-    const bool mcol_ok = m % kDrCols < ncols;
-    const int mcol = mcol_ok ? m % kDrCols : 0;  // a column past the end reads column 0 and stores nothing
-    const int64_t mb = (c0 + mcol) / inner;      // the column's batch entry (done flags)
+    const int mrow = m / kDrCols;                                   // wave-uniform
+    const int mcol = m % kDrCols < ncols ? m % kDrCols : 0;         // a column past the end doubles column 0
+    const int64_t mb = (c0 + mcol) / inner;                         // the column's batch entry (done flags)
     const int nchunks = (int)((timesteps + kDrChunk - 1) / kDrChunk);
-    // chunk c covers the steps [lo, lo + steps), counted from the end of the time axis
+    // chunk c covers the steps [lo, lo + steps), counted from the end of the time axis; past the end: one row
     auto chunk_lo = [&](int c) -> int64_t {
         const int64_t hi = timesteps - (int64_t)c * kDrChunk;
         return hi > kDrChunk ? hi - kDrChunk : 0;
     };
     auto chunk_steps = [&](int c) -> int {
         const int64_t hi = timesteps - (int64_t)c * kDrChunk;
-        return (int)(hi > kDrChunk ? kDrChunk : hi);
+        return (int)(hi > kDrChunk ? kDrChunk : hi > 0 ? hi : 1);
     };
+    // (1 - done) * gamma has two values, computed once
+    const float scaled_live = (1.0f - 0.0f) * gamma, scaled_done = (1.0f - 1.0f) * gamma;
     // (done flags travel as 32-bit values: byte-sized register arrays make the compiler pack and unpack them)
-    auto request = [&](int c, float (&r)[kDrPer], uint32_t (&d)[kDrPer]) {
-        if (c >= nchunks) return;
+    // kDrAhead register sets take turns: chunk c travels in set c % kDrAhead, requested kDrAhead stages before it
+    // is deposited, so that several chunks are on their way at any time (one chunk in flight per compute unit is
+    // less than the memory system needs to stay busy: it waited out a trip to memory per stage)
+    float r[kDrAhead][kDrPer];
+    uint32_t d[kDrAhead][kDrPer];
+    auto request = [&](int c, float (&rr)[kDrPer], uint32_t (&dd)[kDrPer]) {
         const int64_t lo = chunk_lo(c);
-        const int steps = chunk_steps(c);
-        const float* rp = reward + (lo + mrow) * cols + c0 + mcol;
-        const uint8_t* dp = done + (lo + mrow) * batch + mb;
-        const int64_t rstep = kDrSweep * cols, dstep = kDrSweep * batch;  // wave-uniform
+        const int last_row = chunk_steps(c) - 1;
 #pragma unroll
         for (int u = 0; u < kDrPer; ++u) {
-            if (mrow + u * kDrSweep < steps) {
-                r[u] = __builtin_nontemporal_load(rp);
-                d[u] = *dp;
-            }
-            rp += rstep;
-            dp += dstep;
+            const int row = mrow + u * kDrSweep < last_row ? mrow + u * kDrSweep : last_row;  // wave-uniform
+            rr[u] = __builtin_nontemporal_load(reward + (lo + row) * cols + c0 + mcol);
+            dd[u] = done[(lo + row) * batch + mb];
         }
     };
-    auto deposit = [&](int c, const float (&r)[kDrPer], const uint32_t (&d)[kDrPer]) {
-        if (c >= nchunks) return;
-        const int steps = chunk_steps(c);
-        float* dv = s_val[c % 3] + m;
-        uint8_t* dd = s_done[c % 3] + m;
+    auto deposit = [&](int c, const float (&rr)[kDrPer], const uint32_t (&dd)[kDrPer]) {
+        float2* dv = s_val[c % 3] + mrow * kDrCols + mcol;
 #pragma unroll
-        for (int u = 0; u < kDrPer; ++u) {
-            if (mrow + u * kDrSweep < steps) {
-                dv[u * kDrMovers] = r[u];
-                dd[u * kDrMovers] = (uint8_t)d[u];
-            }
-        }
+        for (int u = 0; u < kDrPer; ++u) dv[u * kDrMovers] = make_float2(rr[u], dd[u] ? scaled_done : scaled_live);
     };
     auto drain = [&](int c) {
-        if (c < 0 || c >= nchunks || !mcol_ok) return;
         const int64_t lo = chunk_lo(c);
-        const int steps = chunk_steps(c);
-        const float* src = s_val[c % 3] + m;
-        float* op = out + (lo + mrow) * cols + c0 + mcol;
-        const int64_t ostep = kDrSweep * cols;  // wave-uniform
+        const int last_row = chunk_steps(c) - 1;
+        const float2* src = s_val[c % 3] + mcol;
 #pragma unroll
         for (int u = 0; u < kDrPer; ++u) {
-            if (mrow + u * kDrSweep < steps) __builtin_nontemporal_store(src[u * kDrMovers], op);
-            op += ostep;
+            const int row = mrow + u * kDrSweep < last_row ? mrow + u * kDrSweep : last_row;  // wave-uniform
+            __builtin_nontemporal_store(src[row * kDrCols].x, out + (lo + row) * cols + c0 + mcol);
         }
     };
     float last = 0.0f;
     if (wave == 0 && lane < ncols) last = last_value[c0 + lane];
-    // (1 - done) * gamma has two values; computing both once leaves a select, a multiply and an add per step
-    const float scaled_live = (1.0f - 0.0f) * gamma, scaled_done = (1.0f - 1.0f) * gamma;
     auto recur = [&](int c) {
-        if (c < 0 || c >= nchunks || lane >= ncols) return;
+        if (c >= nchunks || lane >= ncols) return;
         const int steps = chunk_steps(c);
-        float* val = s_val[c % 3];
-        const uint8_t* dn = s_done[c % 3];
+        float2* val = s_val[c % 3];
         // 16 steps at a time through registers, so that the LDS reads are not serialised behind the
         // recurrence's stores
-        constexpr int STEP = 16;
+        constexpr int STEP = 15;
         int tt = steps - 1;
         for (; tt >= STEP - 1; tt -= STEP) {
-            float r[STEP];
-            uint32_t d[STEP];
+            float2 v[STEP];
+#pragma unroll
+            for (int u = 0; u < STEP; ++u) v[u] = val[(tt - u) * kDrCols + lane];
 #pragma unroll
             for (int u = 0; u < STEP; ++u) {
-                r[u] = val[(tt - u) * kDrCols + lane];
-                d[u] = dn[(tt - u) * kDrCols + lane];
+                last = v[u].x + v[u].y * last;
+                v[u].x = last;
             }
 #pragma unroll
-            for (int u = 0; u < STEP; ++u) {
-                last = r[u] + (d[u] ? scaled_done : scaled_live) * last;
-                r[u] = last;
-            }
-#pragma unroll
-            for (int u = 0; u < STEP; ++u) val[(tt - u) * kDrCols + lane] = r[u];
+            for (int u = 0; u < STEP; ++u) val[(tt - u) * kDrCols + lane].x = v[u].x;
         }
         for (; tt >= 0; --tt) {
-            last = val[tt * kDrCols + lane] + (dn[tt * kDrCols + lane] ? scaled_done : scaled_live) * last;
-            val[tt * kDrCols + lane] = last;
+            const float2 v = val[tt * kDrCols + lane];
+            last = v.x + v.y * last;
+            val[tt * kDrCols + lane].x = last;
         }
     };
-    // two register sets take turns: the chunk requested in one stage is deposited in the next
-    float ra[kDrPer], rb[kDrPer];
-    uint32_t da[kDrPer], db[kDrPer];
-    if (mover) request(0, ra, da);
-    for (int s = 0; s < nchunks + 2; s += 2) {
-        if (mover) {
-            request(s + 1, rb, db);
-            drain(s - 2);
-            deposit(s, ra, da);
-        } else if (wave == 0) {
+    // stage s: the movers deposit chunk s, request chunk s + kDrAhead into the registers just emptied and drain
+    // chunk s - 2; wave 0 runs the recurrence over chunk s - 1. The two roles run their own loops (the same number
+    // of barriers each): the movers' loop then holds nothing but its own loads and stores, in fixed numbers.
+    static_assert(kDrAhead >= 2, "the two stages without a drain use the first two register sets");
+    if (!mover) {
+        lds_barrier();
+        for (int s = 1; s < nchunks + 2; ++s) {
             recur(s - 1);
+            lds_barrier();
         }
-        lds_barrier();
-        if (mover) {
-            request(s + 2, ra, da);
-            drain(s - 1);
-            deposit(s + 1, rb, db);
-        } else if (wave == 0) {
-            recur(s);
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < kDrAhead; ++j) request(j, r[j], d[j]);
+    deposit(0, r[0], d[0]);
+    request(kDrAhead, r[0], d[0]);
+    lds_barrier();
+    deposit(1, r[1], d[1]);
+    request(1 + kDrAhead, r[1], d[1]);
+    lds_barrier();
+    for (int s = 2; s < nchunks + 2; s += kDrAhead) {
+#pragma unroll
+        for (int j = 0; j < kDrAhead; ++j) {
+            if (s + j >= nchunks + 2) break;  // (uniform; nothing is requested or stored after the loop)
+            constexpr int kFirst = 2 % kDrAhead;
+            const int set = (kFirst + j) % kDrAhead;  // = (s + j) % kDrAhead, known when the loop is unrolled
+            deposit(s + j, r[set], d[set]);  // (past the end of the time axis: a row nobody reads, into a buffer nobody uses)
+            request(s + j + kDrAhead, r[set], d[set]);
+            drain(s + j - 2);
+            lds_barrier();
         }
-        lds_barrier();
     }
 }
 
