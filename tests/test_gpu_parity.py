@@ -705,7 +705,12 @@ def test_discounted_return_reference_vectors(mrb):
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 1), (5, 1, 1), (37, 3, 1), (100, 64, 5), (1000, 256, 1), (9, 1000, 17),
-                                   (300, 65, 1), (257, 130, 3), (40, 70000, 1), (33, 9000, 8)])
+                                   (300, 65, 1), (257, 130, 3), (40, 70000, 1), (33, 9000, 8),
+                                   # the tiled kernel's chunks of 60 steps (one, one and a step, as many as are kept
+                                   # in flight, one more, ...) and grids that divide by eight (column groups are dealt
+                                   # to the dies in another order then), up to the 256 workgroups of 16,384 columns
+                                   (60, 512, 1), (61, 1024, 1), (120, 515, 1), (180, 1536, 1), (181, 100, 2),
+                                   (240, 2048, 1), (241, 4096, 1), (59, 16384, 1), (130, 2047, 8)])
 def test_discounted_return_bit_exact(mrb, orc, shape):
     from mindrl_amd.utils import DiscountedReturn
     t, b, inner = shape
