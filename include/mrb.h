@@ -88,13 +88,12 @@ int mrb_version(void);
  *   "sample_path"  prioritized buffers: 0 = choose by row size, 1 = wide-row kernel, 2 = LDS-top kernel
  *   "lds_levels"   prioritized buffers: tree levels staged in LDS by the LDS-top kernel (0 = auto, max 12)
  *   "device_counters" prioritized and uniform buffers: 1 = the ring position, the number of stored rows and the generator's
- *                  call counter are kept in device memory, read there by the kernels and advanced there by
- *                  a one-thread kernel after every push and every generator-driven sample - for callers that
- *                  record push / sample / update into a HIP graph: every replay then continues where the last
- *                  one stopped (pushes land in the next slots, draws differ, weights use the current row
- *                  count). While it is on: a push takes at most `capacity` rows, an update at most 1024
- *                  entries, a generator-driven sample at most max(4096, min(capacity, 2^20)) rows, sample
- *                  calls on one handle must not overlap (they share a scratch array), and mrb_per_state and
+ *                  call counter are kept in device memory, read there by the kernels and advanced there - by
+ *                  the push's own last launch, and by a one-thread kernel after a generator-driven sample - for
+ *                  callers that record push / sample / update into a HIP graph: every replay then continues
+ *                  where the last one stopped (pushes land in the next slots, draws differ, weights use the
+ *                  current row count). While it is on: a push takes at most `capacity` rows, an update at most
+ *                  1024 entries, and mrb_per_state and
  *                  the checkpoint calls wait for the device to read the counters back. Switching it (either
  *                  way) waits for the device. 0 (default) = host-side counters, passed as kernel arguments.
  *                  Uniform buffers: count, head and the generator's call counter; an append takes at most

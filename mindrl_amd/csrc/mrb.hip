@@ -1399,19 +1399,11 @@ static int per_sample_impl(Per* b, int64_t nbatch, int64_t batch, float beta, co
     a.err = b->err;
     if (b->device_counters) {
         a.size = -1;  // the kernels take the number of stored rows from the device
-        if (!uniforms) {
-            // the generator's call counter is on the device: its draws are written out first (into the scratch
-            // update_priorities uses; calls on one handle are ordered) and the sample kernel reads them
-            if (nbatch * batch > b->powered_cap)
-                return fail(MRB_ESTATE, "with device_counters a generator-driven sample takes at most %lld rows",
-                            (long long)b->powered_cap);
-            hipLaunchKernelGGL(k_fill_uniforms, dim3(grid_exact((uint64_t)(nbatch * batch))), dim3(kWG), 0, s, b->powered,
-                               b->seed, b->counters, batch, nbatch);
-            LAUNCH_CHECK("k_fill_uniforms");
-            a.uniforms = b->powered;
-        }
+        // the generator's call counter is on the device too: the kernels read it there and add the number of the
+        // batch (see generator_calls)
+        if (!uniforms) a.calls = 0;
     }
-    const float* const draws = a.uniforms;  // the caller's, the written-out generator's, or NULL
+    const float* const draws = a.uniforms;  // the caller's, or NULL: the generator's, computed by the kernels
     const int64_t max_bytes = widest_field(b->rows);
     int path = (int)b->sample_path;
     if (path == 0) path = (batch >= 8192 && max_bytes <= 256) ? 2 : 1;

@@ -161,6 +161,14 @@ __device__ __forceinline__ void counters_store_advanced(int64_t* counters, int64
     counters[kCntPos] = pos < capacity ? pos : pos - capacity;
 }
 
+// The generator's call counter for a sample kernel: the argument, or - when the counters live on the device (a
+// negative row count tells) and the generator supplies the draws - the device's counter plus the argument (the
+// number of the batch among those the call launches one by one).
+__device__ __forceinline__ uint64_t generator_calls(const float* uniforms, uint64_t calls, int64_t size, const uint32_t* err) {
+    if (uniforms || size >= 0) return calls;
+    return (uint64_t)counters_behind(err)[kCntCalls] + calls;
+}
+
 // The counters as a wave found them, and what its report returned (see counters_report).
 struct CounterTicket {
     int64_t pushes, size, pos;
@@ -716,7 +724,8 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
         if (mine) {
             group_request(sum, (1u << share) + w, kGroupMaxLevels, lane, r0, r1, r2, r3);
             total = sum[1];
-            u = uniforms ? uniforms[k] : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+            const uint64_t calls_now = generator_calls(uniforms, calls, tail.size, tail.err);
+            u = uniforms ? uniforms[k] : rng_uniform(seed, calls_now + nth, (uint64_t)stratum);
             __builtin_amdgcn_sched_barrier(0);
             v = group_finish(kGroupMaxLevels, lane, r0, r1, r2, r3);
             const float t = group_total(v);
@@ -770,8 +779,9 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
             group_request(sum, 1u, g, lane, r0, r1, r2, r3);
             total = sum[1];
             const float u_given = *(uniforms ? uniforms + k : sum + 1);
+            const uint64_t calls_now = generator_calls(uniforms, calls, tail.size, tail.err);
             __builtin_amdgcn_sched_barrier(0);
-            const float u = uniforms ? u_given : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+            const float u = uniforms ? u_given : rng_uniform(seed, calls_now + nth, (uint64_t)stratum);
             mass = (u + (float)stratum) * (total / (float)batch);  // each operation rounded once
             node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
 #pragma nounroll
@@ -785,7 +795,7 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
         } else {
             // one or two leaves
             total = sum[1];
-            const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+            const float u = uniforms ? uniforms[k] : rng_uniform(seed, generator_calls(uniforms, calls, tail.size, tail.err) + nth, (uint64_t)stratum);
             mass = (u + (float)stratum) * (total / (float)batch);
             picked = total;
             node = (1u << depth) + (depth ? group_walk(group_load_tiny(sum, 1u, depth, lane), depth, lane, mass, picked) : 0u);
@@ -930,11 +940,12 @@ __global__ __launch_bounds__(kRowWaveWG) void k_per_sample_rows(const float* __r
         group_request(sum, 1u, g, lane, r0, r1, r2, r3);
         total = sum[1];
         const float u_given = *(uniforms ? uniforms + k : sum + 1);
+        const uint64_t calls_now = generator_calls(uniforms, calls, tail.size, tail.err);
         __builtin_amdgcn_sched_barrier(0);
         // the field table, while the first group is on its way
         work.prepare(plan, k, 0, (uint32_t)lane);
         if (narrow) nw.prepare(plan, k, (uint32_t)lane);
-        const float u = uniforms ? u_given : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+        const float u = uniforms ? u_given : rng_uniform(seed, calls_now + nth, (uint64_t)stratum);
         mass = (u + (float)stratum) * (total / (float)batch);  // each operation rounded once
         node = (1u << g) + group_walk(group_finish(g, lane, r0, r1, r2, r3), g, lane, mass, picked);
 #pragma nounroll
@@ -947,7 +958,7 @@ __global__ __launch_bounds__(kRowWaveWG) void k_per_sample_rows(const float* __r
         }
     } else {
         total = sum[1];
-        const float u = uniforms ? uniforms[k] : rng_uniform(seed, calls + nth, (uint64_t)stratum);
+        const float u = uniforms ? uniforms[k] : rng_uniform(seed, generator_calls(uniforms, calls, tail.size, tail.err) + nth, (uint64_t)stratum);
         work.prepare(plan, k, 0, (uint32_t)lane);
         if (narrow) nw.prepare(plan, k, (uint32_t)lane);
         mass = (u + (float)stratum) * (total / (float)batch);
@@ -1103,7 +1114,7 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
     float weight = 0.0f;
     if (k < batch) {
         const float total = s_top[1];
-        if (!uniforms) u = rng_uniform(seed, calls, (uint64_t)k);
+        if (!uniforms) u = rng_uniform(seed, generator_calls(uniforms, calls, a.size, a.err), (uint64_t)k);
         float mass = (u + (float)k) * (total / (float)batch);  // each operation rounded once
         uint32_t node = 1;
         int d = 0;
@@ -2928,16 +2939,6 @@ __global__ __launch_bounds__(kWG) void k_urb_slots(int64_t* dst, uint64_t seed, 
     }
     const int64_t t = count - head;
     dst[0] = at < t ? at + head : at - t;
-}
-
-// The generator's draws for `nbatch` batches, written out for a sample kernel to read: with the call
-// counter on the device the kernel cannot take it as an argument.
-__global__ __launch_bounds__(kWG) void k_fill_uniforms(float* dst, uint64_t seed, const int64_t* counters, int64_t batch,
-                                                       int64_t nbatch) {
-    const int64_t i = (int64_t)blockIdx.x * kWG + threadIdx.x;
-    if (i >= batch * nbatch) return;
-    const int64_t nth = i / batch;
-    dst[i] = rng_uniform(seed, (uint64_t)counters[kCntCalls] + (uint64_t)nth, (uint64_t)(i - nth * batch));
 }
 
 // Fills a float array with one value (tree initialisation: sums 0, mins FLT_MAX).
