@@ -4,6 +4,7 @@
 // entry point that touches a buffer fails with MRB_EHIP.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cfloat>
 #include <cstdarg>
@@ -376,7 +377,10 @@ int gather_rows(const RowStore& r, const int64_t* indices, int64_t fixed_slot, i
         LAUNCH_CHECK("k_rows_gather_wide");
         return MRB_OK;
     }
-    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(t.prefix[t.nfields])), dim3(kWG), 0, s, t, r.capacity, count,
+    // a row of workgroups per field, as many as the field with the most granules needs
+    uint64_t most = 0;
+    for (int f = 0; f < t.nfields; ++f) most = std::max<uint64_t>(most, t.prefix[f + 1] - t.prefix[f]);
+    hipLaunchKernelGGL(k_rows_gather, dim3(grid_for(most), (uint32_t)t.nfields), dim3(kWG), 0, s, t, r.capacity, count,
                        indices, fixed_slot, seed, calls, out_indices, err);
     LAUNCH_CHECK("k_rows_gather");
     return MRB_OK;

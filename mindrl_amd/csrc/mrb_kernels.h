@@ -286,13 +286,20 @@ __global__ __launch_bounds__(kWG) void k_rows_gather(IoTable t, int64_t capacity
                                                      uint64_t seed, uint64_t calls,
                                                      int64_t* __restrict__ out_indices,
                                                      uint32_t* __restrict__ err) {
-    const uint64_t total = t.prefix[t.nfields];
-    const uint64_t stride = (uint64_t)gridDim.x * kWG;
-    for (uint64_t w = (uint64_t)blockIdx.x * kWG + threadIdx.x; w < total; w += stride) {
-        const int f = field_of(t, w);
+    // blockIdx.y is the field: the table's entries for it are the same for every thread of the launch's row of
+    // workgroups and come through scalar registers, requested with the other arguments. (Indexed by a field number
+    // each thread works out for itself they were two more dependent trips to memory in a kernel that is a chain of
+    // such trips and nothing else.)
+    const int f = blockIdx.y;
+    const uint32_t units = t.units[f], vl = t.vec_log2[f], row_bytes = t.row_bytes[f], stride_f = t.stride[f];
+    const gbyte* const store = as_global(t.store[f]);
+    gbyte* const io = as_global(t.io[f]);
+    const uint64_t total = t.prefix[f + 1] - t.prefix[f];  // rows * units
+    const uint64_t step = (uint64_t)gridDim.x * kWG;
+    for (uint64_t w = (uint64_t)blockIdx.x * kWG + threadIdx.x; w < total; w += step) {
         uint64_t row;
         uint32_t unit;
-        split_work(w - t.prefix[f], t.units[f], row, unit);
+        split_work(w, units, row, unit);
         int64_t slot = fixed_slot >= 0 ? fixed_slot : indices ? indices[row] : rng_below(seed, calls, row, count);
         // a fixed slot was range-checked by the host against the ring (it may lie above `count` after a reset)
         if (fixed_slot < 0 && (slot < 0 || slot >= count)) {
@@ -301,9 +308,8 @@ __global__ __launch_bounds__(kWG) void k_rows_gather(IoTable t, int64_t capacity
             if (slot >= capacity) slot = capacity - 1;
         }
         if (out_indices && f == 0 && unit == 0) out_indices[row] = slot;
-        const uint32_t vl = t.vec_log2[f];
         const uint64_t off = (uint64_t)unit << vl;
-        copy_granule(as_global(t.io[f]) + row * t.row_bytes[f] + off, as_global(t.store[f]) + (uint64_t)slot * t.stride[f] + off, vl);
+        copy_granule(io + row * row_bytes + off, store + (uint64_t)slot * stride_f + off, vl);
     }
 }
 
