@@ -1208,6 +1208,26 @@ def test_out_of_domain_inputs_are_clamped_and_flagged(mrb, orc, path):
     g.destroy()
 
 
+def test_gather_of_more_granules_than_one_grid_row_holds(mrb):
+    """A gather of narrow rows whose widest field needs more workgroups than a launch's row of them may have
+    (16,384 x 256 threads, a thread per 16-byte granule): the threads go round more than once; fields of other
+    sizes end earlier. Checked against torch's own indexing of the storage."""
+    from mindrl_amd.core import PriorityReplayBuffer
+    cap, n = 3000, 170_000
+    shapes, types = [(120,), (1,), (3,)], [torch.float32, torch.int32, torch.uint8]  # 30 granules, one, three bytes
+    g = PriorityReplayBuffer(0.6, cap, 4, shapes, types, seed0=1)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    rows = [torch.randn(cap, 120, device="cuda", generator=gen), torch.arange(cap, dtype=torch.int32, device="cuda")[:, None],
+            torch.randint(0, 255, (cap, 3), dtype=torch.uint8, device="cuda", generator=gen)]
+    g.insert(*rows)
+    idx = torch.randint(0, cap, (n,), device="cuda", generator=gen)
+    got = g.gather(idx)
+    for f in range(3):
+        assert torch.equal(got[f], rows[f][idx]), f
+    g.check()
+    g.destroy()
+
+
 # ----------------------------------------------- the five benchmark configurations
 def test_config1_dqn_per_cartpole_full_loop(mrb, orc):
     """Config 1: capacity 10 000, alpha .6, beta .4, eps 1e-6; fill, then 1000 x
