@@ -1075,6 +1075,63 @@ __device__ __forceinline__ uint32_t walk8(const float4 lo, const float4 hi, floa
     return p;
 }
 
+// One dependent load of the thread-per-stratum descent: the 2^g descendants of `node` g levels down (g <= 5: at most
+// one cache line), the levels between rebuilt with the additions the tree was built with. Returns the node the
+// mass falls into, g levels down; `mass` becomes what is left of it inside that node, `picked` the node's value.
+__device__ __forceinline__ uint32_t descend_group(const float* __restrict__ sum, uint32_t node, int g, float& mass, float& picked) {
+    if (g == 5) {
+        const f32x4* src = reinterpret_cast<const f32x4*>(sum + ((uint64_t)node << 5));
+        const f32x4 t0 = src[0], t1 = src[1], t2 = src[2], t3 = src[3], t4 = src[4], t5 = src[5], t6 = src[6], t7 = src[7];
+        const f32x16 lo = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
+                                                  __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
+                                                  2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+        const f32x16 hi = __builtin_shufflevector(__builtin_shufflevector(t4, t5, 0, 1, 2, 3, 4, 5, 6, 7),
+                                                  __builtin_shufflevector(t6, t7, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
+                                                  2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+        node = (node << 5) + walk32(lo, hi, mass, picked);
+    } else if (g == 4) {
+        const f32x4* src = reinterpret_cast<const f32x4*>(sum + ((uint64_t)node << 4));
+        const f32x4 t0 = src[0], t1 = src[1], t2 = src[2], t3 = src[3];
+        const f32x16 v = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
+                                                 __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
+                                                 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+        node = (node << 4) + walk16(v, mass, picked);
+    } else if (g == 3) {
+        const float4* src = reinterpret_cast<const float4*>(sum + ((uint64_t)node << 3));
+        const float4 lo = src[0], hi = src[1];
+        node = (node << 3) + walk8(lo, hi, mass, picked);
+    } else if (g == 2) {
+        const float4 v = *reinterpret_cast<const float4*>(sum + ((uint64_t)node << 2));
+        const float left = v.x + v.y;
+        uint32_t p = 0;
+        if (!(mass <= left)) {
+            mass -= left;
+            p = 2;
+        }
+        const float n0 = p ? v.z : v.x, n1 = p ? v.w : v.y;
+        if (!(mass <= n0)) {
+            mass -= n0;
+            p += 1;
+            picked = n1;
+        } else {
+            picked = n0;
+        }
+        node = (node << 2) + p;
+    } else {
+        const float2 pair = *reinterpret_cast<const float2*>(sum + 2 * (uint64_t)node);
+        if (mass <= pair.x) {
+            node = 2 * node;
+            picked = pair.x;
+        } else {
+            mass -= pair.x;
+            node = 2 * node + 1;
+            picked = pair.y;
+        }
+    }
+    return node;
+}
+
+
 // ---------------------------------------------------------------------------
 // PER sample, many narrow rows: one workgroup per 256 strata. The top
 // `lds_levels` levels of the sum tree (nodes [1, 2 << lds_levels)) are staged
@@ -1151,55 +1208,7 @@ __global__ __launch_bounds__(kLdsWG) void k_per_sample_lds(const float* __restri
         while (d < depth) {  // wave-uniform
             const int rest = depth - d;
             const int g = rest >= 5 ? (rest == 7 ? 4 : 5) : rest;
-            if (g == 5) {
-                const f32x4* src = reinterpret_cast<const f32x4*>(sum + ((uint64_t)node << 5));
-                const f32x4 t0 = src[0], t1 = src[1], t2 = src[2], t3 = src[3], t4 = src[4], t5 = src[5], t6 = src[6], t7 = src[7];
-                const f32x16 lo = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
-                                                          __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
-                                                          2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
-                const f32x16 hi = __builtin_shufflevector(__builtin_shufflevector(t4, t5, 0, 1, 2, 3, 4, 5, 6, 7),
-                                                          __builtin_shufflevector(t6, t7, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
-                                                          2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
-                node = (node << 5) + walk32(lo, hi, mass, picked);
-            } else if (g == 4) {
-                const f32x4* src = reinterpret_cast<const f32x4*>(sum + ((uint64_t)node << 4));
-                const f32x4 t0 = src[0], t1 = src[1], t2 = src[2], t3 = src[3];
-                const f32x16 v = __builtin_shufflevector(__builtin_shufflevector(t0, t1, 0, 1, 2, 3, 4, 5, 6, 7),
-                                                         __builtin_shufflevector(t2, t3, 0, 1, 2, 3, 4, 5, 6, 7), 0, 1,
-                                                         2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
-                node = (node << 4) + walk16(v, mass, picked);
-            } else if (g == 3) {
-                const float4* src = reinterpret_cast<const float4*>(sum + ((uint64_t)node << 3));
-                const float4 lo = src[0], hi = src[1];
-                node = (node << 3) + walk8(lo, hi, mass, picked);
-            } else if (g == 2) {
-                const float4 v = *reinterpret_cast<const float4*>(sum + ((uint64_t)node << 2));
-                const float left = v.x + v.y;
-                uint32_t p = 0;
-                if (!(mass <= left)) {
-                    mass -= left;
-                    p = 2;
-                }
-                const float n0 = p ? v.z : v.x, n1 = p ? v.w : v.y;
-                if (!(mass <= n0)) {
-                    mass -= n0;
-                    p += 1;
-                    picked = n1;
-                } else {
-                    picked = n0;
-                }
-                node = (node << 2) + p;
-            } else {
-                const float2 pair = *reinterpret_cast<const float2*>(sum + 2 * (uint64_t)node);
-                if (mass <= pair.x) {
-                    node = 2 * node;
-                    picked = pair.x;
-                } else {
-                    mass -= pair.x;
-                    node = 2 * node + 1;
-                    picked = pair.y;
-                }
-            }
+            node = descend_group(sum, node, g, mass, picked);
             d += g;
         }
         const int64_t idx = (int64_t)node - ((int64_t)1 << depth);
@@ -2254,11 +2263,14 @@ constexpr int kPushOneMaxDepth = 30;
 // `taken`: this launch moves the device's counters on, `ticket` holds them as the caller took them - the position is theirs,
 // and, unless the caller has reported already (`report`), the wave's report (see counters_report) goes out behind the
 // walk's own requests, so that nothing the walk waits for queues up behind the atomic.
-template <bool kAfterUpdate>
+// kTop: the workgroup holds the latest values of nodes [1, top_nodes) of both trees in LDS (top_s, top_m) and goes on
+// using them after the walk: siblings among them are read there, and what the walk writes goes there as well.
+template <bool kAfterUpdate, bool kTop = false>
 __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp, int64_t first_slot,
                                               int64_t capacity, int64_t leaves, int depth, float alpha,
                                               const float* priority, uint32_t* err, uint32_t lane,
-                                              CounterTicket& ticket, bool taken, bool report, uint32_t readers) {
+                                              CounterTicket& ticket, bool taken, bool report, uint32_t readers,
+                                              float* top_s = nullptr, float* top_m = nullptr, uint32_t top_nodes = 0) {
     // negative: the ring position is on the device (see Counters)
     const int64_t slot = taken             ? ticket_position(ticket, capacity)
                          : first_slot >= 0 ? first_slot
@@ -2267,8 +2279,13 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
     float sib_s = 0.0f, sib_m = 0.0f;
     if (lane >= 1 && lane <= (uint32_t)depth) {
         const uint32_t node = (v >> ((uint32_t)depth - lane)) ^ 1u;
-        sib_s = sum[node];
-        sib_m = mn[node];
+        if (kTop && node < top_nodes) {
+            sib_s = top_s[node];
+            sib_m = top_m[node];
+        } else {
+            sib_s = sum[node];
+            sib_m = mn[node];
+        }
     }
     // the leaf: the running max as the call finds it, or the given priority's power (an invalid one is flagged
     // and the row takes the running max, as a plain push would give it)
@@ -2285,6 +2302,10 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
     if (lane == 0) {
         sum[node] = cs;
         mn[node] = cm;
+        if (kTop && node < top_nodes) {
+            top_s[node] = cs;
+            top_m[node] = cm;
+        }
     }
 #pragma unroll
     for (int L = kPushOneMaxDepth; L >= 1; --L) {
@@ -2297,6 +2318,10 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
             if (lane == 0) {
                 sum[node] = cs;
                 mn[node] = cm;
+                if (kTop && node < top_nodes) {
+                    top_s[node] = cs;
+                    top_m[node] = cm;
+                }
             }
         }
     }
@@ -2426,10 +2451,14 @@ __device__ __forceinline__ bool wg_resolve(const uint32_t* keys, const unsigned 
 // of a few dozen entries leaves it little else to do, while the first waves carry the entries - leaves them in
 // `ticket` (requested behind the body's own first requests, see counters_take) and reports its read once the
 // election is over, so that the report has long returned when the push looks at it (see counters_report).
+// staged_s, staged_m: where the staged top of the two trees lies in LDS, for a caller that goes on using it (every
+// node's latest value, nodes [1, 2 << min(depth, kWgTopLevels)), valid once the workgroup has passed a barrier).
 template <bool kTake>
-__device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket& ticket) {
+__device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket& ticket, float*& staged_s, float*& staged_m) {
     __shared__ __align__(16) float top_s[kWgTopNodes];
     __shared__ __align__(16) float top_m[kWgTopNodes];
+    staged_s = top_s;
+    staged_m = top_m;
     __shared__ __align__(16) uint32_t keys[3][kWgSlots];
     __shared__ __align__(16) unsigned long long vals[3][kWgSlots];
     const uint32_t tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63u;
@@ -2627,7 +2656,8 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
 
 __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
     CounterTicket none{};
-    tree_wg_body<false>(a, none);
+    float *top_s, *top_m;
+    tree_wg_body<false>(a, none, top_s, top_m);
 }
 
 // ---------------------------------------------------------------------------
@@ -2653,7 +2683,8 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(UpdateArgs a, in
     __shared__ int64_t s_position;
     const bool keeper = kDev && threadIdx.x >= blockDim.x - 64;
     CounterTicket t{};
-    tree_wg_body<kDev>(a, t);
+    float *top_s, *top_m;
+    tree_wg_body<kDev>(a, t, top_s, top_m);
     if (keeper && (threadIdx.x & 63u) == 0) s_position = ticket_position(t, a.capacity);
     __threadfence_block();
     __syncthreads();
