@@ -330,6 +330,11 @@ class PerRun:
         self._update_push_fn = self.L.mrb_per_update_push
         self._update_push_args = [(self.h, ip, self.upr[j].data_ptr(), self.upd, self.sptr, self.ins_n, self.ins_pr, self.sp)
                                   for j in range(64)]
+        # the whole step as one call: the update at the indices the previous step sampled, the push, the next sample
+        self._step_fn = self.L.mrb_per_update_push_sample
+        self._step_args = [(self.h, ip, self.upr[i % 64].data_ptr(), self.upd, self.sptr, self.ins_n, self.ins_pr, self.batch,
+                            float(self.betas[i]), base + i * self.batch * 4, ip, wp, self.fptr, self.sp)
+                           for i in range(self.n_draws)]
 
     def sample_bound(self, i):
         if self._sample_fn(*self._sample_args[i]):
@@ -344,6 +349,12 @@ class PerRun:
     def loop_fused_bound(self, i):
         """The same step with update_priorities and the push as ONE call (mrb_per_update_push)."""
         if self._sample_fn(*self._sample_args[i]) or self._update_push_fn(*self._update_push_args[i % 64]):
+            self._lib.check(1)
+
+    def loop_one_call_bound(self, i):
+        """The same step as ONE call (mrb_per_update_push_sample): the update at the rows the step before sampled,
+        the push, and the sample the next step learns from."""
+        if self._step_fn(*self._step_args[i]):
             self._lib.check(1)
 
     def sample(self, i, sp=None, out=None):
@@ -564,6 +575,8 @@ def per_extras(a, torch, r, algo_bytes):
     # the same step with update_priorities and the insert as one call (mrb_per_update_push: fewer launches)
     extras["update_push_us_per_call"] = timed(lambda i: r._update_push_fn(*r._update_push_args[i % 64])) * 1e6
     extras["loop_update_push_steps_per_s"] = 1.0 / timed(lambda i: r.loop_fused_bound(W + i % K))
+    # ... and with the sample in that call too (mrb_per_update_push_sample: one launch on a small buffer)
+    extras["loop_one_call_steps_per_s"] = 1.0 / timed(lambda i: r.loop_one_call_bound(W + i % K))
     # the same loop recorded ONCE into a HIP graph (50 steps) with the buffer's counters kept on the device, so
     # that every replay continues where the last one stopped; replayed 10 times
     if r.upd <= 1024:  # device-resident counters take updates of at most 1024 entries

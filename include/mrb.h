@@ -77,8 +77,8 @@ int mrb_backend(void);
  * compares the two before it makes any other call. History: 1 = mrb_set_option(name, value);
  * 2 = mrb_set_option(handle, name, value), mrb_per_sample_many / _next / _update_noalloc added;
  * 3 = mrb_per_update_push, mrb_field_layout and mrb_bench_launch added, library-wide options (handle 0), updates
- * of more than 1024 entries refuse stream capture. */
-#define MRB_ABI_VERSION 3
+ * of more than 1024 entries refuse stream capture; 4 = mrb_per_update_push_sample added. */
+#define MRB_ABI_VERSION 4
 int mrb_version(void);
 /* Tuning knobs of ONE buffer (any kind of handle); they change how its kernels are launched, never a
  * result. Unknown names return MRB_EINVAL. Set them while no call on the handle is in progress.
@@ -214,6 +214,21 @@ int mrb_per_update(int64_t h, const int64_t *indices, const float *priorities, i
 int mrb_per_update_push(int64_t h, const int64_t *indices, const float *priorities, int64_t n,
                         const void *const *src_fields, int64_t nrows, const float *opt_push_priorities,
                         void *stream);
+/* mrb_per_update_push(h, indices, priorities, n, src_fields, nrows, opt_push_priorities) followed by
+ * mrb_per_sample(h, batch, beta, uniforms, out_indices, out_weights, out_fields), as ONE call: a learner's whole
+ * step on the buffer - the priorities of the batch it has just used (priority_replay_buffer.py:108-120), the
+ * transition the actor has just produced (:78-90) and the batch it uses next (:92-106); the reference's loop
+ * issues the three in this order from one iteration to the next (mindspore_rl/algorithm/dqn/dqn_trainer.py:76-87).
+ * Same results, bit for bit, as the calls one after the other (the sample sees the update and the pushed row). No
+ * counterpart among the reference's primitives: on a small buffer each of the three is a launch of a few
+ * microseconds, and here they are ONE launch of one workgroup when the update has at most 384 entries, the tree at
+ * most 14 levels (capacity up to 16,384), one row is pushed, the batch has at most 512 rows of together at most
+ * 32,768 copy granules, and the buffer's counters are on the host; any other call runs as mrb_per_update_push and
+ * mrb_per_sample would. Arguments that either of them refuses are refused before anything is changed. */
+int mrb_per_update_push_sample(int64_t h, const int64_t *indices, const float *priorities, int64_t n,
+                               const void *const *src_fields, int64_t nrows, const float *opt_push_priorities,
+                               int64_t batch, float beta, const float *uniforms, int64_t *out_indices,
+                               float *out_weights, void *const *out_fields, void *stream);
 /* mrb_per_update for callers that cannot allocate: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments, same result
  * bit for bit; the scratch that mrb_per_update keeps per buffer (p^alpha of the call's entries) lives

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmrb.so")
 MRB_OK, MRB_EINVAL, MRB_EHANDLE, MRB_EHIP, MRB_ESTATE, MRB_EDEVICE = 0, 1, 2, 3, 4, 5
 DERR_INDEX, DERR_PRIORITY, DERR_TOTAL, DERR_UNFILLED = 1, 2, 4, 8
 MAX_FIELDS = 16
-ABI_VERSION = 3  # MRB_ABI_VERSION of include/mrb.h this binding was written against
+ABI_VERSION = 4  # MRB_ABI_VERSION of include/mrb.h this binding was written against
 
 _vp, _i64, _u64, _f32, _int = C.c_void_p, C.c_int64, C.c_uint64, C.c_float, C.c_int
 _pvp = C.POINTER(C.c_void_p)
@@ -44,6 +44,7 @@ SIGNATURES = {
     "mrb_per_gather": [_i64, _vp, _i64, _pvp, _vp],
     "mrb_per_update": [_i64, _vp, _vp, _i64, _vp],
     "mrb_per_update_push": [_i64, _vp, _vp, _i64, _pvp, _i64, _vp, _vp],
+    "mrb_per_update_push_sample": [_i64, _vp, _vp, _i64, _pvp, _i64, _vp, _i64, _f32, _vp, _vp, _vp, _pvp, _vp],
     "mrb_per_update_noalloc": [_i64, _vp, _vp, _i64, _vp],
     "mrb_per_export_tree": [_i64, _vp, _vp, _pi64, _vp],
     "mrb_per_state": [_i64, _pi64, _pi64, C.POINTER(C.c_float), _vp],

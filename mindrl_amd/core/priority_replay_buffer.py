@@ -208,6 +208,55 @@ class PriorityReplayBuffer:
         self._keep = (idx, pr, src, ipr)
         return self._handle
 
+    def update_priorities_insert_and_sample(self, indices, priorities, *transition, beta, insert_priorities=None,
+                                            uniforms=None, out=None):
+        """update_priorities(indices, priorities), insert(*transition, priorities=insert_priorities) and
+        sample(beta, uniforms, out) as ONE library call (mrb_per_update_push_sample): a learner's whole step on the
+        buffer (mindspore_rl/algorithm/dqn/dqn_trainer.py:76-87 and the sample of the next iteration). The results
+        are the three calls', bit for bit; on a small buffer (capacity up to 16,384, up to 384 entries, one
+        transition, up to 512 sampled rows) they take one kernel launch instead of two or three. Returns what
+        sample() returns."""
+        idx = flat_on_device(indices, torch.int64, self._dev)
+        pr = flat_on_device(priorities, torch.float32, self._dev)
+        if idx.numel() != pr.numel():
+            raise ValueError("indices and priorities differ in length")
+        if len(transition) == 1 and isinstance(transition[0], (list, tuple)):
+            transition = tuple(transition[0])
+        n = self._layout.rows_if_ready(transition, self._dev)
+        if n is not None:
+            src = transition
+        else:
+            n = self._layout.batch_of(transition)
+            src = self._layout.to_device(transition, self._dev)
+        ipr = None
+        if insert_priorities is not None:
+            ipr = flat_on_device(insert_priorities, torch.float32, self._dev)
+            if ipr.numel() != n:
+                raise ValueError("insert_priorities must hold one value per pushed row")
+        b = self._sample_size
+        u = None
+        if uniforms is not None:
+            u = flat_on_device(uniforms, torch.float32, self._dev)
+            if u.numel() != b:
+                raise ValueError("uniforms must hold sample_size = %d values" % b)
+        if out is not None:
+            oidx, w, fields = out
+            fields = self._layout.check_out(fields, b, self._dev)
+            fptr = pointers(fields)
+        elif self._ring_size > 0:
+            oidx, w, fields, fptr = self._next_outputs()
+        else:
+            oidx = torch.empty(b, dtype=torch.int64, device=self._dev)
+            w = torch.empty(b, dtype=torch.float32, device=self._dev)
+            fields = self._layout.empty(b, self._dev)
+            fptr = pointers(fields)
+        _lib.check(_lib.lib().mrb_per_update_push_sample(
+            self._h, idx.data_ptr(), pr.data_ptr(), idx.numel(), pointers(src), n,
+            ipr.data_ptr() if ipr is not None else None, b, float(beta), u.data_ptr() if u is not None else None,
+            oidx.data_ptr(), w.data_ptr(), fptr, stream_ptr()))
+        self._keep = (idx, pr, src, ipr, u)
+        return (oidx, w) + tuple(fields)
+
     def gather(self, indices, out=None):
         """Rows at the given slots (int64, each in [0, size)): one [n, *shape_i] tensor per field.
         For transitions that store the slot of their successor instead of a copy of it, e.g.

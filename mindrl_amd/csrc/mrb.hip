@@ -1457,6 +1457,64 @@ int mrb_per_sample_many(int64_t h, int64_t nbatch, int64_t batch, float beta, co
                            static_cast<hipStream_t>(stream));
 }
 
+int mrb_per_update_push_sample(int64_t h, const int64_t* indices, const float* priorities, int64_t n,
+                               const void* const* src_fields, int64_t nrows, const float* opt_push_priorities,
+                               int64_t batch, float beta, const float* uniforms, int64_t* out_indices,
+                               float* out_weights, void* const* out_fields, void* stream) {
+    GET_PER(b, h);
+    // (everything the three calls would refuse is refused before the first of them runs)
+    if (n <= 0) return fail(MRB_EINVAL, "n %lld must be positive", (long long)n);
+    if (!indices || !priorities) return fail(MRB_EINVAL, "indices or priorities is NULL");
+    if (nrows <= 0) return fail(MRB_EINVAL, "nrows %lld must be positive", (long long)nrows);
+    if (!src_fields) return fail(MRB_EINVAL, "field pointer array is NULL");
+    if (batch <= 0 || batch > (1ll << 24)) return fail(MRB_EINVAL, "batch %lld outside [1, 2^24]", (long long)batch);
+    if (!out_indices || !out_weights) return fail(MRB_EINVAL, "out_indices or out_weights is NULL");
+    IoTable t;
+    int rc = make_table(b->rows, out_fields, batch, t);
+    if (rc) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t cap = b->rows.capacity;
+    // one launch of one workgroup: the update of at most 384 entries on a tree of at most 14 levels, one row, a batch
+    // of at most a thread per stratum, and rows small enough for one workgroup to copy; the counters on the host
+    if (b->fused && !b->device_counters && b->sample_path == 0 && nrows == 1 && n <= kWgBestEntries && b->depth >= 2 &&
+        b->depth <= kWgMaxDepth && batch <= kStepThreads) {
+        PutArgs put{};
+        const int64_t first = b->pushes % cap;
+        rc = put_args(b->rows, src_fields, 0, 1, first, put);
+        if (rc) return rc;
+        if (put.t.prefix[put.t.nfields] <= kStepMaxPut && t.prefix[t.nfields] <= kStepMaxGather) {
+            rc = next_epoch(*b, s);
+            if (rc) return rc;
+            UpdateArgs a = update_args(*b);
+            a.indices = indices;
+            a.priorities = priorities;
+            a.n = n;
+            StepLate late{};
+            late.err = b->err;
+            late.priority = opt_push_priorities;
+            late.uniforms = uniforms;
+            late.out_idx = out_indices;
+            late.out_w = out_weights;
+            late.size = b->size + 1 < cap ? b->size + 1 : cap;  // as the push leaves it
+            late.seed = b->seed;
+            late.calls = b->calls;
+            late.beta = beta;
+            late.put = put.t;
+            late.get = t;
+            hipLaunchKernelGGL(k_tree_wg_push_sample, dim3(1), dim3(kStepThreads), 0, s, indices, priorities, b->sum, b->mn,
+                               a.maxp, (int)(cap << 16 | first), (int)(n << 18 | batch << 8) | b->depth, a.alpha, late);
+            LAUNCH_CHECK("k_tree_wg_push_sample");
+            b->pushes += 1;
+            b->size = late.size;
+            if (!uniforms) b->calls += 1;
+            return MRB_OK;
+        }
+    }
+    rc = mrb_per_update_push(h, indices, priorities, n, src_fields, nrows, opt_push_priorities, stream);
+    if (rc) return rc;
+    return per_sample_impl(b.get(), 1, batch, beta, uniforms, out_indices, out_weights, out_fields, s);
+}
+
 int mrb_per_sample_next(int64_t h, int64_t batch, float beta, const float* uniforms, int slot_field, int row_field,
                         int64_t* out_indices, float* out_weights, void* const* out_fields, void* out_next_rows,
                         void* stream) {

@@ -228,6 +228,13 @@ __device__ __forceinline__ float dpp_move(float x) {
     return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), CTRL, 0xF, 0xF, true));
 }
 
+// What lane + N of the same row of 16 lanes holds in x; `fill` in the lanes whose row has no such lane.
+template <int N>
+__device__ __forceinline__ float row_lane_above(float x, float fill) {
+    static_assert(N >= 1 && N <= 15, "within a row of 16 lanes");
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(x), 0x100 + N, 0xF, 0xF, false));
+}
+
 __device__ __forceinline__ float lane_value(float x, uint32_t src_lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), (int)src_lane));
 }

@@ -1075,6 +1075,34 @@ __device__ __forceinline__ uint32_t walk8(const float4 lo, const float4 hi, floa
     return p;
 }
 
+// Two levels, and one, of the same descent.
+__device__ __forceinline__ uint32_t walk4(const float4 v, float& mass, float& picked) {
+    const float left = v.x + v.y;
+    uint32_t p = 0;
+    if (!(mass <= left)) {
+        mass -= left;
+        p = 2;
+    }
+    const float n0 = p ? v.z : v.x, n1 = p ? v.w : v.y;
+    if (!(mass <= n0)) {
+        mass -= n0;
+        p += 1;
+        picked = n1;
+    } else {
+        picked = n0;
+    }
+    return p;
+}
+__device__ __forceinline__ uint32_t walk2(const float2 pair, float& mass, float& picked) {
+    if (mass <= pair.x) {
+        picked = pair.x;
+        return 0;
+    }
+    mass -= pair.x;
+    picked = pair.y;
+    return 1;
+}
+
 // One dependent load of the thread-per-stratum descent: the 2^g descendants of `node` g levels down (g <= 5: at most
 // one cache line), the levels between rebuilt with the additions the tree was built with. Returns the node the
 // mass falls into, g levels down; `mass` becomes what is left of it inside that node, `picked` the node's value.
@@ -1102,31 +1130,10 @@ __device__ __forceinline__ uint32_t descend_group(const float* __restrict__ sum,
         node = (node << 3) + walk8(lo, hi, mass, picked);
     } else if (g == 2) {
         const float4 v = *reinterpret_cast<const float4*>(sum + ((uint64_t)node << 2));
-        const float left = v.x + v.y;
-        uint32_t p = 0;
-        if (!(mass <= left)) {
-            mass -= left;
-            p = 2;
-        }
-        const float n0 = p ? v.z : v.x, n1 = p ? v.w : v.y;
-        if (!(mass <= n0)) {
-            mass -= n0;
-            p += 1;
-            picked = n1;
-        } else {
-            picked = n0;
-        }
-        node = (node << 2) + p;
+        node = (node << 2) + walk4(v, mass, picked);
     } else {
         const float2 pair = *reinterpret_cast<const float2*>(sum + 2 * (uint64_t)node);
-        if (mass <= pair.x) {
-            node = 2 * node;
-            picked = pair.x;
-        } else {
-            mass -= pair.x;
-            node = 2 * node + 1;
-            picked = pair.y;
-        }
+        node = 2 * node + walk2(pair, mass, picked);
     }
     return node;
 }
@@ -2263,14 +2270,11 @@ constexpr int kPushOneMaxDepth = 30;
 // `taken`: this launch moves the device's counters on, `ticket` holds them as the caller took them - the position is theirs,
 // and, unless the caller has reported already (`report`), the wave's report (see counters_report) goes out behind the
 // walk's own requests, so that nothing the walk waits for queues up behind the atomic.
-// kTop: the workgroup holds the latest values of nodes [1, top_nodes) of both trees in LDS (top_s, top_m) and goes on
-// using them after the walk: siblings among them are read there, and what the walk writes goes there as well.
-template <bool kAfterUpdate, bool kTop = false>
+template <bool kAfterUpdate>
 __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp, int64_t first_slot,
                                               int64_t capacity, int64_t leaves, int depth, float alpha,
                                               const float* priority, uint32_t* err, uint32_t lane,
-                                              CounterTicket& ticket, bool taken, bool report, uint32_t readers,
-                                              float* top_s = nullptr, float* top_m = nullptr, uint32_t top_nodes = 0) {
+                                              CounterTicket& ticket, bool taken, bool report, uint32_t readers) {
     // negative: the ring position is on the device (see Counters)
     const int64_t slot = taken             ? ticket_position(ticket, capacity)
                          : first_slot >= 0 ? first_slot
@@ -2279,13 +2283,8 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
     float sib_s = 0.0f, sib_m = 0.0f;
     if (lane >= 1 && lane <= (uint32_t)depth) {
         const uint32_t node = (v >> ((uint32_t)depth - lane)) ^ 1u;
-        if (kTop && node < top_nodes) {
-            sib_s = top_s[node];
-            sib_m = top_m[node];
-        } else {
-            sib_s = sum[node];
-            sib_m = mn[node];
-        }
+        sib_s = sum[node];
+        sib_m = mn[node];
     }
     // the leaf: the running max as the call finds it, or the given priority's power (an invalid one is flagged
     // and the row takes the running max, as a plain push would give it)
@@ -2302,10 +2301,6 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
     if (lane == 0) {
         sum[node] = cs;
         mn[node] = cm;
-        if (kTop && node < top_nodes) {
-            top_s[node] = cs;
-            top_m[node] = cm;
-        }
     }
 #pragma unroll
     for (int L = kPushOneMaxDepth; L >= 1; --L) {
@@ -2318,10 +2313,6 @@ __device__ __forceinline__ void push_one_walk(float* sum, float* mn, float* maxp
             if (lane == 0) {
                 sum[node] = cs;
                 mn[node] = cm;
-                if (kTop && node < top_nodes) {
-                    top_s[node] = cs;
-                    top_m[node] = cm;
-                }
             }
         }
     }
@@ -2428,6 +2419,19 @@ __device__ __forceinline__ uint32_t wg_claim(uint32_t* keys, uint32_t node) {
         slot = (slot + 1) & (kWgSlots - 1);
     }
 }
+// The same in two halves, for a caller with arithmetic to do while the first attempt is on its way: `found` is what
+// wg_claim_first's attempt on the node's home slot returned.
+__device__ __forceinline__ uint32_t wg_claim_first(uint32_t* keys, uint32_t node) {
+    return atomicCAS(&keys[wg_hash(node)], 0u, node);
+}
+__device__ __forceinline__ uint32_t wg_claim_rest(uint32_t* keys, uint32_t node, uint32_t found) {
+    uint32_t slot = wg_hash(node);
+    while (!(found == 0u || found == node)) {
+        slot = (slot + 1) & (kWgSlots - 1);
+        found = atomicCAS(&keys[slot], 0u, node);
+    }
+    return slot;
+}
 
 // One probe of a lookup, its reads issued by the caller (so that several lookups' reads travel together):
 // `key` and `val` are what the table holds at `slot`. Returns whether the call has changed `node`; then
@@ -2453,15 +2457,46 @@ __device__ __forceinline__ bool wg_resolve(const uint32_t* keys, const unsigned 
 // election is over, so that the report has long returned when the push looks at it (see counters_report).
 // staged_s, staged_m: where the staged top of the two trees lies in LDS, for a caller that goes on using it (every
 // node's latest value, nodes [1, 2 << min(depth, kWgTopLevels)), valid once the workgroup has passed a barrier).
-template <bool kTake>
-__device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket& ticket, float*& staged_s, float*& staged_m) {
+// What a kernel that goes on after the update (k_tree_wg_push_sample) takes from it through LDS instead of
+// reading memory again: the largest p^alpha of the update's entries, and the update's values of the nodes beside
+// the path of the leaf that the kernel writes next - those below the staged top, where LDS does not hold the tree
+// ([i]: the node i levels above the leaf level).
+struct StepShared {
+    uint32_t flags;  // MRB_DERR_* of the update's entries
+    uint32_t qmax;   // as bits; 0: no valid entry
+    uint32_t watch_set[4];
+    float watch_s[4], watch_m[4];
+    float leaf_value;  // (the other way: the written leaf's value, for the sample that follows)
+    float max_w;       // the weights' common denominator, by a wave that does not sample
+};
+
+__device__ __forceinline__ void top_write_back(const UpdateArgs& a, const float* top_s, const float* top_m, uint32_t nthreads) {
+    const int T = a.depth < kWgTopLevels ? a.depth : kWgTopLevels;
+    const uint32_t top_vec = 1u << (T - 1);
+#pragma unroll
+    for (int j = 0; j < kWgPieces; ++j) {
+        const uint32_t i = threadIdx.x + j * nthreads;
+        if (i < top_vec) {
+            reinterpret_cast<f32x4*>(a.sum)[i] = reinterpret_cast<const f32x4*>(top_s)[i];
+            reinterpret_cast<f32x4*>(a.mn)[i] = reinterpret_cast<const f32x4*>(top_m)[i];
+        }
+    }
+}
+
+// kStep: the caller goes on with the staged top and writes it back itself (top_write_back); `step` (zeroed by the
+// caller before the workgroup's first barrier) receives what StepShared describes, watch_leaf being the heap
+// number of the leaf the caller writes next.
+template <bool kTake, bool kStep = false>
+__device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket& ticket, float*& staged_s, float*& staged_m,
+                                             StepShared* step = nullptr, uint32_t watch_leaf = 0) {
     __shared__ __align__(16) float top_s[kWgTopNodes];
     __shared__ __align__(16) float top_m[kWgTopNodes];
     staged_s = top_s;
     staged_m = top_m;
     __shared__ __align__(16) uint32_t keys[3][kWgSlots];
     __shared__ __align__(16) unsigned long long vals[3][kWgSlots];
-    const uint32_t tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63u;
+    // (kStep: a fixed number of threads - the launch's own is a read of the kernel-argument segment)
+    const uint32_t tid = threadIdx.x, nthreads = kStep ? (uint32_t)kWgMinThreads : blockDim.x, lane = tid & 63u;
     const int D = a.depth;                                // 2 .. kWgMaxDepth
     const int T = D < kWgTopLevels ? D : kWgTopLevels;    // the staged top ends at level T
     const int H = D - T;                                  // levels below it
@@ -2475,6 +2510,10 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
         idx = a.indices[tid];
         p = a.priorities[tid];
     }
+    // the running max as the kernel finds it, for the test that spares the atomic below (see raise_max; the max only
+    // grows, so an older value spares no atomic that matters - and read now it is no round trip behind the power)
+    // (a vector load: a scalar one would be waited for by the next barrier's wait for LDS)
+    const float seen_max = __uint_as_float(__hip_atomic_load(reinterpret_cast<unsigned int*>(a.maxp), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     // the top of both trees, on its way while the entries arrive
     const uint32_t top_vec = 1u << (T - 1);  // 16-byte pieces per tree: (2 << T) / 4, at most kWgPieces * kWgMinThreads
     f32x4 st_s[kWgPieces], st_m[kWgPieces];
@@ -2496,8 +2535,13 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
     }
     lds_barrier();
     const bool idx_ok = idx >= 0 && idx < a.capacity, p_ok = valid_priority(p);
-    if (__any(have && !idx_ok) && lane == 0) atomicOr(a.err, MRB_DERR_INDEX);
-    if (__any(have && !p_ok) && lane == 0) atomicOr(a.err, MRB_DERR_PRIORITY);
+    if (kStep) {  // (the caller raises the flags: it has not read the buffer's flag word's address yet)
+        if (__any(have && !idx_ok) && lane == 0) atomicOr(&step->flags, (uint32_t)MRB_DERR_INDEX);
+        if (__any(have && !p_ok) && lane == 0) atomicOr(&step->flags, (uint32_t)MRB_DERR_PRIORITY);
+    } else {
+        if (__any(have && !idx_ok) && lane == 0) atomicOr(a.err, MRB_DERR_INDEX);
+        if (__any(have && !p_ok) && lane == 0) atomicOr(a.err, MRB_DERR_PRIORITY);
+    }
     const bool valid = have && idx_ok && p_ok;
     const uint32_t leaf_node = (uint32_t)a.leaves + (uint32_t)(valid ? idx : 0);
     // memory's values of the nodes the steps below the top may need: requested now, used when the call has
@@ -2524,15 +2568,19 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
         }
     }
     if (kTake && tid >= nthreads - 64) ticket = counters_take(a.err);
+    // the election's first step: a slot for the entry's leaf (the attempt is on its way during the power)
+    uint32_t found = 0;
+    if (valid) found = wg_claim_first(keys[0], leaf_node);
     // the power, while all of that is on its way; every valid entry's counts for the running max, also that
     // of an entry that loses its leaf
     const float q = valid ? powf_det(p, a.alpha) : 0.0f;
     const float qmax = wave_max(q);
-    if (lane == 0 && qmax > 0.0f) raise_max(a.maxp, qmax);
+    if (lane == 0 && qmax > seen_max) atomicMax(reinterpret_cast<unsigned int*>(a.maxp), __float_as_uint(qmax));
+    if (kStep && lane == 0 && qmax > 0.0f) atomicMax(&step->qmax, __float_as_uint(qmax));
     // the election: the latest entry aimed at a leaf owns it
     uint32_t slot = 0;
     if (valid) {
-        slot = wg_claim(keys[0], leaf_node);
+        slot = wg_claim_rest(keys[0], leaf_node, found);
         atomicMax(&vals[0][slot], ((unsigned long long)tid << 32) | __float_as_uint(q));
     }
     // the staged top goes into LDS (needed only after several more barriers)
@@ -2556,9 +2604,15 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
             const uint32_t* kt = keys[s % 3];
             const unsigned long long* vt = vals[s % 3];
             const bool two = s > 0 || h_first == 2;
+            const int up = s == 0 ? 0 : h_first + 2 * (s - 1);  // levels between v and the leaves
             if (act) {
                 a.sum[v] = cs;
                 a.mn[v] = cm;
+                if (kStep && (v ^ 1u) == (watch_leaf >> up)) {
+                    step->watch_s[up] = cs;
+                    step->watch_m[up] = cm;
+                    step->watch_set[up] = 1u;
+                }
                 const uint32_t sib = v ^ 1u, c0 = ((v >> 1) ^ 1u) << 1, c1 = c0 | 1u;
                 const uint32_t h0 = wg_hash(sib), h1 = wg_hash(c0), h2 = wg_hash(c1);
                 const uint32_t k0 = kt[h0], k1 = two ? kt[h1] : 0u, k2 = two ? kt[h2] : 0u;
@@ -2584,6 +2638,11 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
                     if (!(right && d_sib)) {  // the lower changed child stores the parent
                         a.sum[par] = ps;
                         a.mn[par] = pm;
+                        if (kStep && (par ^ 1u) == (watch_leaf >> (up + 1))) {
+                            step->watch_s[up + 1] = ps;
+                            step->watch_m[up + 1] = pm;
+                            step->watch_set[up + 1] = 1u;
+                        }
                     }
                     const bool pright = (par & 1u) != 0;
                     cs = pright ? us + ps : ps + us;
@@ -2643,15 +2702,10 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
         top_s[v] = cs;
         top_m[v] = cm;
     }
+    // (kStep: the update's stores are performed before the caller's - to the same nodes, possibly - are issued)
+    if (kStep) __builtin_amdgcn_s_waitcnt(0);
     lds_barrier();
-#pragma unroll
-    for (int j = 0; j < kWgPieces; ++j) {
-        const uint32_t i = tid + j * nthreads;
-        if (i < top_vec) {
-            reinterpret_cast<f32x4*>(a.sum)[i] = reinterpret_cast<const f32x4*>(top_s)[i];
-            reinterpret_cast<f32x4*>(a.mn)[i] = reinterpret_cast<const f32x4*>(top_m)[i];
-        }
-    }
+    if (!kStep) top_write_back(a, top_s, top_m, nthreads);
 }
 
 __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
@@ -2701,6 +2755,398 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(UpdateArgs a, in
         counters_settle(t, a.err, a.advance, a.capacity, a.readers, threadIdx.x & 63u);
     }
 }
+// ---------------------------------------------------------------------------
+// A learner's whole step on a small buffer in ONE launch of ONE workgroup (mrb_per_update_push_sample): the
+// priorities of the batch it has just used, the transition the actor has just produced, and the batch it uses
+// next - update_priorities, insert and sample of the reference's loop (mindspore_rl/algorithm/dqn/dqn_trainer.py:76-87
+// with the sample of the following iteration). Every one of the three is a launch of a few microseconds whose
+// kernel works for a fraction of that; here the update's staged top of both trees stays in LDS, the walk of the
+// pushed row reads and patches it there, and the sample's strata descend through it - a thread per stratum, three
+// levels per LDS read, the levels below the staged top with one load from memory - and gather their rows.
+// The workgroup copies the pushed row itself: the sample may pick it.
+// The results are those of the three calls, bit for bit.
+// ---------------------------------------------------------------------------
+constexpr int kStepThreads = kWgMinThreads;  // most entries, most strata
+constexpr uint32_t kStepMaxPut = 2 * 64;  // most granules of the pushed row, which one wave copies
+constexpr uint32_t kStepMaxGather = 64 * kStepThreads;  // most granules of the sampled batch
+
+// A field table in LDS: the kernel-argument segment is not cached across launches, and a lookup in it by a thread's
+// own field number is a memory round trip; two waves request the tables when the kernel starts and put them into
+// LDS when the update is through.
+struct LdsTable {
+    uint8_t* store[MRB_MAX_FIELDS];
+    uint8_t* io[MRB_MAX_FIELDS];
+    uint32_t row_bytes[MRB_MAX_FIELDS], stride[MRB_MAX_FIELDS], units[MRB_MAX_FIELDS], vec_log2[MRB_MAX_FIELDS];
+    uint64_t prefix[MRB_MAX_FIELDS + 1];
+};
+
+// Granule w of a table's work (fields one after the other, rows within a field, granules within a row): its field,
+// row and byte offset in the row.
+__device__ __forceinline__ int wg_locate(const LdsTable& l, int nfields, uint32_t w, uint32_t& row, uint32_t& off) {
+    int f = 0;
+    while (f + 1 < nfields && w >= (uint32_t)l.prefix[f + 1]) ++f;
+    const uint32_t local = w - (uint32_t)l.prefix[f], units = l.units[f];
+    row = local / units;
+    off = (local - row * units) << l.vec_log2[f];
+    return f;
+}
+
+// The walk of the pushed row's leaf to the root by one wave, lane L holding the sibling at level L as in
+// push_one_walk - but nothing is read from memory after the update: the siblings inside the staged top are read
+// in LDS, those below it were requested when the kernel started (sib_s, sib_m: memory's values BEFORE the update)
+// and are replaced by the update's where it has changed them (StepShared); the running max is the one the kernel
+// found (old_max) raised by the update's entries. Lane L ends up with the path's node at level L and stores it -
+// inside the staged top to LDS only (the workgroup writes the top back), below it to memory -, the leaf's value is
+// left in LDS for the sample. The sums are the chain of single additions from the leaf up (an addition gives the
+// same bits whichever operand is the left child), one lane picking up each; the minima do not depend on the order
+// they are taken in: lane L's is the least of the leaf and the siblings at the levels below L, a scan over the
+// lanes of a row (depth <= kWgMaxDepth < 16).
+// q: the leaf's value when the row comes with a valid priority of its own (`given`), else the running max is taken.
+__device__ __forceinline__ void step_walk(const UpdateArgs& a, uint32_t leaf_node, uint32_t sib_node, float sib_s, float sib_m,
+                                          float old_max, bool given, float q, float* top_s, float* top_m,
+                                          uint32_t top_nodes, StepShared& step, uint32_t lane) {
+    const int depth = a.depth;
+    const bool holds = lane >= 1 && lane <= (uint32_t)depth;
+    if (holds) {
+        if (sib_node < top_nodes) {
+            sib_s = top_s[sib_node];
+            sib_m = top_m[sib_node];
+        } else {
+            const uint32_t up = (uint32_t)depth - lane;
+            if (step.watch_set[up]) {
+                sib_s = step.watch_s[up];
+                sib_m = step.watch_m[up];
+            }
+        }
+    }
+    if (!given) {
+        const uint32_t ob = __float_as_uint(old_max), ub = step.qmax;
+        q = __uint_as_float(ob > ub ? ob : ub);  // (non-negative floats order like their bits)
+    }
+    if (lane == 0) step.leaf_value = q;
+    // minima: y = the least sibling at this lane's level or below, then the lane above's y against the leaf
+    const float inf = __builtin_inff();
+    float y = holds ? sib_m : inf;
+    y = fminf(y, row_lane_above<1>(y, inf));
+    y = fminf(y, row_lane_above<2>(y, inf));
+    y = fminf(y, row_lane_above<4>(y, inf));
+    y = fminf(y, row_lane_above<8>(y, inf));
+    const float cm = fminf(q, row_lane_above<1>(y, inf));
+    // sums: lane L - 1 keeps the chain's value after the sibling at level L has been added
+    float chain = q, cs = q;
+#pragma unroll
+    for (int L = kWgMaxDepth; L >= 1; --L) {
+        if (L <= depth) {  // wave-uniform
+            chain = chain + lane_value(sib_s, L);
+            cs = lane == (uint32_t)(L - 1) ? chain : cs;
+        }
+    }
+    if (lane <= (uint32_t)depth) {
+        const uint32_t node = leaf_node >> ((uint32_t)depth - lane);
+        if (node < top_nodes) {
+            top_s[node] = cs;
+            top_m[node] = cm;
+        } else {
+            a.sum[node] = cs;
+            a.mn[node] = cm;
+        }
+    }
+    if (given && lane == 0 && q > 0.0f) raise_max(a.maxp, q);
+}
+
+// What the kernel needs only when the update is through: read from the kernel-argument segment then, not before.
+// (A scalar read of that segment ahead of a barrier would make the barrier's wait for LDS wait for the read as
+// well - the two share a counter -, and the segment's first read is a memory round trip of a microsecond.)
+struct StepLate {
+    uint32_t* err;          // the buffer's flag word
+    const float* priority;  // the pushed row's priority, or NULL: the running max
+    const float* uniforms;  // the sample's draws, or NULL: the generator (seed, calls)
+    int64_t* out_idx;
+    float* out_w;
+    int64_t size;           // rows stored once the row is pushed
+    uint64_t seed, calls;
+    float beta;
+    IoTable put, get;       // the pushed row (io: the caller's row), the sampled batch (io: the caller's outputs)
+};
+// The kernel's arguments as the segment holds them.
+struct StepKernarg {
+    const int64_t* indices;
+    const float* priorities;
+    float *sum, *mn, *maxp;
+    int slot_capacity, sizes;
+    float alpha;
+    StepLate late;
+};
+using StepKernargPtr = const __attribute__((address_space(1))) StepKernarg*;
+
+__device__ __forceinline__ StepKernargPtr step_kernarg(bool not_before_here) {
+    uint64_t bits = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
+    if (not_before_here) asm volatile("" : "+s"(bits));  // what is read through the result is requested after this point
+    return (StepKernargPtr)bits;
+}
+
+// The sample, first half: a thread per stratum descends - through the staged top in LDS, three levels per read, and
+// through the at most three levels below it with one load of the leaves under its node, among which the leaf
+// written by this launch is replaced by its value from LDS (its store may still be on its way) - and leaves the
+// slot in LDS. Returns the index; `picked` receives the leaf's value.
+__device__ __forceinline__ int64_t wg_descend(const float* top_s, int top_levels, const float* sum, int depth, int64_t capacity,
+                                              uint32_t batch, float u, uint32_t leaf_node, float leaf_value, float& picked,
+                                              int64_t* s_slot) {
+    const uint32_t tid = threadIdx.x;
+    const float total = top_s[1];
+    float mass = (u + (float)tid) * (total / (float)batch);  // each operation rounded once
+    uint32_t node = 1;
+    int d = 0;
+    picked = total;
+    while (d < top_levels) {  // uniform
+        const int rest = top_levels - d, g = rest < 3 ? rest : 3;  // (four levels per read would be fewer reads and
+                                                                   // more arithmetic: slower)
+        if (g == 3) {
+            const float4 lo = *reinterpret_cast<const float4*>(top_s + ((size_t)node << 3));
+            const float4 hi = *reinterpret_cast<const float4*>(top_s + ((size_t)node << 3) + 4);
+            node = (node << 3) + walk8(lo, hi, mass, picked);
+        } else if (g == 2) {
+            node = (node << 2) + walk4(*reinterpret_cast<const float4*>(top_s + ((size_t)node << 2)), mass, picked);
+        } else {
+            node = 2 * node + walk2(*reinterpret_cast<const float2*>(top_s + 2 * (size_t)node), mass, picked);
+        }
+        d += g;
+    }
+    const int g = depth - d;  // 0 .. kWgMaxDepth - kWgTopLevels
+    if (g > 0) {
+        const uint32_t first = node << g, at = leaf_node - first;  // (at: the written leaf's place among the loaded ones, if below 1 << g)
+        if (g == 3) {
+            float4 lo = *reinterpret_cast<const float4*>(sum + first), hi = *reinterpret_cast<const float4*>(sum + first + 4);
+            lo.x = at == 0 ? leaf_value : lo.x;
+            lo.y = at == 1 ? leaf_value : lo.y;
+            lo.z = at == 2 ? leaf_value : lo.z;
+            lo.w = at == 3 ? leaf_value : lo.w;
+            hi.x = at == 4 ? leaf_value : hi.x;
+            hi.y = at == 5 ? leaf_value : hi.y;
+            hi.z = at == 6 ? leaf_value : hi.z;
+            hi.w = at == 7 ? leaf_value : hi.w;
+            node = first + walk8(lo, hi, mass, picked);
+        } else if (g == 2) {
+            float4 v = *reinterpret_cast<const float4*>(sum + first);
+            v.x = at == 0 ? leaf_value : v.x;
+            v.y = at == 1 ? leaf_value : v.y;
+            v.z = at == 2 ? leaf_value : v.z;
+            v.w = at == 3 ? leaf_value : v.w;
+            node = first + walk4(v, mass, picked);
+        } else {
+            float2 v = *reinterpret_cast<const float2*>(sum + first);
+            v.x = at == 0 ? leaf_value : v.x;
+            v.y = at == 1 ? leaf_value : v.y;
+            node = first + walk2(v, mass, picked);
+        }
+    }
+    const int64_t idx = (int64_t)node - ((int64_t)1 << depth);
+    s_slot[tid] = idx < capacity ? idx : capacity - 1;
+    return idx;
+}
+
+// One granule of a copy: where it comes from, where it goes, its size.
+struct GranulePlace {
+    const gbyte* src;
+    gbyte* dst;
+    uint32_t vl;
+};
+
+// Sixteen 32-bit words are preloaded into scalar registers, two of them the segment's address: the fourteen leading
+// parameters are what the update needs first (the numbers among them packed: slot_capacity = capacity << 16 | slot,
+// sizes = n << 18 | batch << 8 | depth), so that its first requests go out when a wave starts.
+__global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int64_t* __restrict__ indices,
+                                                                      const float* __restrict__ priorities, float* sum, float* mn,
+                                                                      float* maxp, int slot_capacity, int sizes, float alpha,
+                                                                      StepLate late_args) {
+    __shared__ int64_t s_slot[kStepThreads];
+    __shared__ LdsTable s_put, s_get;
+    __shared__ StepShared s_step;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    // the last wave holds no entry of the update (n <= 384) and walks for the push, the one before it copies the row
+    const bool walker = tid >= kStepThreads - 64, putter = !walker && tid >= kStepThreads - 128;
+    const int depth = sizes & 255;
+    const uint32_t batch = ((uint32_t)sizes >> 8) & 1023u;
+    const int64_t slot = slot_capacity & 0xffff, capacity = (uint32_t)slot_capacity >> 16;
+    const int top_levels = depth < kWgTopLevels ? depth : kWgTopLevels;
+    const uint32_t top_nodes = 2u << top_levels, leaf_node = (1u << depth) + (uint32_t)slot;
+    UpdateArgs a{};
+    a.indices = indices;
+    a.priorities = priorities;
+    a.n = (uint32_t)sizes >> 18;
+    a.sum = sum;
+    a.mn = mn;
+    a.maxp = maxp;
+    a.depth = depth;
+    a.leaves = (int64_t)1 << depth;
+    a.capacity = capacity;
+    a.alpha = alpha;
+    // what depends on nothing before it is requested with the update's first loads: the tables (by vector loads, which
+    // no barrier of the update waits for, and held in registers until the update is through) and the walking wave's
+    // view of the tree below the staged top as the update finds it
+    // ... and the few pointers the waves need as soon as the update is through (also by vector loads: through an
+    // offset the compiler cannot see through, or it would make them scalar ones)
+    uint32_t opaque_zero = 0;
+    asm volatile("" : "+v"(opaque_zero));
+    const StepKernargPtr early = step_kernarg(false);
+    const float* const uniforms = *(&early->late.uniforms + opaque_zero);
+    const float* priority = nullptr;
+    uint32_t* err_early = nullptr;
+    float sib_s = 0.0f, sib_m = 0.0f, old_max = 0.0f;
+    uint32_t sib_node = 0;
+    uint8_t *t_store = nullptr, *t_io = nullptr;
+    uint32_t t_row_bytes = 0, t_stride = 0, t_units = 0, t_vec = 0;
+    uint64_t t_prefix = 0;
+    if (walker) {
+        if (lane >= 1 && lane <= (uint32_t)depth) {
+            sib_node = (leaf_node >> ((uint32_t)depth - lane)) ^ 1u;
+            if (sib_node >= top_nodes) {
+                sib_s = sum[sib_node];
+                sib_m = mn[sib_node];
+            }
+        }
+        old_max = __uint_as_float(__hip_atomic_load(reinterpret_cast<unsigned int*>(maxp), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        priority = *(&early->late.priority + opaque_zero);
+        err_early = *(&early->late.err + opaque_zero);
+        if (lane < 4) s_step.watch_set[lane] = 0u;
+        if (lane == 0) {
+            s_step.qmax = 0u;
+            s_step.flags = 0u;
+        }
+    }
+    if (walker || putter) {
+        const __attribute__((address_space(1))) IoTable* t = walker ? &early->late.get : &early->late.put;
+        if (lane <= MRB_MAX_FIELDS) t_prefix = t->prefix[lane];
+        if (lane < MRB_MAX_FIELDS) {
+            t_store = t->store[lane];
+            t_io = t->io[lane];
+            t_row_bytes = t->row_bytes[lane];
+            t_stride = t->stride[lane];
+            t_units = t->units[lane];
+            t_vec = t->vec_log2[lane];
+        }
+    }
+    CounterTicket none{};
+    float *top_s, *top_m;
+    tree_wg_body<false, true>(a, none, top_s, top_m, &s_step, leaf_node);  // (ends behind a barrier)
+    const StepKernargPtr ka = step_kernarg(true);
+    uint32_t* const err = ka->late.err;
+    const int put_fields = ka->late.put.nfields, get_fields = ka->late.get.nfields;
+    if (walker || putter) {
+        LdsTable* mine = walker ? &s_get : &s_put;
+        if (lane <= MRB_MAX_FIELDS) mine->prefix[lane] = t_prefix;
+        if (lane < MRB_MAX_FIELDS) {
+            mine->store[lane] = t_store;
+            mine->io[lane] = t_io;
+            mine->row_bytes[lane] = t_row_bytes;
+            mine->stride[lane] = t_stride;
+            mine->units[lane] = t_units;
+            mine->vec_log2[lane] = t_vec;
+        }
+    }
+    // the strata's draws: needed a barrier from here
+    float u = 0.0f;
+    if (tid < batch && uniforms) u = uniforms[tid];
+    if (walker) {  // from the pushed row's leaf to the root
+        float q = 0.0f;
+        bool given = false;
+        if (priority) {
+            const float p = *priority;
+            given = valid_priority(p);
+            if (!given && lane == 0) atomicOr(err_early, MRB_DERR_PRIORITY);
+            if (given) q = powf_det_call(p, alpha);
+        }
+        step_walk(a, leaf_node, sib_node, sib_s, sib_m, old_max, given, q, top_s, top_m, top_nodes, s_step, lane);
+        if (lane == 0 && s_step.flags) atomicOr(err_early, s_step.flags);
+    }
+    lds_barrier();
+    // ---- the sample's descent; the other waves find their granules' places meanwhile
+    const bool mine = tid < batch;
+    const float total = top_s[1];
+    float picked = total;
+    int64_t idx = 0;
+    const uint64_t calls = ka->late.calls;
+    if (mine) {
+        if (!uniforms) u = rng_uniform(ka->late.seed, calls, (uint64_t)tid);
+        idx = wg_descend(top_s, top_levels, sum, depth, capacity, batch, u, leaf_node, s_step.leaf_value, picked, s_slot);
+    }
+    // the pushed row: the wave before the last requests its granules now and stores them at the end
+    constexpr int kPutPer = kStepMaxPut / 64;
+    AnyGranule put_granule[kPutPer];
+    GranulePlace put_place[kPutPer];
+    uint32_t put_work = 0;
+    if (putter) {
+        put_work = (uint32_t)s_put.prefix[put_fields];  // (its own writes to the table: no barrier needed)
+#pragma unroll
+        for (int j = 0; j < kPutPer; ++j) {
+            const uint32_t w = lane + 64u * j;
+            put_place[j].vl = 0;
+            if (w < put_work) {
+                uint32_t row, off;
+                const int f = wg_locate(s_put, put_fields, w, row, off);  // (row is 0: one row)
+                put_place[j].vl = s_put.vec_log2[f];
+                put_place[j].dst = as_global(s_put.store[f]) + (uint64_t)slot * s_put.stride[f] + off;
+                put_granule[j].load(as_global(s_put.io[f]) + off, put_place[j].vl);
+            }
+        }
+    }
+    // the weights' common denominator (pmin / total * size)^-beta: by the last wave, unless it holds strata itself
+    const int64_t size = ka->late.size;
+    const float beta = ka->late.beta;
+    const bool spare_wave = batch <= kStepThreads - 64;
+    if (spare_wave && walker) {
+        const float max_w = powf_det(top_m[1] / total * (float)size, -beta);
+        if (lane == 0) s_step.max_w = max_w;
+    }
+    // the sampled rows by granule number over the batch, dealt to the threads behind the strata's waves first
+    const uint32_t work = (uint32_t)s_get.prefix[get_fields];
+    const uint32_t behind = (batch + 63u) & ~63u;
+    const uint32_t w0 = tid >= behind ? tid - behind : tid + kStepThreads - behind;
+    uint32_t row0 = 0, off0 = 0, vl0 = 0, stride0 = 0;
+    int f0 = 0;
+    gbyte* dst0 = nullptr;
+    if (w0 < work) {
+        f0 = wg_locate(s_get, get_fields, w0, row0, off0);
+        vl0 = s_get.vec_log2[f0];
+        stride0 = s_get.stride[f0];
+        dst0 = as_global(s_get.io[f0]) + (uint64_t)row0 * s_get.row_bytes[f0] + off0;
+    }
+    lds_barrier();
+    // ---- the rows (a sampled row that is the pushed one is read where the push reads it: its store may still be on
+    // its way), the weights while they are on their way, the outputs behind them
+    AnyGranule first_granule;
+    if (w0 < work) {
+        const int64_t from = s_slot[row0];
+        const gbyte* src = from == slot ? as_global(s_put.io[f0]) + off0 : as_global(s_get.store[f0]) + (uint64_t)from * stride0 + off0;
+        first_granule.load(src, vl0);
+    }
+    float weight = 0.0f;
+    if (mine) {
+        const float max_w = spare_wave ? s_step.max_w : powf_det(top_m[1] / total * (float)size, -beta);
+        weight = powf_det(picked / total * (float)size, -beta) / max_w;
+    }
+    if (w0 < work) first_granule.store(dst0, vl0);
+    if (mine) {
+        ka->late.out_idx[tid] = idx;
+        ka->late.out_w[tid] = weight;
+        if (!(total > 0.0f) || total > 3.0e38f) atomicOr(err, MRB_DERR_TOTAL);
+        if (idx >= size) atomicOr(err, MRB_DERR_UNFILLED);
+    }
+    for (uint32_t w = w0 + kStepThreads; w < work; w += kStepThreads) {
+        uint32_t row, off;
+        const int f = wg_locate(s_get, get_fields, w, row, off);
+        const int64_t from = s_slot[row];
+        const gbyte* src = from == slot ? as_global(s_put.io[f]) + off : as_global(s_get.store[f]) + (uint64_t)from * s_get.stride[f] + off;
+        copy_granule(as_global(s_get.io[f]) + (uint64_t)row * s_get.row_bytes[f] + off, src, s_get.vec_log2[f]);
+    }
+    if (putter) {
+#pragma unroll
+        for (int j = 0; j < kPutPer; ++j)
+            if (lane + 64u * j < put_work) put_granule[j].store(put_place[j].dst, put_place[j].vl);
+    }
+    top_write_back(a, top_s, top_m, kStepThreads);  // (last: its stores are ahead of no load)
+}
+
 template <bool kDev>
 __global__ __launch_bounds__(kWG) void k_tree_paths_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
     if (__builtin_expect(blockIdx.x >= 1, 0)) {  // (the tree workgroup's code comes first: it is the one the call waits for)

@@ -1748,6 +1748,81 @@ def test_update_push_equals_update_then_push(mrb, orc, cap):
     g.destroy()
 
 
+@pytest.mark.parametrize("gen", [False, True])
+@pytest.mark.parametrize("cap,batch", [(2, 2), (3, 5), (100, 64), (3000, 48), (4096, 512), (5000, 33), (10_000, 64), (16_384, 200),
+                                       (16_385, 64), (70_000, 64), (10_000, 600)])
+def test_update_push_sample_equals_the_three_calls(mrb, orc, cap, batch, gen):
+    """mrb_per_update_push_sample against the oracle's update, push and sample, one after the other: the learner's
+    step as one call, which is one launch of one workgroup on trees of 2 to 14 levels (here 1 to 14: capacities 2 to
+    16,384) and the separate calls beyond (capacity 16,385 and 70,000, batches over 512, more than 384 entries, several
+    rows). Duplicate, invalid and out-of-range entries, entries aimed at the slot the push overwrites, a pushed
+    row that takes a new running max or a priority of its own - so large that nearly every stratum samples the
+    row pushed by the same call -, across the ring's wrap, with the caller's draws and with the buffer's generator.
+    Indices, weights, rows, both trees, the running max, size and head are compared after every call."""
+    rng = np.random.default_rng(cap * 7 + batch + gen)
+    shapes, dtypes = [(3,), (1,), (5,)], [np.float32, np.int32, np.uint8]
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=5, shapes=shapes, dtypes=dtypes)
+
+    def rows_of(n, start):
+        ids = np.arange(start, start + n)
+        return [np.repeat(ids[:, None], 3, 1).astype(np.float32), ids.astype(np.int32)[:, None],
+                (ids[:, None] + np.arange(5)[None, :]).astype(np.uint8)]
+
+    fill = max(1, cap - 5)
+    rows = rows_of(fill, 0)
+    g.insert(*to_dev(rows)), c.push(rows, fill)
+    serial = fill
+    exp_flags = 0
+    for step, (k, nrows) in enumerate([(1, 1), (64, 1), (17, 1), (300, 1), (384, 1), (385, 1), (40, 3), (64, 1), (2, 1),
+                                       (200, 1), (64, 1), (33, 1), (64, 2), (64, 1)]):
+        idx = rng.integers(0, min(cap, serial), k)
+        if step % 3 == 0 and k > 4:
+            idx[: k // 3] = idx[0]  # duplicates: the last entry wins
+        head = c.head
+        if step % 2 == 1 and k > 2:
+            idx[-1] = head  # the slot the push overwrites next: the push's value must win
+        pr = (rng.pareto(1.5, k) + 1e-6).astype(np.float32)
+        if step % 4 == 2 and k > 8:
+            pr[3] = -1.0
+            idx[5] = cap + 9
+            exp_flags |= 3
+        if step == 7:
+            pr[k // 2] = np.float32(1e5)  # a new running max that the pushed row takes, and the sample sees
+        rows = rows_of(nrows, serial)
+        serial += nrows
+        ipr = None
+        if step % 5 == 4:
+            ipr = (np.abs(rng.normal(size=nrows)) + 1e-6).astype(np.float32)
+        if step == 10:
+            ipr = np.full(nrows, 1e12, np.float32)  # the pushed row outweighs all the others together
+        u = None if gen else rng.random(batch).astype(np.float32)
+        got = g.update_priorities_insert_and_sample(
+            torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda(), *to_dev(rows), beta=0.4 + 0.05 * step,
+            insert_priorities=None if ipr is None else torch.from_numpy(ipr).cuda(),
+            uniforms=None if gen else torch.from_numpy(u).cuda())
+        ok = (idx >= 0) & (idx < cap) & np.isfinite(pr) & (pr >= 0)  # the device skips and flags the others
+        c.update(idx[ok], pr[ok])
+        pushed_at = c.head
+        c.push(rows, nrows, ipr)
+        want = c.sample(batch, 0.4 + 0.05 * step, u)
+        what = "cap %d batch %d step %d (%d entries, %d rows)" % (cap, batch, step, k, nrows)
+        assert_sample_equal(got, want, what)
+        if step == 10 and cap > 8:
+            assert np.mean(want[0] == pushed_at) > 0.5, what  # the sample did pick the row of this very call
+        assert_tree_equal(g, c, what)
+        assert g.size() == c.size and g._state()[1] == c.head, what
+        assert np.float32(g.max_priority) == np.float32(c.max_priority), what
+        if step % 4 == 3:  # the separate calls go on from the same state (the generator's counter included)
+            u2 = None if gen else rng.random(batch).astype(np.float32)
+            assert_sample_equal(g.sample(0.5, uniforms=None if gen else torch.from_numpy(u2).cuda()), c.sample(batch, 0.5, u2), what)
+    for f, (a, b) in enumerate(zip(g.storage(), [c.field(0), c.field(1), c.field(2)])):
+        assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8)), f
+    flags = C.c_uint32(0)
+    assert mrb.lib.lib().mrb_per_check(g._h, C.byref(flags), None) == 0
+    assert (flags.value & 3) == exp_flags, flags.value
+    g.destroy()
+
+
 @pytest.mark.parametrize("cap,npush,batch", [(3000, 1, 48), (10_000, 1, 64), (70_000, 1, 48), (70_000, 3, 300), (1_000_000, 4, 512),
                                              (3_000_000, 1, 40), (3_000_000, 2, 100)])
 def test_hip_graph_replays_sample_then_update_push_with_device_counters(mrb, orc, cap, npush, batch):

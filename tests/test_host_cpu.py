@@ -24,12 +24,12 @@ def declared_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = declared_symbols()
-    assert len(names) == 46
+    assert len(names) == 47
     L = _lib.lib()
     for n in names:
         assert hasattr(L, n), "libmrb.so does not export %s" % n
     assert set(_lib.SIGNATURES) | {"mrb_last_error"} == set(names)
-    assert L.mrb_backend() == 1 and L.mrb_version() == _lib.ABI_VERSION == 3
+    assert L.mrb_backend() == 1 and L.mrb_version() == _lib.ABI_VERSION == 4
 
 
 def test_status_codes_without_a_device():
@@ -100,7 +100,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
     assert sum("k_per_sample_wide" in k for k in kernels) == 8 and sum("k_rows_gather_wide" in k for k in kernels) == 4
-    assert len(kernels) == 51, sorted(kernels)
+    assert len(kernels) == 52, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)
