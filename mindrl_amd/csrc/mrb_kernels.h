@@ -2807,21 +2807,24 @@ __device__ __forceinline__ void step_walk(const UpdateArgs& a, uint32_t leaf_nod
                                           uint32_t top_nodes, StepShared& step, uint32_t lane) {
     const int depth = a.depth;
     const bool holds = lane >= 1 && lane <= (uint32_t)depth;
-    if (holds) {
-        if (sib_node < top_nodes) {
-            sib_s = top_s[sib_node];
-            sib_m = top_m[sib_node];
-        } else {
-            const uint32_t up = (uint32_t)depth - lane;
-            if (step.watch_set[up]) {
-                sib_s = step.watch_s[up];
-                sib_m = step.watch_m[up];
-            }
+    {
+        // (every LDS read is issued whether its lane needs it or not, at an index made harmless: one round trip
+        // instead of one per nested condition)
+        const bool in_top = sib_node < top_nodes;
+        const uint32_t at = in_top ? sib_node : 0u;
+        const uint32_t up = holds && !in_top ? (uint32_t)depth - lane : 0u;  // at most kWgMaxDepth - kWgTopLevels - 1
+        const float ts = top_s[at], tm = top_m[at];
+        const uint32_t changed = step.watch_set[up];
+        const float ws = step.watch_s[up], wm = step.watch_m[up];
+        const uint32_t ub = step.qmax;
+        if (holds) {
+            sib_s = in_top ? ts : changed ? ws : sib_s;
+            sib_m = in_top ? tm : changed ? wm : sib_m;
         }
-    }
-    if (!given) {
-        const uint32_t ob = __float_as_uint(old_max), ub = step.qmax;
-        q = __uint_as_float(ob > ub ? ob : ub);  // (non-negative floats order like their bits)
+        if (!given) {
+            const uint32_t ob = __float_as_uint(old_max);
+            q = __uint_as_float(ob > ub ? ob : ub);  // (non-negative floats order like their bits)
+        }
     }
     if (lane == 0) step.leaf_value = q;
     // minima: y = the least sibling at this lane's level or below, then the lane above's y against the leaf
@@ -2878,6 +2881,14 @@ struct StepKernarg {
     StepLate late;
 };
 using StepKernargPtr = const __attribute__((address_space(1))) StepKernarg*;
+
+// A read of the segment as a VECTOR load (`opaque_zero`: a zero the compiler cannot see through; with a uniform
+// address it would make the load a scalar one): a scalar read in flight makes every wait for LDS - the next barrier,
+// the next LDS read - wait for it too, the two share a counter.
+template <typename T>
+__device__ __forceinline__ T vector_read(const __attribute__((address_space(1))) T* p, uint32_t opaque_zero) {
+    return *(p + opaque_zero);
+}
 
 __device__ __forceinline__ StepKernargPtr step_kernarg(bool not_before_here) {
     uint64_t bits = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
@@ -2989,7 +3000,7 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     uint32_t opaque_zero = 0;
     asm volatile("" : "+v"(opaque_zero));
     const StepKernargPtr early = step_kernarg(false);
-    const float* const uniforms = *(&early->late.uniforms + opaque_zero);
+    const float* const uniforms = vector_read(&early->late.uniforms, opaque_zero);
     const float* priority = nullptr;
     uint32_t* err_early = nullptr;
     float sib_s = 0.0f, sib_m = 0.0f, old_max = 0.0f;
@@ -3006,8 +3017,8 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
             }
         }
         old_max = __uint_as_float(__hip_atomic_load(reinterpret_cast<unsigned int*>(maxp), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        priority = *(&early->late.priority + opaque_zero);
-        err_early = *(&early->late.err + opaque_zero);
+        priority = vector_read(&early->late.priority, opaque_zero);
+        err_early = vector_read(&early->late.err, opaque_zero);
         if (lane < 4) s_step.watch_set[lane] = 0u;
         if (lane == 0) {
             s_step.qmax = 0u;
@@ -3029,9 +3040,6 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     CounterTicket none{};
     float *top_s, *top_m;
     tree_wg_body<false, true>(a, none, top_s, top_m, &s_step, leaf_node);  // (ends behind a barrier)
-    const StepKernargPtr ka = step_kernarg(true);
-    uint32_t* const err = ka->late.err;
-    const int put_fields = ka->late.put.nfields, get_fields = ka->late.get.nfields;
     if (walker || putter) {
         LdsTable* mine = walker ? &s_get : &s_put;
         if (lane <= MRB_MAX_FIELDS) mine->prefix[lane] = t_prefix;
@@ -3044,14 +3052,25 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
             mine->vec_log2[lane] = t_vec;
         }
     }
+    // (behind the tables, and behind a use of what was requested when the kernel started: a wave's requests come back
+    // in order, and a wait for an old one that the compiler cannot tell from these would wait for these)
+    asm volatile("" ::"v"(sib_s), "v"(sib_m), "v"(old_max), "v"(priority), "v"(err_early), "v"(uniforms));
+    const StepKernargPtr ka = step_kernarg(true);
+    uint32_t* const err = vector_read(&ka->late.err, opaque_zero);
+    const int put_fields = vector_read(&ka->late.put.nfields, opaque_zero), get_fields = vector_read(&ka->late.get.nfields, opaque_zero);
+    const int64_t size = vector_read(&ka->late.size, opaque_zero);
+    const float beta = vector_read(&ka->late.beta, opaque_zero);
+    const uint64_t seed = vector_read(&ka->late.seed, opaque_zero), calls = vector_read(&ka->late.calls, opaque_zero);
+    int64_t* const out_idx = vector_read(&ka->late.out_idx, opaque_zero);
+    float* const out_w = vector_read(&ka->late.out_w, opaque_zero);
     // the strata's draws: needed a barrier from here
     float u = 0.0f;
-    if (tid < batch && uniforms) u = uniforms[tid];
+    if (tid < batch && uniforms) u = ((const __attribute__((address_space(1))) float*)uniforms)[tid];
     if (walker) {  // from the pushed row's leaf to the root
         float q = 0.0f;
         bool given = false;
         if (priority) {
-            const float p = *priority;
+            const float p = *(const __attribute__((address_space(1))) float*)priority;
             given = valid_priority(p);
             if (!given && lane == 0) atomicOr(err_early, MRB_DERR_PRIORITY);
             if (given) q = powf_det_call(p, alpha);
@@ -3065,9 +3084,8 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     const float total = top_s[1];
     float picked = total;
     int64_t idx = 0;
-    const uint64_t calls = ka->late.calls;
     if (mine) {
-        if (!uniforms) u = rng_uniform(ka->late.seed, calls, (uint64_t)tid);
+        if (!uniforms) u = rng_uniform(seed, calls, (uint64_t)tid);
         idx = wg_descend(top_s, top_levels, sum, depth, capacity, batch, u, leaf_node, s_step.leaf_value, picked, s_slot);
     }
     // the pushed row: the wave before the last requests its granules now and stores them at the end
@@ -3091,8 +3109,6 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
         }
     }
     // the weights' common denominator (pmin / total * size)^-beta: by the last wave, unless it holds strata itself
-    const int64_t size = ka->late.size;
-    const float beta = ka->late.beta;
     const bool spare_wave = batch <= kStepThreads - 64;
     if (spare_wave && walker) {
         const float max_w = powf_det(top_m[1] / total * (float)size, -beta);
@@ -3127,8 +3143,8 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     }
     if (w0 < work) first_granule.store(dst0, vl0);
     if (mine) {
-        ka->late.out_idx[tid] = idx;
-        ka->late.out_w[tid] = weight;
+        ((__attribute__((address_space(1))) int64_t*)out_idx)[tid] = idx;
+        ((__attribute__((address_space(1))) float*)out_w)[tid] = weight;
         if (!(total > 0.0f) || total > 3.0e38f) atomicOr(err, MRB_DERR_TOTAL);
         if (idx >= size) atomicOr(err, MRB_DERR_UNFILLED);
     }
