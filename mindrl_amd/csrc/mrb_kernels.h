@@ -1130,10 +1130,31 @@ __device__ __forceinline__ uint32_t descend_group(const float* __restrict__ sum,
         node = (node << 3) + walk8(lo, hi, mass, picked);
     } else if (g == 2) {
         const float4 v = *reinterpret_cast<const float4*>(sum + ((uint64_t)node << 2));
-        node = (node << 2) + walk4(v, mass, picked);
+        const float left = v.x + v.y;
+        uint32_t p = 0;
+        if (!(mass <= left)) {
+            mass -= left;
+            p = 2;
+        }
+        const float n0 = p ? v.z : v.x, n1 = p ? v.w : v.y;
+        if (!(mass <= n0)) {
+            mass -= n0;
+            p += 1;
+            picked = n1;
+        } else {
+            picked = n0;
+        }
+        node = (node << 2) + p;
     } else {
         const float2 pair = *reinterpret_cast<const float2*>(sum + 2 * (uint64_t)node);
-        node = 2 * node + walk2(pair, mass, picked);
+        if (mass <= pair.x) {
+            node = 2 * node;
+            picked = pair.x;
+        } else {
+            mass -= pair.x;
+            node = 2 * node + 1;
+            picked = pair.y;
+        }
     }
     return node;
 }
