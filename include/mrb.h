@@ -221,10 +221,12 @@ int mrb_per_update_push(int64_t h, const int64_t *indices, const float *prioriti
  * issues the three in this order from one iteration to the next (mindspore_rl/algorithm/dqn/dqn_trainer.py:76-87).
  * Same results, bit for bit, as the calls one after the other (the sample sees the update and the pushed row). No
  * counterpart among the reference's primitives: on a small buffer each of the three is a launch of a few
- * microseconds, and here they are ONE launch of one workgroup when the update has at most 384 entries, the tree at
- * most 14 levels (capacity up to 16,384), one row is pushed, the batch has at most 512 rows of together at most
- * 32,768 copy granules, and the buffer's counters are on the host; any other call runs as mrb_per_update_push and
- * mrb_per_sample would. Arguments that either of them refuses are refused before anything is changed. */
+ * microseconds, and here they are ONE launch of one workgroup when the update has at most 384 entries, the tree 2
+ * to 14 levels (capacity 3 to 16,384), one row of at most 128 copy granules (2 KB in 16-byte fields) is pushed,
+ * the batch has at most 512 rows of together at most 32,768 copy granules, and the buffer's counters are on the
+ * host; any other call runs as mrb_per_update_push and mrb_per_sample would. Arguments that either of them refuses
+ * are refused before anything is changed. out_indices may be the array `indices` points to (a loop that updates the
+ * rows it sampled the step before): the update has read its entries when the sample writes. */
 int mrb_per_update_push_sample(int64_t h, const int64_t *indices, const float *priorities, int64_t n,
                                const void *const *src_fields, int64_t nrows, const float *opt_push_priorities,
                                int64_t batch, float beta, const float *uniforms, int64_t *out_indices,

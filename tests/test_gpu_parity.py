@@ -1796,10 +1796,14 @@ def test_update_push_sample_equals_the_three_calls(mrb, orc, cap, batch, gen):
         if step == 10:
             ipr = np.full(nrows, 1e12, np.float32)  # the pushed row outweighs all the others together
         u = None if gen else rng.random(batch).astype(np.float32)
+        out = None
+        if k == batch:  # the sampled indices go where the update's indices come from (a loop's own buffer)
+            out = (torch.from_numpy(idx).cuda(), torch.empty(batch, dtype=torch.float32, device="cuda"),
+                   g._layout.empty(batch, g._dev))
         got = g.update_priorities_insert_and_sample(
-            torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda(), *to_dev(rows), beta=0.4 + 0.05 * step,
+            out[0] if out else torch.from_numpy(idx).cuda(), torch.from_numpy(pr).cuda(), *to_dev(rows), beta=0.4 + 0.05 * step,
             insert_priorities=None if ipr is None else torch.from_numpy(ipr).cuda(),
-            uniforms=None if gen else torch.from_numpy(u).cuda())
+            uniforms=None if gen else torch.from_numpy(u).cuda(), out=out)
         ok = (idx >= 0) & (idx < cap) & np.isfinite(pr) & (pr >= 0)  # the device skips and flags the others
         c.update(idx[ok], pr[ok])
         pushed_at = c.head

@@ -116,6 +116,16 @@ def test_kernels_use_no_scratch_memory(tmp_path):
                 assert 512 * 8 + 2 * 648 <= lds - base <= 512 * 8 + 2 * 648 + 128, (name, lds)
             else:
                 assert lds == base + (8 if "pushILb1E" in name else 0), (name, lds)
+    # The whole-step kernel reads the kernel-argument segment with vector loads only (a scalar read in flight would
+    # hold up its barriers' waits for LDS): past the loads that stand in for the preloaded arguments on firmware
+    # without preloading - they end with a branch to the kernel proper - its code holds no scalar load.
+    step = re.search(r"^(_ZN3mrb21k_tree_wg_push_sample\w+):[^\n]*\n(.*?)^\.Lfunc_end", text, re.S | re.M)
+    assert step, "k_tree_wg_push_sample not found in the assembly"
+    code = [l.strip() for l in step.group(2).splitlines() if l.startswith("\t") and not l.strip().startswith((".", ";"))]
+    first_branch = next(i for i, l in enumerate(code) if l.startswith("s_branch"))
+    assert first_branch < 8 and all(l.startswith(("s_load", "s_waitcnt")) for l in code[:first_branch]), code[:8]
+    late = [l for l in code[first_branch:] if l.startswith(("s_load", "s_buffer_load"))]
+    assert not late, late[:4]
 
 
 def test_only_the_documented_entry_points_wait_or_allocate():
