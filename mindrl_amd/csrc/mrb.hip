@@ -730,7 +730,8 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
     // On these trees it also beats the one-wave kernel below for 64 entries or fewer: 5.45 against 5.87 us at 64.)
     if (!sparse && b->fused && n <= kWgBestEntries && b->depth >= 2 && b->depth <= kWgMaxDepth) {
         const uint32_t threads = n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
-        hipLaunchKernelGGL(k_tree_wg, dim3(1), dim3(threads), 0, s, a);
+        hipLaunchKernelGGL(k_tree_wg, dim3(1), dim3(threads), 0, s, a.indices, a.priorities, a.sum, a.mn, a.maxp, (int)a.n,
+                           a.depth, (int)a.capacity, a.alpha, a);
         LAUNCH_CHECK("k_tree_wg");
         return MRB_OK;
     }
@@ -1340,7 +1341,8 @@ int mrb_per_update_push(int64_t h, const int64_t* indices, const float* prioriti
                 const uint32_t threads = n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
                 a.readers = 1 + put.blocks * (threads / 64);
                 hipLaunchKernelGGL(b->device_counters ? k_tree_wg_push<true> : k_tree_wg_push<false>, dim3(1 + put.blocks),
-                                   dim3(threads), 0, s, a, slot, opt_push_priorities, put);
+                                   dim3(threads), 0, s, a.indices, a.priorities, a.sum, a.mn, a.maxp, (int)a.n, a.depth,
+                                   (int)a.capacity, a.alpha, a, slot, opt_push_priorities, put);
                 LAUNCH_CHECK("k_tree_wg_push");
             } else {
                 a.readers = 1 + put.blocks * (kWG / 64);

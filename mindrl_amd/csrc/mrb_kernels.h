@@ -2729,7 +2729,37 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
     if (!kStep) top_write_back(a, top_s, top_m, nthreads);
 }
 
-__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
+// What the one-workgroup update needs first, as plain leading kernel parameters: those are preloaded into scalar
+// registers, so the entries are requested when a wave starts, not a trip to the kernel-argument segment later
+// (of three dependent trips - arguments, entries, the nodes beside the entries' leaves - the first goes away).
+struct WgLead {
+    const int64_t* indices;
+    const float* priorities;
+    float *sum, *mn, *maxp;
+    int n, depth, capacity;
+    float alpha;
+};
+#define MRB_WG_LEAD_PARAMS                                                                                      \
+    const int64_t *__restrict__ lead_indices, const float *__restrict__ lead_priorities, float *lead_sum, float *lead_mn, \
+        float *lead_maxp, int lead_n, int lead_depth, int lead_capacity, float lead_alpha
+__device__ __forceinline__ UpdateArgs with_lead(const UpdateArgs& from, const WgLead& lead) {
+    UpdateArgs a = from;
+    a.indices = lead.indices;
+    a.priorities = lead.priorities;
+    a.sum = lead.sum;
+    a.mn = lead.mn;
+    a.maxp = lead.maxp;
+    a.n = lead.n;
+    a.depth = lead.depth;
+    a.leaves = (int64_t)1 << lead.depth;
+    a.capacity = lead.capacity;
+    a.alpha = lead.alpha;
+    return a;
+}
+#define MRB_WG_LEAD WgLead{lead_indices, lead_priorities, lead_sum, lead_mn, lead_maxp, lead_n, lead_depth, lead_capacity, lead_alpha}
+
+__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(MRB_WG_LEAD_PARAMS, UpdateArgs a_in) {
+    const UpdateArgs a = with_lead(a_in, MRB_WG_LEAD);
     CounterTicket none{};
     float *top_s, *top_m;
     tree_wg_body<false>(a, none, top_s, top_m);
@@ -2747,12 +2777,14 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg(UpdateArgs a) {
 // kDev: the buffer's counters live on the device and this launch moves them on (see Counters); the other
 // instantiation carries none of that.
 template <bool kDev>
-__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(UpdateArgs a, int64_t slot, const float* priority, PutArgs put) {
+__global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(MRB_WG_LEAD_PARAMS, UpdateArgs a_in, int64_t slot,
+                                                                const float* priority, PutArgs put) {
     if (__builtin_expect(blockIdx.x >= 1, 0)) {  // (the tree workgroup's code comes first: it is the one the call waits for)
-        if (kDev) push_rider(put, blockIdx.x - 1, a.err, a.advance, a.capacity, a.readers);
+        if (kDev) push_rider(put, blockIdx.x - 1, a_in.err, a_in.advance, a_in.capacity, a_in.readers);
         else rows_put_part(put, blockIdx.x - 1, put.blocks);
         rider_ends();
     }
+    const UpdateArgs a = with_lead(a_in, MRB_WG_LEAD);
     // The device's counters are the last wave's business: it requests them among the update's first requests, hands
     // the position to the walking wave through LDS and moves the counters on while that wave walks.
     __shared__ int64_t s_position;
