@@ -1827,6 +1827,77 @@ def test_update_push_sample_equals_the_three_calls(mrb, orc, cap, batch, gen):
     g.destroy()
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_whole_step_calls_in_bursts_without_a_wait(mrb, orc, seed):
+    """Seeded random configurations of mrb_per_update_push_sample - capacities 3 to 40,000, batches 1 to 600, rows of
+    7 bytes to over 2 KB, one array per field and packed - called in bursts of up to 24 calls with no wait in between,
+    in half of the bursts every call updating the rows the call before sampled (its indices read from that call's
+    output on the device). Every call's sample, then trees, size, head and running max, against the oracle."""
+    rng = np.random.default_rng(7000 + seed)
+    layouts = [([(3,), (1,)], [np.float32, np.int32]), ([(300,), (1,), (3,)], [np.float32, np.int32, np.uint8]),
+               ([(4,), (1,), (1,), (4,), (1,)], [np.float32, np.int32, np.float32, np.float32, np.bool_]),
+               ([(512,), (1,)], [np.float32, np.int32]), ([(520,), (5,)], [np.float32, np.uint8]), ([(7,)], [np.uint8])]
+    cap = int(rng.choice([3, 4, 5, 64, 200, 257, 1000, 2048, 2049, 4096, 5000, 9000, 10000, 16384, 16385, 40000]))
+    shapes, dtypes = layouts[rng.integers(0, len(layouts))]
+    alpha = float(rng.choice([0.0, 0.4, 0.6, 1.0]))
+    batch = int(rng.choice([1, 2, 8, 33, 64, 64, 200, 384, 448, 449, 512, 600]))
+    g = mrb.PER(alpha, cap, batch, shapes, torch_types(dtypes), seed0=seed + 1, packed_rows=bool(rng.integers(0, 3) == 0))
+    c = orc.OraclePER(alpha, cap, shapes, dtypes, seed=seed + 1)
+    gen = bool(rng.integers(0, 3) == 0)
+    fill = int(rng.choice([cap, cap, max(1, cap // 2), max(1, cap - 5)]))
+    rows = random_rows(rng, fill, shapes, dtypes)
+    pr = (rng.pareto(1.5, fill) + 1e-6).astype(np.float32)
+    g.insert(*to_dev(rows), priorities=torch.from_numpy(pr).cuda()), c.push(rows, fill, pr)
+    for burst in range(3):
+        nb = int(rng.integers(1, 25))
+        follow = bool(rng.integers(0, 2))
+        first = rng.integers(0, min(cap, c.size), batch)
+        steps = []
+        for k in range(nb):
+            n = batch if follow else int(rng.choice([1, 7, 64, int(rng.integers(1, 385)), 384, 385]))
+            ent = rng.integers(0, min(cap, c.size), n)
+            if n > 4 and rng.integers(0, 3) == 0:
+                ent[: n // 3] = ent[0]
+            if n > 2 and rng.integers(0, 3) == 0:
+                ent[-1] = (c.head + k) % cap  # the slot this call's push overwrites
+            p = (rng.pareto(1.5, n) + 1e-6).astype(np.float32)
+            if n > 8 and rng.integers(0, 6) == 0:
+                p[3] = -1.0
+            m = 1 if rng.integers(0, 8) else int(rng.integers(2, 5))
+            kind = rng.integers(0, 4)
+            ipr = (rng.pareto(1.5, m) + 1e-6).astype(np.float32) if kind == 0 else np.full(m, 1e9, np.float32) if kind == 1 else None
+            steps.append(dict(ent=ent, p=p, row=random_rows(rng, m, shapes, dtypes), m=m, ipr=ipr,
+                              u=None if gen else rng.random(batch).astype(np.float32), beta=float(rng.uniform(0, 1))))
+        dev_in = [dict(ent=torch.from_numpy(s["ent"]).cuda(), p=torch.from_numpy(s["p"]).cuda(), row=to_dev(s["row"]),
+                       ipr=None if s["ipr"] is None else torch.from_numpy(s["ipr"]).cuda(),
+                       u=None if s["u"] is None else torch.from_numpy(s["u"]).cuda()) for s in steps]
+        outs = [(torch.empty(batch, dtype=torch.int64, device="cuda"), torch.empty(batch, dtype=torch.float32, device="cuda"),
+                 g._layout.empty(batch, g._dev)) for _ in range(nb)]
+        torch.cuda.synchronize()
+        prev = torch.from_numpy(first).cuda()
+        for k in range(nb):
+            d = dev_in[k]
+            g.update_priorities_insert_and_sample(prev if follow else d["ent"], d["p"], *d["row"], beta=steps[k]["beta"],
+                                                  insert_priorities=d["ipr"], uniforms=d["u"], out=outs[k])
+            prev = outs[k][0]
+        torch.cuda.synchronize()
+        cprev = first
+        for k, s in enumerate(steps):
+            ent = cprev if follow else s["ent"]
+            ok = (ent >= 0) & (ent < cap) & np.isfinite(s["p"]) & (s["p"] >= 0)
+            c.update(ent[ok], s["p"][ok])
+            c.push(s["row"], s["m"], s["ipr"])
+            want = c.sample(batch, s["beta"], s["u"])
+            what = "seed %d burst %d call %d of %d (follow %d, %d entries, %d rows)" % (seed, burst, k, nb, follow, len(ent), s["m"])
+            assert_sample_equal((outs[k][0], outs[k][1]) + tuple(outs[k][2]), want, what)
+            cprev = want[0]
+        assert_tree_equal(g, c, "seed %d burst %d" % (seed, burst))
+        assert g.size() == c.size and g._state()[1] == c.head
+        assert np.float32(g.max_priority) == np.float32(c.max_priority)
+    mrb.lib.lib().mrb_per_check(g._h, C.byref(C.c_uint32(0)), None)  # (flags of the invalid entries: not this test's subject)
+    g.destroy()
+
+
 @pytest.mark.parametrize("cap,npush,batch", [(3000, 1, 48), (10_000, 1, 64), (70_000, 1, 48), (70_000, 3, 300), (1_000_000, 4, 512),
                                              (3_000_000, 1, 40), (3_000_000, 2, 100)])
 def test_hip_graph_replays_sample_then_update_push_with_device_counters(mrb, orc, cap, npush, batch):
