@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Replay-buffer hot-path benchmark on one MI355X.
 
-A step is one pass of the hot path over one batch. The default workload is BASELINE config 3:
+A step is one pass of the hot path over one batch. The default workload is the benchmark's config 3:
 PriorityReplayBuffer.sample (stratified sum-tree descent + importance weights + row gather) on the
 Atari-shaped buffer of capacity 1,000,000 (28,241 stored bytes per row, batch 512), one C-ABI call
 per step on one stream, every call ordered after the one before it. Inputs are synthetic and resident
