@@ -142,7 +142,7 @@ def test_uniform_loop_recorded_into_a_hip_graph_with_device_counters(mrb, orc, l
 
 
 def test_config2_sac_shape_full_size(mrb, orc):
-    """BASELINE config 2 at its real size: capacity 1,000,000, rows f32[17] + f32[6] + f32[1] + f32[17] + bool
+    """The benchmark's config 2 at its real size: capacity 1,000,000, rows f32[17] + f32[6] + f32[1] + f32[17] + bool
     (165 B, mindspore_rl/algorithm/sac/config.py:95-100), filled by 1000 appends of 1000 rows
     (mindspore_rl/core/uniform_replay_buffer.py:101-115), then batches of 256 gathered at seeded host-drawn
     indices integers(0, count) (uniform_replay_buffer.py:130-139). Storage, count / head and every gathered
