@@ -625,7 +625,8 @@ int tree_rebuild(Per& b, UpdateArgs a, hipStream_t s, const PutArgs* ride = null
         }
         const PutArgs& put = (r == 0 && ride) ? *ride : none;
         if (r == 0 && a.inline_election) tiles = (a.n > kPairedAbove ? 2u : 1u) * (uint32_t)a.n;  // one or two waves per entry (see k_tree_update)
-        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4 + put.blocks), dim3(kWG), 0, s, a, r, tile_base, put);
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4 + put.blocks), dim3(kWG), 0, s, a.indices, a.priorities, a.sum, a.mn,
+                           a.n, a.capacity, r | a.lo[r] << 8 | a.g[r] << 16, a.alpha, a, tile_base, put);
         LAUNCH_CHECK("k_tree_update");
     }
     PutArgs put = (a.nrounds == 0 && ride) ? *ride : none;
@@ -755,7 +756,8 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
     const PutArgs none{};
     for (int r = 0; r < b->s_rounds; ++r) {
         const uint32_t tiles = (1u << b->s_lo[r]) / kBlockNodes;
-        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a, r, 0u, none);
+        hipLaunchKernelGGL(k_tree_update, dim3((tiles + 3) / 4), dim3(kWG), 0, s, a.indices, a.priorities, a.sum, a.mn, a.n,
+                           a.capacity, r | a.lo[r] << 8 | a.g[r] << 16, a.alpha, a, 0u, none);
         LAUNCH_CHECK("k_tree_update");
     }
     hipLaunchKernelGGL(k_tree_top, dim3(1), dim3(kTopWG), 0, s, a, none);
@@ -1205,7 +1207,9 @@ static int per_push(Per* b, const void* const* src_fields, int64_t nrows, const 
     if (lead) {
         // the update's leaf round (a wave or two per entry), with this push's row copy as further workgroups
         const uint32_t waves = (lead->a.n > kPairedAbove ? 2u : 1u) * (uint32_t)lead->a.n;
-        hipLaunchKernelGGL(k_tree_update, dim3((waves + 3) / 4 + put.blocks), dim3(kWG), 0, s, lead->a, 0, 0u, put);
+        const UpdateArgs& la = lead->a;
+        hipLaunchKernelGGL(k_tree_update, dim3((waves + 3) / 4 + put.blocks), dim3(kWG), 0, s, la.indices, la.priorities, la.sum,
+                           la.mn, la.n, la.capacity, 0 | la.lo[0] << 8 | la.g[0] << 16, la.alpha, la, 0u, put);
         LAUNCH_CHECK("k_tree_update");
         put.blocks = 0;
     }

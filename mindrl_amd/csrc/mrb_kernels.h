@@ -1969,15 +1969,30 @@ __device__ __forceinline__ void top_rebuild(const UpdateArgs& a, int top, unsign
 // launch (the copy and the tree work touch different memory): workgroups past the tiles do it.
 // `tile_base`: the launch covers tiles tile_base, tile_base + 1, ... only (a push knows which leaf
 // tiles its slot range meets).
-__global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, uint32_t tile_base, PutArgs put) {
+// The leading plain parameters repeat members of `a_in` (plan: round | lo[round] << 8 | g[round] << 16): they are
+// preloaded into scalar registers, so an entry-driven round requests its entries when a wave starts and the tiles
+// when the entries have arrived, not a trip to the kernel-argument segment later.
+__global__ __launch_bounds__(kWG) void k_tree_update(const int64_t* __restrict__ lead_indices,
+                                                     const float* __restrict__ lead_priorities, float* lead_sum, float* lead_mn,
+                                                     int64_t lead_n, int64_t lead_capacity, int plan, float lead_alpha,
+                                                     UpdateArgs a_in, uint32_t tile_base, PutArgs put) {
     __shared__ unsigned long long s_win[kWG / 64][kBlockNodes];
     const uint32_t tile_blocks = gridDim.x - put.blocks;
     if (blockIdx.x >= tile_blocks) {
         rows_put_part(put, blockIdx.x - tile_blocks, put.blocks);
         rider_ends();
     }
+    UpdateArgs a = a_in;
+    a.indices = lead_indices;
+    a.priorities = lead_priorities;
+    a.sum = lead_sum;
+    a.mn = lead_mn;
+    a.n = lead_n;
+    a.capacity = lead_capacity;
+    a.alpha = lead_alpha;
+    const int round = plan & 255;
     const uint32_t lane = threadIdx.x & 63;
-    const int lo = a.lo[round], g = a.g[round];
+    const int lo = (plan >> 8) & 255, g = (plan >> 16) & 255;
     uint32_t tile = tile_base + blockIdx.x * (kWG / 64) + (threadIdx.x >> 6);
     const uint32_t ntiles = (1u << lo) / kBlockNodes;
     const bool last_round = round + 1 == a.nrounds;
@@ -1987,8 +2002,8 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
         // falls into, with every entry of the call that falls into it; entries sharing a tile make
         // their waves write the same values to the same nodes. (4096 tiles scanned for 512 entries
         // cost three times as much as the rebuild itself.)
-        uint32_t* const dirty_next = last_round ? nullptr : a.dirty[round + 1];
-        const int g_next = last_round ? 0 : a.g[round + 1];
+        uint32_t* const dirty_next = last_round ? nullptr : a_in.dirty[round + 1];
+        const int g_next = last_round ? 0 : a_in.g[round + 1];
         if (a.n > kPairedAbove) {
             // two waves per entry (see entry_pair; the launch brings a workgroup per two entries)
             const uint32_t pair = threadIdx.x >> 7, role = (threadIdx.x >> 6) & 1u;
@@ -2009,8 +2024,8 @@ __global__ __launch_bounds__(kWG) void k_tree_update(UpdateArgs a, int round, ui
         tile = ((uint32_t)(ring_position(counters_behind(a.err), a.capacity) / kBlockNodes) + unit) % ring_tiles;
     }
     if (tile >= ntiles) return;
-    tile_round(a, lo, g, tile, true, (elect || (round == 0 && !a.indices)) ? nullptr : a.dirty[round],
-               last_round ? nullptr : a.dirty[round + 1], last_round ? 0 : a.g[round + 1], lane,
+    tile_round(a, lo, g, tile, true, (elect || (round == 0 && !a.indices)) ? nullptr : a_in.dirty[round],
+               last_round ? nullptr : a_in.dirty[round + 1], last_round ? 0 : a_in.g[round + 1], lane,
                s_win[threadIdx.x >> 6]);
 }
 
