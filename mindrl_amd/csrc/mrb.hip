@@ -226,6 +226,12 @@ uint32_t pack_groups(int depth) {
     for (int i = 0; i < count; ++i) packed |= (uint32_t)(depth / count + (i < depth % count ? 1 : 0)) << (4 + 5 * i);
     return packed;
 }
+// The same with what else the sample kernels' `groups` word carries: bit 19 tells that the generator's call counter
+// is on the device (the walk then reads it there; the flag is among the preloaded arguments, the counter's address
+// is not), bits 20-31 the number of batches in the launch minus one.
+uint32_t groups_word(const SampleArgs& a, int64_t nbatch) {
+    return pack_groups(a.depth) | ((uint32_t)(nbatch - 1) << 20) | ((!a.uniforms && a.size < 0) ? 1u << 19 : 0u);
+}
 
 // Threads of a wide-row workgroup: the walker wave, the copy waves and, where rows have narrow fields, their wave.
 inline uint32_t wide_threads(const WidePlan& plan) { return plan.narrow_items ? (uint32_t)kWideWG : (uint32_t)kWideWG - 64u; }
@@ -234,8 +240,7 @@ template <int kInF, bool kTen, bool kOneWide>
 void launch_sample_wide(dim3 grid, const SampleArgs& a, const WidePlan& plan, hipStream_t s) {
     const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
     hipLaunchKernelGGL((k_per_sample_wide<kInF, kTen, kOneWide>), grid, dim3(wide_threads(plan)), 0, s, a.sum, a.uniforms, a.depth,
-                       pack_groups(a.depth) | ((plan.nbatch - 1) << 20), (int)a.batch, (uint32_t)a.capacity, a.seed,
-                       a.calls, tail, plan);
+                       groups_word(a, plan.nbatch), (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, tail, plan);
 }
 
 template <int kInF>
@@ -259,7 +264,7 @@ template <int kInF, bool kTen, bool kOneWide>
 void launch_sample_next(dim3 grid, const SampleArgs& a, const WidePlan& plan, const NextPlan& nx, hipStream_t s) {
     const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
     hipLaunchKernelGGL((k_per_sample_next<kInF, kTen, kOneWide>), grid, dim3(wide_threads(plan)), 0, s, a.sum, a.uniforms, a.depth,
-                       pack_groups(a.depth), (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, tail, plan, nx);
+                       groups_word(a, 1), (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, tail, plan, nx);
 }
 
 template <int kInF>
@@ -313,7 +318,7 @@ int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, int64_
         plan.narrow_items <= 256u && (nrows >= kRowWaveMinRows || r.row_wave == 1)) {
         const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
         const uint32_t blocks = (uint32_t)((nrows + kRowWaveWG / 64 - 1) / (kRowWaveWG / 64));
-        const uint32_t packed = pack_groups(a.depth) | ((plan.nbatch - 1) << 20);
+        const uint32_t packed = groups_word(a, plan.nbatch);
         if (a.depth > 0 && a.depth % kGroupMaxLevels == 0)
             hipLaunchKernelGGL((k_per_sample_rows<true>), dim3(blocks), dim3(kRowWaveWG), 0, s, a.sum, a.uniforms, a.depth, packed,
                                (int)a.batch, (uint32_t)a.capacity, a.seed, a.calls, nrows, tail, plan);
@@ -326,7 +331,7 @@ int sample_wide(const RowStore& r, const SampleArgs& a, const IoTable& t, int64_
     // Fewer rows of that size: the workgroup kernel with two copy waves instead of four (k_per_sample_light).
     if (r.row_split == 0 && plan.split == 1 && plan.wide_items <= 2u * 64u * kLightCopyWaves && a.depth != 22) {
         const SampleTail tail{a.mn, a.out_idx, a.out_w, a.err, a.size, a.beta};
-        const uint32_t packed = pack_groups(a.depth) | ((plan.nbatch - 1) << 20);
+        const uint32_t packed = groups_word(a, plan.nbatch);
         const dim3 threads(plan.narrow_items ? (uint32_t)kLightWG : (uint32_t)kLightWG - 64u);
         const bool ten = a.depth > 0 && a.depth % kGroupMaxLevels == 0, one = plan.nwide == 1;
 #define MRB_LAUNCH_LIGHT(T, O)                                                                                         \

@@ -783,9 +783,14 @@ __device__ __forceinline__ void sample_wide_body(const float* __restrict__ sum, 
             int g = kTen ? kGroupMaxLevels : (int)(packed & 31u);
             f32x4 r0, r1, r2, r3;
             group_request(sum, 1u, g, lane, r0, r1, r2, r3);
-            total = sum[1];
-            const float u_given = *(uniforms ? uniforms + k : sum + 1);
-            const uint64_t calls_now = generator_calls(uniforms, calls, tail.size, tail.err);
+            // (vector loads, through an offset the compiler cannot see through: as scalar loads they would be waited
+            // for together with the reads of the kernel-argument segment that the other waves' code begins with)
+            uint32_t opaque_zero = 0;
+            asm volatile("" : "+v"(opaque_zero));
+            total = sum[1 + opaque_zero];
+            const float u_given = (uniforms ? uniforms + k : sum + 1)[opaque_zero];
+            uint64_t calls_now = calls;
+            if (!uniforms && (groups & (1u << 19))) calls_now += (uint64_t)counters_behind(tail.err)[kCntCalls];
             __builtin_amdgcn_sched_barrier(0);
             const float u = uniforms ? u_given : rng_uniform(seed, calls_now + nth, (uint64_t)stratum);
             mass = (u + (float)stratum) * (total / (float)batch);  // each operation rounded once
