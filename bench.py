@@ -365,6 +365,12 @@ class PerRun:
             self._lib.check(rc)
 
     def loop(self, i, sp=None, fused=False):
+        if fused == "one call":  # the whole step as one library call (mrb_per_update_push_sample)
+            a = self._step_args[i]
+            rc = self._step_fn(*(a[:-1] + (sp or self.sp,)))
+            if rc:
+                self._lib.check(rc)
+            return
         self.sample(i, sp)
         if fused:
             rc = self.L.mrb_per_update_push(self.h, self.idx.data_ptr(), self.upr[i % 64].data_ptr(), self.upd, self.sptr,
@@ -582,7 +588,8 @@ def per_extras(a, torch, r, algo_bytes):
     if r.upd <= 1024:  # device-resident counters take updates of at most 1024 entries
         r.buf.set_option("device_counters", 1)
         n_l = min(K, 50)
-        for key, fused in (("loop_graph_replay_steps_per_s", False), ("loop_update_push_graph_replay_steps_per_s", True)):
+        for key, fused in (("loop_graph_replay_steps_per_s", False), ("loop_update_push_graph_replay_steps_per_s", True),
+                           ("loop_one_call_graph_replay_steps_per_s", "one call")):
             lgraph = torch.cuda.CUDAGraph()
             lside = torch.cuda.Stream()
             with torch.cuda.stream(lside):

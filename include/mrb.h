@@ -223,8 +223,10 @@ int mrb_per_update_push(int64_t h, const int64_t *indices, const float *prioriti
  * counterpart among the reference's primitives: on a small buffer each of the three is a launch of a few
  * microseconds, and here they are ONE launch of one workgroup when the update has at most 384 entries, the tree 2
  * to 14 levels (capacity 3 to 16,384), one row of at most 128 copy granules (2 KB in 16-byte fields) is pushed,
- * the batch has at most 512 rows of together at most 32,768 copy granules, and the buffer's counters are on the
- * host; any other call runs as mrb_per_update_push and mrb_per_sample would. Arguments that either of them refuses
+ * the batch has at most 512 rows of together at most 32,768 copy granules (with the option device_counters the
+ * kernel takes the ring position, the row count and the generator's call counter from the device and moves them on
+ * itself: a loop of such calls can be recorded into a HIP graph); any other call runs as mrb_per_update_push and
+ * mrb_per_sample would. Arguments that either of them refuses
  * are refused before anything is changed. out_indices may be the array `indices` points to (a loop that updates the
  * rows it sampled the step before): the update has read its entries when the sample writes. */
 int mrb_per_update_push_sample(int64_t h, const int64_t *indices, const float *priorities, int64_t n,

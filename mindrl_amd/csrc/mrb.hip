@@ -491,7 +491,6 @@ struct Per {
         if (sum) (void)hipFree(sum);
         if (mn) (void)hipFree(mn);
         if (stamp) (void)hipFree(stamp);
-        if (maxp) (void)hipFree(maxp);
         if (powered) (void)hipFree(powered);
         for (auto* d : retired) (void)hipFree(d);
         for (auto* d : s_dirty)
@@ -1131,10 +1130,13 @@ int mrb_per_create(int64_t capacity, float alpha, int nfields, const int64_t* fi
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->sum), nodes * sizeof(float)));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->mn), nodes * sizeof(float)));
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->stamp), (size_t)b->leaves * sizeof(unsigned long long)));
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->maxp), 16));
-    // one allocation: the error word (16 bytes), then the device copy of the counters (kernels find them there)
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), 16 + kCntWords * sizeof(int64_t)));
+    // one allocation: the error word (16 bytes), the device copy of the counters (kernels find them behind the error
+    // word), and kMaxpBehindErr bytes in the running max (16 bytes; a kernel that is given its address finds the
+    // counters in front of it: counters_before)
+    static_assert(16 + kCntWords * sizeof(int64_t) <= kMaxpBehindErr, "the counters end before the running max");
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b->err), kMaxpBehindErr + 16));
     b->counters = reinterpret_cast<int64_t*>(b->err + 4);
+    b->maxp = reinterpret_cast<float*>(reinterpret_cast<char*>(b->err) + kMaxpBehindErr);
     HIP_TRY(hipMemset(b->counters, 0, kCntWords * sizeof(int64_t)));
     // update_priorities scratch, sized once: a call rarely names more entries than there are rows
     b->powered_cap = capacity < 4096 ? 4096 : (capacity > (1ll << 20) ? (1ll << 20) : capacity);
@@ -1487,7 +1489,7 @@ int mrb_per_update_push_sample(int64_t h, const int64_t* indices, const float* p
     const int64_t cap = b->rows.capacity;
     // one launch of one workgroup: the update of at most 384 entries on a tree of at most 14 levels, one row, a batch
     // of at most a thread per stratum, and rows small enough for one workgroup to copy; the counters on the host
-    if (b->fused && !b->device_counters && b->sample_path == 0 && nrows == 1 && n <= kWgBestEntries && b->depth >= 2 &&
+    if (b->fused && b->sample_path == 0 && nrows == 1 && n <= kWgBestEntries && b->depth >= 2 &&
         b->depth <= kWgMaxDepth && batch <= kStepThreads) {
         PutArgs put{};
         const int64_t first = b->pushes % cap;
@@ -1512,8 +1514,12 @@ int mrb_per_update_push_sample(int64_t h, const int64_t* indices, const float* p
             late.beta = beta;
             late.put = put.t;
             late.get = t;
-            hipLaunchKernelGGL(k_tree_wg_push_sample, dim3(1), dim3(kStepThreads), 0, s, indices, priorities, b->sum, b->mn,
-                               a.maxp, (int)(cap << 16 | first), (int)(n << 18 | batch << 8) | b->depth, a.alpha, late);
+            // (with device_counters the kernel takes the slot, the row count and the generator's call counter from the
+            // device and moves them on itself)
+            hipLaunchKernelGGL(b->device_counters ? k_tree_wg_push_sample<true> : k_tree_wg_push_sample<false>, dim3(1),
+                               dim3(kStepThreads), 0, s, indices, priorities, b->sum, b->mn, a.maxp,
+                               (int)(cap << 16 | (b->device_counters ? 0 : first)), (int)(n << 18 | batch << 8) | b->depth, a.alpha,
+                               late);
             LAUNCH_CHECK("k_tree_wg_push_sample");
             b->pushes += 1;
             b->size = late.size;

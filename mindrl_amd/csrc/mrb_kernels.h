@@ -148,6 +148,12 @@ constexpr int kCntPushes = 0, kCntSize = 1, kCntCalls = 2, kCntPos = 4, kCntWord
 __device__ __forceinline__ const int64_t* counters_behind(const uint32_t* err) {
     return reinterpret_cast<const int64_t*>(err + 4);
 }
+// A prioritized buffer's running max lives in the same allocation, kMaxpBehindErr bytes behind the error word: a
+// kernel that has its address among its preloaded arguments finds the counters without reading another argument.
+constexpr int kMaxpBehindErr = 64;
+__device__ __forceinline__ int64_t* counters_before(float* maxp) {
+    return reinterpret_cast<int64_t*>(reinterpret_cast<char*>(maxp) - kMaxpBehindErr + 16);
+}
 __device__ __forceinline__ int64_t ring_position(const int64_t* counters, int64_t capacity) {
     return counters[kCntPos];
 }
@@ -2509,6 +2515,10 @@ struct StepShared {
     float watch_s[4], watch_m[4];
     float leaf_value;  // (the other way: the written leaf's value, for the sample that follows)
     float max_w;       // the weights' common denominator, by a wave that does not sample
+    // counters on the device: what the walking wave found there
+    uint32_t watch_leaf;  // the leaf the caller writes next (else an argument of tree_wg_body)
+    int64_t slot, size_after;
+    uint64_t calls;
 };
 
 __device__ __forceinline__ void top_write_back(const UpdateArgs& a, const float* top_s, const float* top_m, uint32_t nthreads) {
@@ -2526,8 +2536,9 @@ __device__ __forceinline__ void top_write_back(const UpdateArgs& a, const float*
 
 // kStep: the caller goes on with the staged top and writes it back itself (top_write_back); `step` (zeroed by the
 // caller before the workgroup's first barrier) receives what StepShared describes, watch_leaf being the heap
-// number of the leaf the caller writes next.
-template <bool kTake, bool kStep = false>
+// number of the leaf the caller writes next - with kStep == 2 taken from `step` (left there before the first
+// barrier: the caller had to read it from the device).
+template <bool kTake, int kStep = 0>
 __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket& ticket, float*& staged_s, float*& staged_m,
                                              StepShared* step = nullptr, uint32_t watch_leaf = 0) {
     __shared__ __align__(16) float top_s[kWgTopNodes];
@@ -2646,6 +2657,7 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
             const unsigned long long* vt = vals[s % 3];
             const bool two = s > 0 || h_first == 2;
             const int up = s == 0 ? 0 : h_first + 2 * (s - 1);  // levels between v and the leaves
+            if (kStep == 2) watch_leaf = step->watch_leaf;
             if (act) {
                 a.sum[v] = cs;
                 a.mn[v] = cm;
@@ -3039,6 +3051,11 @@ struct GranulePlace {
 // Sixteen 32-bit words are preloaded into scalar registers, two of them the segment's address: the fourteen leading
 // parameters are what the update needs first (the numbers among them packed: slot_capacity = capacity << 16 | slot,
 // sizes = n << 18 | batch << 8 | depth), so that its first requests go out when a wave starts.
+// kDev: the buffer's counters live on the device (see Counters): the walking wave reads the ring position, the row
+// count and the generator's call counter there when the kernel starts (they lie in front of the running max, whose
+// address is preloaded), hands them to the others through LDS and stores them moved on; this one workgroup is the
+// launch's only reader, so nobody has to be waited for. The other instantiation carries none of that.
+template <bool kDev>
 __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int64_t* __restrict__ indices,
                                                                       const float* __restrict__ priorities, float* sum, float* mn,
                                                                       float* maxp, int slot_capacity, int sizes, float alpha,
@@ -3051,9 +3068,19 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     const bool walker = tid >= kStepThreads - 64, putter = !walker && tid >= kStepThreads - 128;
     const int depth = sizes & 255;
     const uint32_t batch = ((uint32_t)sizes >> 8) & 1023u;
-    const int64_t slot = slot_capacity & 0xffff, capacity = (uint32_t)slot_capacity >> 16;
+    int64_t slot = slot_capacity & 0xffff;  // (kDev: known to the walking wave first, to the others after the update)
+    const int64_t capacity = (uint32_t)slot_capacity >> 16;
     const int top_levels = depth < kWgTopLevels ? depth : kWgTopLevels;
-    const uint32_t top_nodes = 2u << top_levels, leaf_node = (1u << depth) + (uint32_t)slot;
+    const uint32_t top_nodes = 2u << top_levels;
+    int64_t c_pushes = 0, c_size = 0, c_calls = 0;
+    if (kDev && walker) {
+        int64_t* const cnt = counters_before(maxp);
+        c_pushes = __hip_atomic_load(cnt + kCntPushes, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        c_size = __hip_atomic_load(cnt + kCntSize, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        c_calls = __hip_atomic_load(cnt + kCntCalls, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        slot = __hip_atomic_load(cnt + kCntPos, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    uint32_t leaf_node = (1u << depth) + (uint32_t)slot;
     UpdateArgs a{};
     a.indices = indices;
     a.priorities = priorities;
@@ -3096,6 +3123,12 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
         if (lane == 0) {
             s_step.qmax = 0u;
             s_step.flags = 0u;
+            if (kDev) {
+                s_step.watch_leaf = leaf_node;
+                s_step.slot = slot;
+                s_step.size_after = c_size + 1 < capacity ? c_size + 1 : capacity;
+                s_step.calls = (uint64_t)c_calls;
+            }
         }
     }
     if (walker || putter) {
@@ -3112,7 +3145,19 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     }
     CounterTicket none{};
     float *top_s, *top_m;
-    tree_wg_body<false, true>(a, none, top_s, top_m, &s_step, leaf_node);  // (ends behind a barrier)
+    tree_wg_body<false, kDev ? 2 : 1>(a, none, top_s, top_m, &s_step, leaf_node);  // (ends behind a barrier)
+    if (kDev) {
+        if (walker) {  // the counters moved on (this launch has no other reader of them)
+            int64_t* const cnt = counters_before(maxp);
+            if (lane == 0) {
+                counters_store_advanced(cnt, c_pushes, c_size, slot, 1, capacity);
+                if (!uniforms) cnt[kCntCalls] = c_calls + 1;
+            }
+        } else {
+            slot = s_step.slot;
+            leaf_node = (1u << depth) + (uint32_t)slot;
+        }
+    }
     if (walker || putter) {
         LdsTable* mine = walker ? &s_get : &s_put;
         if (lane <= MRB_MAX_FIELDS) mine->prefix[lane] = t_prefix;
@@ -3131,9 +3176,10 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     const StepKernargPtr ka = step_kernarg(true);
     uint32_t* const err = vector_read(&ka->late.err, opaque_zero);
     const int put_fields = vector_read(&ka->late.put.nfields, opaque_zero), get_fields = vector_read(&ka->late.get.nfields, opaque_zero);
-    const int64_t size = vector_read(&ka->late.size, opaque_zero);
+    const int64_t size = kDev ? s_step.size_after : vector_read(&ka->late.size, opaque_zero);
     const float beta = vector_read(&ka->late.beta, opaque_zero);
-    const uint64_t seed = vector_read(&ka->late.seed, opaque_zero), calls = vector_read(&ka->late.calls, opaque_zero);
+    const uint64_t seed = vector_read(&ka->late.seed, opaque_zero);
+    const uint64_t calls = kDev ? s_step.calls : vector_read(&ka->late.calls, opaque_zero);
     int64_t* const out_idx = vector_read(&ka->late.out_idx, opaque_zero);
     float* const out_w = vector_read(&ka->late.out_w, opaque_zero);
     // the strata's draws: needed a barrier from here

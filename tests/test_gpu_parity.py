@@ -1827,6 +1827,81 @@ def test_update_push_sample_equals_the_three_calls(mrb, orc, cap, batch, gen):
     g.destroy()
 
 
+@pytest.mark.parametrize("gen", [True, False])
+@pytest.mark.parametrize("cap,batch,steps", [(3000, 48, 3), (10_000, 64, 5), (16_384, 300, 2), (100, 64, 4), (70_000, 64, 2)])
+def test_hip_graph_replays_the_whole_step_with_device_counters(mrb, orc, cap, batch, steps, gen):
+    """`steps` calls of mrb_per_update_push_sample, each updating the rows the call before sampled (in place: one
+    index buffer), recorded ONCE into a HIP graph with device_counters and replayed 8 times: the one-workgroup kernel
+    takes the ring position, the row count and the generator's call counter from the device and moves them on
+    itself; the buffer fills during the replays, then the ring wraps. After every replay the last sample, both trees,
+    size, head and running max equal the oracle's; eager calls in between use the same counters. (Capacity 70,000
+    lies outside the one-launch kernel: the same call as its two-call fallback.)"""
+    rng = np.random.default_rng(cap + batch + gen)
+    shapes, dtypes = [(4,), (1,), (1,), (4,), (1,)], [np.float32, np.int32, np.float32, np.float32, np.bool_]
+    g, c = make_pair(mrb, orc, 0.6, cap, batch, seed=23, shapes=shapes, dtypes=dtypes)
+    fill = cap - 3 * steps - 1  # not full: the row count changes during the replays, then the ring wraps
+    rows = random_rows(rng, fill, shapes, dtypes)
+    pr0 = (rng.pareto(1.5, fill) + 1e-6).astype(np.float32)
+    g.insert(*to_dev(rows), priorities=torch.from_numpy(pr0).cuda()), c.push(rows, fill, pr0)
+    g.set_option("device_counters", 1)
+    new_rows = [[torch.zeros((1,) + tuple(s), dtype=t).cuda() for s, t in zip(shapes, torch_types(dtypes))] for _ in range(steps)]
+    pr_dev = torch.ones((steps, batch), dtype=torch.float32, device="cuda")
+    u_dev = torch.zeros((steps, batch), dtype=torch.float32, device="cuda")
+    out = (torch.empty(batch, dtype=torch.int64, device="cuda"), torch.empty(batch, dtype=torch.float32, device="cuda"),
+           g._layout.empty(batch, g._dev))
+    first = rng.integers(0, fill, batch)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        for k in range(steps):
+            g.update_priorities_insert_and_sample(out[0], pr_dev[k], *new_rows[k], beta=0.5, uniforms=None if gen else u_dev[k], out=out)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    prev = first
+    for rep in range(8):
+        fresh = [random_rows(rng, 1, shapes, dtypes) for _ in range(steps)]
+        pr = (rng.pareto(1.5, (steps, batch)) + 1e-6).astype(np.float32)
+        u = rng.random((steps, batch)).astype(np.float32)
+        for k in range(steps):
+            for dst, src in zip(new_rows[k], fresh[k]):
+                dst.copy_(torch.from_numpy(src))
+        pr_dev.copy_(torch.from_numpy(pr))
+        u_dev.copy_(torch.from_numpy(u))
+        out[0].copy_(torch.from_numpy(prev))
+        graph.replay()
+        torch.cuda.synchronize()
+        for k in range(steps):
+            ok = (prev >= 0) & (prev < cap)
+            c.update(prev[ok], pr[k][ok])
+            c.push(fresh[k], 1)
+            want = c.sample(batch, 0.5, None if gen else u[k])
+            prev = want[0]
+        what = "cap %d replay %d" % (cap, rep)
+        assert_sample_equal((out[0], out[1]) + tuple(out[2]), want, what)
+        assert_tree_equal(g, c, what)
+        assert g.size() == c.size and g._state()[1] == c.head, what
+        assert np.float32(g.max_priority) == np.float32(c.max_priority)
+        if rep % 3 == 1:  # eager calls in between
+            extra = random_rows(rng, 2, shapes, dtypes)
+            g.insert(*to_dev(extra)), c.push(extra, 2)
+            got = g.update_priorities_insert_and_sample(torch.from_numpy(prev).cuda(), torch.from_numpy(pr[0]).cuda(),
+                                                        *to_dev(fresh[0]), beta=0.7)
+            ok = (prev >= 0) & (prev < cap)
+            c.update(prev[ok], pr[0][ok]), c.push(fresh[0], 1)
+            want = c.sample(batch, 0.7)
+            assert_sample_equal(got, want, "eager after replay %d" % rep)
+            prev = want[0]
+    for f, (a, b) in enumerate(zip(g.storage(), [c.field(i) for i in range(len(shapes))])):
+        assert np.array_equal(t2n(a).view(np.uint8), b.view(np.uint8)), f
+    g.set_option("device_counters", 0)
+    assert g.size() == c.size
+    mrb.lib.lib().mrb_per_check(g._h, C.byref(C.c_uint32(0)), None)
+    del graph
+    g.destroy()
+
+
 @pytest.mark.parametrize("seed", range(40))
 def test_whole_step_calls_in_bursts_without_a_wait(mrb, orc, seed):
     """Seeded random configurations of mrb_per_update_push_sample - capacities 3 to 40,000, batches 1 to 600, rows of

@@ -100,7 +100,7 @@ def test_kernels_use_no_scratch_memory(tmp_path):
                          int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", block).group(1)),
                          int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)))
     assert sum("k_per_sample_wide" in k for k in kernels) == 8 and sum("k_rows_gather_wide" in k for k in kernels) == 4
-    assert len(kernels) == 52, sorted(kernels)
+    assert len(kernels) == 53, sorted(kernels)
     for name, (scratch, lds, vgprs) in kernels.items():
         assert scratch == 0, "%s uses %d bytes of scratch per lane" % (name, scratch)
         assert vgprs <= 128, (name, vgprs)
@@ -119,13 +119,14 @@ def test_kernels_use_no_scratch_memory(tmp_path):
     # The whole-step kernel reads the kernel-argument segment with vector loads only (a scalar read in flight would
     # hold up its barriers' waits for LDS): past the loads that stand in for the preloaded arguments on firmware
     # without preloading - they end with a branch to the kernel proper - its code holds no scalar load.
-    step = re.search(r"^(_ZN3mrb21k_tree_wg_push_sample\w+):[^\n]*\n(.*?)^\.Lfunc_end", text, re.S | re.M)
-    assert step, "k_tree_wg_push_sample not found in the assembly"
-    code = [l.strip() for l in step.group(2).splitlines() if l.startswith("\t") and not l.strip().startswith((".", ";"))]
-    first_branch = next(i for i, l in enumerate(code) if l.startswith("s_branch"))
-    assert first_branch < 8 and all(l.startswith(("s_load", "s_waitcnt")) for l in code[:first_branch]), code[:8]
-    late = [l for l in code[first_branch:] if l.startswith(("s_load", "s_buffer_load"))]
-    assert not late, late[:4]
+    steps = re.findall(r"^(_ZN3mrb21k_tree_wg_push_sample\w+):[^\n]*\n(.*?)^\.Lfunc_end", text, re.S | re.M)
+    assert len(steps) == 2, "both instantiations of k_tree_wg_push_sample in the assembly"
+    for name, body in steps:
+        code = [l.strip() for l in body.splitlines() if l.startswith("\t") and not l.strip().startswith((".", ";"))]
+        first_branch = next(i for i, l in enumerate(code) if l.startswith("s_branch"))
+        assert first_branch < 8 and all(l.startswith(("s_load", "s_waitcnt")) for l in code[:first_branch]), (name, code[:8])
+        late = [l for l in code[first_branch:] if l.startswith(("s_load", "s_buffer_load"))]
+        assert not late, (name, late[:4])
 
 
 def test_only_the_documented_entry_points_wait_or_allocate():
