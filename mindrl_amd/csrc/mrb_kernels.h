@@ -2562,6 +2562,17 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
         idx = a.indices[tid];
         p = a.priorities[tid];
     }
+    // A call of so few entries that eight threads can share one takes the levels below the staged top in ONE step
+    // and without hash tables of its own: thread t is lane t & 7 of the cluster of entry t >> 3 and looks after
+    // one leaf of the entry's group (the 2, 4 or 8 leaves under its ancestor at the staged top's lowest level).
+    const bool clustered = H > 0 && (uint64_t)a.n * 8u <= nthreads;  // uniform
+    const uint32_t ce = tid >> 3, cj = tid & 7u;
+    int64_t cidx = -1;
+    float cp = -1.0f;
+    if (clustered && (int64_t)ce < a.n) {
+        cidx = a.indices[ce];
+        cp = a.priorities[ce];
+    }
     // the running max as the kernel finds it, for the test that spares the atomic below (see raise_max; the max only
     // grows, so an older value spares no atomic that matters - and read now it is no round trip behind the power)
     // (a vector load: a scalar one would be waited for by the next barrier's wait for LDS)
@@ -2606,7 +2617,7 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
             pre_s[s][c] = 0.0f;
             pre_m[s][c] = 0.0f;
         }
-        if (s < nh && valid) {
+        if (s < nh && valid && !clustered) {
             const uint32_t v = leaf_node >> (s == 0 ? 0 : h_first + 2 * (s - 1));
             pre_s[s][0] = a.sum[v ^ 1u];
             pre_m[s][0] = a.mn[v ^ 1u];
@@ -2618,6 +2629,14 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
                 pre_m[s][2] = a.mn[c0 | 1u];
             }
         }
+    }
+    // (clustered: memory's value of this lane's leaf of its entry's group, both trees)
+    const bool cvalid = clustered && cidx >= 0 && cidx < a.capacity && valid_priority(cp) && cj < (1u << H);
+    const uint32_t cgroup = (((uint32_t)a.leaves + (uint32_t)(cvalid ? cidx : 0)) >> H) << H;  // the group's first leaf
+    float cl_s = 0.0f, cl_m = 0.0f;
+    if (cvalid) {
+        cl_s = a.sum[cgroup + cj];
+        cl_m = a.mn[cgroup + cj];
     }
     if (kTake && tid >= nthreads - 64) ticket = counters_take(a.err);
     // the election's first step: a slot for the entry's leaf (the attempt is on its way during the power)
@@ -2649,10 +2668,67 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
     bool act = valid && (uint32_t)(vals[0][slot] >> 32) == tid;
     uint32_t v = leaf_node;
     float cs = q, cm = q;
+    if (clustered) {
+        // ---- below the staged top, a cluster per entry: every lane takes this call's value of its leaf where the
+        // call changes it (the election's table holds every such leaf with the elected entry's power), the cluster
+        // rebuilds the group's levels among its lanes and lane 0 goes on with the group's root. Clusters of entries
+        // that share a group - or a leaf - do the same work and store the same bits.
+        if (cvalid) {
+            const uint32_t node = cgroup + cj, h = wg_hash(node);
+            if (wg_resolve<true>(keys[0], vals[0], node, h, keys[0][h], vals[0][h], cl_s, cl_m)) {
+                a.sum[node] = cl_s;
+                a.mn[node] = cl_m;
+            }
+        }
+        // (every lane takes part in the exchanges; lanes without a leaf hold values that go nowhere)
+        const float s1 = cl_s + butterfly_peer<0>(cl_s), m1 = fminf(cl_m, butterfly_peer<0>(cl_m));
+        const float s2 = s1 + butterfly_peer<1>(s1), m2 = fminf(m1, butterfly_peer<1>(m1));
+        const float s3 = s2 + butterfly_peer<2>(s2), m3 = fminf(m2, butterfly_peer<2>(m2));
+        if (cvalid) {
+            if (H >= 2 && (cj & 1u) == 0) {
+                a.sum[(cgroup + cj) >> 1] = s1;
+                a.mn[(cgroup + cj) >> 1] = m1;
+            }
+            if (H == 3 && (cj & 3u) == 0) {
+                a.sum[(cgroup + cj) >> 2] = s2;
+                a.mn[(cgroup + cj) >> 2] = m2;
+            }
+            if (kStep) {
+                if (kStep == 2) watch_leaf = step->watch_leaf;
+                if ((watch_leaf >> H) << H == cgroup) {  // the group of the leaf the caller writes next: what lies beside its path
+                    const uint32_t rel = watch_leaf - cgroup;
+                    if (cj == (rel ^ 1u)) {
+                        step->watch_s[0] = cl_s;
+                        step->watch_m[0] = cl_m;
+                        step->watch_set[0] = 1u;
+                    }
+                    if (H >= 2 && cj == (((rel >> 1) ^ 1u) << 1)) {
+                        step->watch_s[1] = s1;
+                        step->watch_m[1] = m1;
+                        step->watch_set[1] = 1u;
+                    }
+                    if (H == 3 && cj == (((rel >> 2) ^ 1u) << 2)) {
+                        step->watch_s[2] = s2;
+                        step->watch_m[2] = m2;
+                        step->watch_set[2] = 1u;
+                    }
+                }
+            }
+        }
+        // The group's root goes into the staged top, and the ENTRY's thread takes the path from there (the entries'
+        // threads sit in the first wave: the clusters' first lanes are spread over all of them, and a step inside the
+        // top costs every wave that has a path to carry): it picks its node's value up behind the next barrier.
+        if (cvalid && cj == 0) {
+            top_s[cgroup >> H] = H == 3 ? s3 : H == 2 ? s2 : s1;
+            top_m[cgroup >> H] = H == 3 ? m3 : H == 2 ? m2 : m1;
+        }
+        act = valid;  // (also an entry that lost its leaf to a later one: it carries the same values up the same path)
+        v = leaf_node >> H;
+    }
     // ---- below the staged top: the call's nodes in hash tables
 #pragma unroll
     for (int s = 0; s < kWgHashSteps; ++s) {
-        if (s < nh) {  // uniform
+        if (s < nh && !clustered) {  // uniform
             const uint32_t* kt = keys[s % 3];
             const unsigned long long* vt = vals[s % 3];
             const bool two = s > 0 || h_first == 2;
@@ -2723,11 +2799,15 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
 #pragma unroll
     for (int u = 0; u < kWgTopSteps; ++u) {
         if (u < nt) {  // uniform
-            if (act) {
+            if (act && !(clustered && u == 0)) {
                 top_s[v] = cs;
                 top_m[v] = cm;
             }
             lds_barrier();
+            if (clustered && u == 0 && act) {
+                cs = top_s[v];
+                cm = top_m[v];
+            }
             if (act) {
                 const bool two = u > 0 || t_first == 2;
                 const bool right = (v & 1u) != 0;
