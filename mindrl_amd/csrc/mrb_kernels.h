@@ -2533,6 +2533,17 @@ __device__ __forceinline__ void top_write_back(const UpdateArgs& a, const float*
         }
     }
 }
+// The same by `count` threads of the workgroup, this one being number `index` among them.
+__device__ __forceinline__ void top_write_back_by(const UpdateArgs& a, const float* top_s, const float* top_m, uint32_t index,
+                                                  uint32_t count) {
+    const int T = a.depth < kWgTopLevels ? a.depth : kWgTopLevels;
+    const uint32_t top_vec = 1u << (T - 1);
+#pragma unroll 4
+    for (uint32_t i = index; i < top_vec; i += count) {
+        reinterpret_cast<f32x4*>(a.sum)[i] = reinterpret_cast<const f32x4*>(top_s)[i];
+        reinterpret_cast<f32x4*>(a.mn)[i] = reinterpret_cast<const f32x4*>(top_m)[i];
+    }
+}
 
 // kStep: the caller goes on with the staged top and writes it back itself (top_write_back); `step` (zeroed by the
 // caller before the workgroup's first barrier) receives what StepShared describes, watch_leaf being the heap
@@ -3211,16 +3222,17 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
             }
         }
     }
-    if (walker || putter) {
-        const __attribute__((address_space(1))) IoTable* t = walker ? &early->late.get : &early->late.put;
-        if (lane <= MRB_MAX_FIELDS) t_prefix = t->prefix[lane];
-        if (lane < MRB_MAX_FIELDS) {
-            t_store = t->store[lane];
-            t_io = t->io[lane];
-            t_row_bytes = t->row_bytes[lane];
-            t_stride = t->stride[lane];
-            t_units = t->units[lane];
-            t_vec = t->vec_log2[lane];
+    const uint32_t t_lane = lane & 31u;  // (the wave before the last: lanes 0.. the pushed row's table, lanes 32.. the batch's)
+    if (putter) {
+        const __attribute__((address_space(1))) IoTable* t = lane >= 32 ? &early->late.get : &early->late.put;
+        if (t_lane <= MRB_MAX_FIELDS) t_prefix = t->prefix[t_lane];
+        if (t_lane < MRB_MAX_FIELDS) {
+            t_store = t->store[t_lane];
+            t_io = t->io[t_lane];
+            t_row_bytes = t->row_bytes[t_lane];
+            t_stride = t->stride[t_lane];
+            t_units = t->units[t_lane];
+            t_vec = t->vec_log2[t_lane];
         }
     }
     CounterTicket none{};
@@ -3238,34 +3250,22 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
             leaf_node = (1u << depth) + (uint32_t)slot;
         }
     }
-    if (walker || putter) {
-        LdsTable* mine = walker ? &s_get : &s_put;
-        if (lane <= MRB_MAX_FIELDS) mine->prefix[lane] = t_prefix;
-        if (lane < MRB_MAX_FIELDS) {
-            mine->store[lane] = t_store;
-            mine->io[lane] = t_io;
-            mine->row_bytes[lane] = t_row_bytes;
-            mine->stride[lane] = t_stride;
-            mine->units[lane] = t_units;
-            mine->vec_log2[lane] = t_vec;
+    if (putter) {
+        LdsTable* mine = lane >= 32 ? &s_get : &s_put;
+        if (t_lane <= MRB_MAX_FIELDS) mine->prefix[t_lane] = t_prefix;
+        if (t_lane < MRB_MAX_FIELDS) {
+            mine->store[t_lane] = t_store;
+            mine->io[t_lane] = t_io;
+            mine->row_bytes[t_lane] = t_row_bytes;
+            mine->stride[t_lane] = t_stride;
+            mine->units[t_lane] = t_units;
+            mine->vec_log2[t_lane] = t_vec;
         }
     }
-    // (behind the tables, and behind a use of what was requested when the kernel started: a wave's requests come back
-    // in order, and a wait for an old one that the compiler cannot tell from these would wait for these)
-    asm volatile("" ::"v"(sib_s), "v"(sib_m), "v"(old_max), "v"(priority), "v"(err_early), "v"(uniforms));
-    const StepKernargPtr ka = step_kernarg(true);
-    uint32_t* const err = vector_read(&ka->late.err, opaque_zero);
-    const int put_fields = vector_read(&ka->late.put.nfields, opaque_zero), get_fields = vector_read(&ka->late.get.nfields, opaque_zero);
-    const int64_t size = kDev ? s_step.size_after : vector_read(&ka->late.size, opaque_zero);
-    const float beta = vector_read(&ka->late.beta, opaque_zero);
-    const uint64_t seed = vector_read(&ka->late.seed, opaque_zero);
-    const uint64_t calls = kDev ? s_step.calls : vector_read(&ka->late.calls, opaque_zero);
-    int64_t* const out_idx = vector_read(&ka->late.out_idx, opaque_zero);
-    float* const out_w = vector_read(&ka->late.out_w, opaque_zero);
     // the strata's draws: needed a barrier from here
     float u = 0.0f;
     if (tid < batch && uniforms) u = ((const __attribute__((address_space(1))) float*)uniforms)[tid];
-    if (walker) {  // from the pushed row's leaf to the root
+    if (walker) {  // from the pushed row's leaf to the root: first thing, the others wait for it
         float q = 0.0f;
         bool given = false;
         if (priority) {
@@ -3277,6 +3277,18 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
         step_walk(a, leaf_node, sib_node, sib_s, sib_m, old_max, given, q, top_s, top_m, top_nodes, s_step, lane);
         if (lane == 0 && s_step.flags) atomicOr(err_early, s_step.flags);
     }
+    // (behind the tables and the walk, i.e. behind every use of what was requested when the kernel started: a wave's
+    // requests come back in order, and a wait for an old one that the compiler cannot tell from these would wait for these)
+    asm volatile("" ::"v"(uniforms), "v"(u));
+    const StepKernargPtr ka = step_kernarg(true);
+    uint32_t* const err = vector_read(&ka->late.err, opaque_zero);
+    const int put_fields = vector_read(&ka->late.put.nfields, opaque_zero), get_fields = vector_read(&ka->late.get.nfields, opaque_zero);
+    const int64_t size = kDev ? s_step.size_after : vector_read(&ka->late.size, opaque_zero);
+    const float beta = vector_read(&ka->late.beta, opaque_zero);
+    const uint64_t seed = vector_read(&ka->late.seed, opaque_zero);
+    const uint64_t calls = kDev ? s_step.calls : vector_read(&ka->late.calls, opaque_zero);
+    int64_t* const out_idx = vector_read(&ka->late.out_idx, opaque_zero);
+    float* const out_w = vector_read(&ka->late.out_w, opaque_zero);
     lds_barrier();
     // ---- the sample's descent; the other waves find their granules' places meanwhile
     const bool mine = tid < batch;
@@ -3327,6 +3339,10 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
         dst0 = as_global(s_get.io[f0]) + (uint64_t)row0 * s_get.row_bytes[f0] + off0;
     }
     lds_barrier();
+    // Threads with neither a stratum nor a granule - whole waves of them on a small batch - write the tree's top back
+    // while the others work (nothing below reads the top from memory); else everybody does at the end.
+    const bool spare_back = behind + work + 64u <= (uint32_t)kStepThreads;
+    if (spare_back && tid >= behind + work) top_write_back_by(a, top_s, top_m, tid - (behind + work), kStepThreads - (behind + work));
     // ---- the rows (a sampled row that is the pushed one is read where the push reads it: its store may still be on
     // its way), the weights while they are on their way, the outputs behind them
     AnyGranule first_granule;
@@ -3359,7 +3375,7 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
         for (int j = 0; j < kPutPer; ++j)
             if (lane + 64u * j < put_work) put_granule[j].store(put_place[j].dst, put_place[j].vl);
     }
-    top_write_back(a, top_s, top_m, kStepThreads);  // (last: its stores are ahead of no load)
+    if (!spare_back) top_write_back(a, top_s, top_m, kStepThreads);  // (last: its stores are ahead of no load)
 }
 
 template <bool kDev>
