@@ -734,7 +734,8 @@ int per_update(Per& pb, const int64_t* indices, const float* priorities, int64_t
     // (k_tree_wg; on deeper trees or with more entries one compute unit's memory traffic costs more than a launch.
     // On these trees it also beats the one-wave kernel below for 64 entries or fewer: 5.45 against 5.87 us at 64.)
     if (!sparse && b->fused && n <= kWgBestEntries && b->depth >= 2 && b->depth <= kWgMaxDepth) {
-        const uint32_t threads = n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
+        // (65 to 128 entries: 1024 threads, eight per entry - the kernel's one-step path below the staged top)
+        const uint32_t threads = n > 64 && n <= 128 ? 1024u : n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
         hipLaunchKernelGGL(k_tree_wg, dim3(1), dim3(threads), 0, s, a.indices, a.priorities, a.sum, a.mn, a.maxp, (int)a.n,
                            a.depth, (int)a.capacity, a.alpha, a);
         LAUNCH_CHECK("k_tree_wg");
@@ -1349,7 +1350,8 @@ int mrb_per_update_push(int64_t h, const int64_t* indices, const float* prioriti
             const int64_t slot = b->device_counters ? -1 : first;
             // (readers: the waves that read the device's counters - the tree wave and every wave of the row copy)
             if (wg) {
-                const uint32_t threads = n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
+                // (65 to 128 entries: 1024 threads, eight per entry - the kernel's one-step path below the staged top)
+        const uint32_t threads = n > 64 && n <= 128 ? 1024u : n <= kWgMinThreads ? (uint32_t)kWgMinThreads : (uint32_t)((n + 63) / 64 * 64);
                 a.readers = 1 + put.blocks * (threads / 64);
                 hipLaunchKernelGGL(b->device_counters ? k_tree_wg_push<true> : k_tree_wg_push<false>, dim3(1 + put.blocks),
                                    dim3(threads), 0, s, a.indices, a.priorities, a.sum, a.mn, a.maxp, (int)a.n, a.depth,

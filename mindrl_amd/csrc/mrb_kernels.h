@@ -2431,7 +2431,7 @@ __global__ __launch_bounds__(kWG) void k_push_one(float* __restrict__ sum, float
 //     with it; the others stop (with consecutive slots in a call, hundreds of threads would otherwise hammer
 //     one hash slot).
 //   * entries aimed at one leaf elect the latest among them with a 64-bit LDS maximum of (position, p^alpha).
-//   * a call of at most 64 entries (eight threads of the 512 per entry) takes the levels below the staged top in ONE
+//   * a call of at most 64 entries (eight threads of the 512 per entry; at most 128 when launched with 1024) takes the levels below the staged top in ONE
 //     step and without the rotating tables: lane j of an entry's cluster holds leaf j of the entry's group - memory's
 //     value or, looked up in the election's table, the call's -, the cluster rebuilds the group's levels among its
 //     lanes (exchanges inside a row of lanes) and puts the group's root into the staged top, where the entry's own

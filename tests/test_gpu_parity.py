@@ -1709,7 +1709,7 @@ def test_update_push_equals_update_then_push(mrb, orc, cap):
         serial += n
     exp_flags = 0
     for step, (k, nrows) in enumerate([(1, 1), (64, 1), (17, 1), (300, 1), (512, 4), (40, 3), (1000, 7), (1100, 2),
-                                       (512, 1), (64, 1), (200, 300), (5, 20), (384, 1), (65, 1)]):
+                                       (512, 1), (64, 1), (200, 300), (5, 20), (384, 1), (65, 1), (100, 1), (128, 1), (129, 1)]):
         idx = rng.integers(0, cap, k)
         if step % 3 == 0 and k > 4:
             idx[: k // 3] = idx[0]  # duplicates: the last entry wins
