@@ -1518,8 +1518,10 @@ int mrb_per_update_push_sample(int64_t h, const int64_t* indices, const float* p
             late.get = t;
             // (with device_counters the kernel takes the slot, the row count and the generator's call counter from the
             // device and moves them on itself)
-            hipLaunchKernelGGL(b->device_counters ? k_tree_wg_push_sample<true> : k_tree_wg_push_sample<false>, dim3(1),
-                               dim3(kStepThreads), 0, s, indices, priorities, b->sum, b->mn, a.maxp,
+            const bool wide = n > 64 && n <= 128;  // 1024 threads, eight per entry (see k_tree_wg)
+            auto* const kernel = b->device_counters ? (wide ? k_tree_wg_push_sample<true, 1024> : k_tree_wg_push_sample<true, kStepThreads>)
+                                                    : (wide ? k_tree_wg_push_sample<false, 1024> : k_tree_wg_push_sample<false, kStepThreads>);
+            hipLaunchKernelGGL(kernel, dim3(1), dim3(wide ? 1024 : kStepThreads), 0, s, indices, priorities, b->sum, b->mn, a.maxp,
                                (int)(cap << 16 | (b->device_counters ? 0 : first)), (int)(n << 18 | batch << 8) | b->depth, a.alpha,
                                late);
             LAUNCH_CHECK("k_tree_wg_push_sample");

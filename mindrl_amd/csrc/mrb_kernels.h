@@ -2554,7 +2554,7 @@ __device__ __forceinline__ void top_write_back_by(const UpdateArgs& a, const flo
 // caller before the workgroup's first barrier) receives what StepShared describes, watch_leaf being the heap
 // number of the leaf the caller writes next - with kStep == 2 taken from `step` (left there before the first
 // barrier: the caller had to read it from the device).
-template <bool kTake, int kStep = 0>
+template <bool kTake, int kStep = 0, int kThreads = 0>
 __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket& ticket, float*& staged_s, float*& staged_m,
                                              StepShared* step = nullptr, uint32_t watch_leaf = 0) {
     __shared__ __align__(16) float top_s[kWgTopNodes];
@@ -2563,8 +2563,8 @@ __device__ __forceinline__ void tree_wg_body(const UpdateArgs& a, CounterTicket&
     staged_m = top_m;
     __shared__ __align__(16) uint32_t keys[3][kWgSlots];
     __shared__ __align__(16) unsigned long long vals[3][kWgSlots];
-    // (kStep: a fixed number of threads - the launch's own is a read of the kernel-argument segment)
-    const uint32_t tid = threadIdx.x, nthreads = kStep ? (uint32_t)kWgMinThreads : blockDim.x, lane = tid & 63u;
+    // (kThreads: the caller's fixed number of threads - the launch's own is a read of the kernel-argument segment)
+    const uint32_t tid = threadIdx.x, nthreads = kThreads ? (uint32_t)kThreads : blockDim.x, lane = tid & 63u;
     const int D = a.depth;                                // 2 .. kWgMaxDepth
     const int T = D < kWgTopLevels ? D : kWgTopLevels;    // the staged top ends at level T
     const int H = D - T;                                  // levels below it
@@ -2947,7 +2947,7 @@ __global__ __launch_bounds__(kWgMaxEntries) void k_tree_wg_push(MRB_WG_LEAD_PARA
 // The workgroup copies the pushed row itself: the sample may pick it.
 // The results are those of the three calls, bit for bit.
 // ---------------------------------------------------------------------------
-constexpr int kStepThreads = kWgMinThreads;  // most entries, most strata
+constexpr int kStepThreads = kWgMinThreads;  // threads of the kernel (1024 for an update of 65 to 128 entries: eight per entry); most strata
 constexpr uint32_t kStepMaxPut = 2 * 64;  // most granules of the pushed row, which one wave copies
 constexpr uint32_t kStepMaxGather = 64 * kStepThreads;  // most granules of the sampled batch
 
@@ -3151,18 +3151,19 @@ struct GranulePlace {
 // count and the generator's call counter there when the kernel starts (they lie in front of the running max, whose
 // address is preloaded), hands them to the others through LDS and stores them moved on; this one workgroup is the
 // launch's only reader, so nobody has to be waited for. The other instantiation carries none of that.
-template <bool kDev>
-__global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int64_t* __restrict__ indices,
+// kThreads: 512, or 1024 for an update of 65 to 128 entries (eight threads per entry: tree_wg_body's one-step path).
+template <bool kDev, int kThreads>
+__global__ __launch_bounds__(kThreads) void k_tree_wg_push_sample(const int64_t* __restrict__ indices,
                                                                       const float* __restrict__ priorities, float* sum, float* mn,
                                                                       float* maxp, int slot_capacity, int sizes, float alpha,
                                                                       StepLate late_args) {
-    __shared__ int64_t s_slot[kStepThreads];
+    __shared__ int64_t s_slot[kThreads];
     __shared__ LdsTable s_put, s_get;
     __shared__ StepShared s_step;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     // the last wave holds none of the update's entries (n <= 384; lanes of a small call's clusters at most) and walks for
     // the push, the one before it copies the row and carries the two field tables
-    const bool walker = tid >= kStepThreads - 64, putter = !walker && tid >= kStepThreads - 128;
+    const bool walker = tid >= kThreads - 64, putter = !walker && tid >= kThreads - 128;
     const int depth = sizes & 255;
     const uint32_t batch = ((uint32_t)sizes >> 8) & 1023u;
     int64_t slot = slot_capacity & 0xffff;  // (kDev: known to the walking wave first, to the others after the update)
@@ -3243,7 +3244,7 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     }
     CounterTicket none{};
     float *top_s, *top_m;
-    tree_wg_body<false, kDev ? 2 : 1>(a, none, top_s, top_m, &s_step, leaf_node);  // (ends behind a barrier)
+    tree_wg_body<false, kDev ? 2 : 1, kThreads>(a, none, top_s, top_m, &s_step, leaf_node);  // (ends behind a barrier)
     if (kDev) {
         if (walker) {  // the counters moved on (this launch has no other reader of them)
             int64_t* const cnt = counters_before(maxp);
@@ -3326,7 +3327,7 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
         }
     }
     // the weights' common denominator (pmin / total * size)^-beta: by the last wave, unless it holds strata itself
-    const bool spare_wave = batch <= kStepThreads - 64;
+    const bool spare_wave = batch <= kThreads - 64;
     if (spare_wave && walker) {
         const float max_w = powf_det(top_m[1] / total * (float)size, -beta);
         if (lane == 0) s_step.max_w = max_w;
@@ -3334,7 +3335,7 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     // the sampled rows by granule number over the batch, dealt to the threads behind the strata's waves first
     const uint32_t work = (uint32_t)s_get.prefix[get_fields];
     const uint32_t behind = (batch + 63u) & ~63u;
-    const uint32_t w0 = tid >= behind ? tid - behind : tid + kStepThreads - behind;
+    const uint32_t w0 = tid >= behind ? tid - behind : tid + kThreads - behind;
     uint32_t row0 = 0, off0 = 0, vl0 = 0, stride0 = 0;
     int f0 = 0;
     gbyte* dst0 = nullptr;
@@ -3347,8 +3348,8 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
     lds_barrier();
     // Threads with neither a stratum nor a granule - whole waves of them on a small batch - write the tree's top back
     // while the others work (nothing below reads the top from memory); else everybody does at the end.
-    const bool spare_back = behind + work + 64u <= (uint32_t)kStepThreads;
-    if (spare_back && tid >= behind + work) top_write_back_by(a, top_s, top_m, tid - (behind + work), kStepThreads - (behind + work));
+    const bool spare_back = behind + work + 64u <= (uint32_t)kThreads;
+    if (spare_back && tid >= behind + work) top_write_back_by(a, top_s, top_m, tid - (behind + work), kThreads - (behind + work));
     // ---- the rows (a sampled row that is the pushed one is read where the push reads it: its store may still be on
     // its way), the weights while they are on their way, the outputs behind them
     AnyGranule first_granule;
@@ -3369,7 +3370,7 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
         if (!(total > 0.0f) || total > 3.0e38f) atomicOr(err, MRB_DERR_TOTAL);
         if (idx >= size) atomicOr(err, MRB_DERR_UNFILLED);
     }
-    for (uint32_t w = w0 + kStepThreads; w < work; w += kStepThreads) {
+    for (uint32_t w = w0 + kThreads; w < work; w += kThreads) {
         uint32_t row, off;
         const int f = wg_locate(s_get, get_fields, w, row, off);
         const int64_t from = s_slot[row];
@@ -3381,7 +3382,7 @@ __global__ __launch_bounds__(kStepThreads) void k_tree_wg_push_sample(const int6
         for (int j = 0; j < kPutPer; ++j)
             if (lane + 64u * j < put_work) put_granule[j].store(put_place[j].dst, put_place[j].vl);
     }
-    if (!spare_back) top_write_back(a, top_s, top_m, kStepThreads);  // (last: its stores are ahead of no load)
+    if (!spare_back) top_write_back(a, top_s, top_m, kThreads);  // (last: its stores are ahead of no load)
 }
 
 template <bool kDev>

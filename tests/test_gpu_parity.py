@@ -1774,7 +1774,7 @@ def test_update_push_sample_equals_the_three_calls(mrb, orc, cap, batch, gen):
     serial = fill
     exp_flags = 0
     for step, (k, nrows) in enumerate([(1, 1), (64, 1), (17, 1), (300, 1), (384, 1), (385, 1), (40, 3), (64, 1), (2, 1),
-                                       (200, 1), (64, 1), (33, 1), (64, 2), (64, 1)]):
+                                       (200, 1), (64, 1), (33, 1), (64, 2), (64, 1), (65, 1), (100, 1), (128, 1), (129, 1)]):
         idx = rng.integers(0, min(cap, serial), k)
         if step % 3 == 0 and k > 4:
             idx[: k // 3] = idx[0]  # duplicates: the last entry wins
@@ -1929,7 +1929,7 @@ def test_whole_step_calls_in_bursts_without_a_wait(mrb, orc, seed):
         first = rng.integers(0, min(cap, c.size), batch)
         steps = []
         for k in range(nb):
-            n = batch if follow else int(rng.choice([1, 7, 64, int(rng.integers(1, 385)), 384, 385]))
+            n = batch if follow else int(rng.choice([1, 7, 64, 65, 128, int(rng.integers(1, 385)), 384, 385]))
             ent = rng.integers(0, min(cap, c.size), n)
             if n > 4 and rng.integers(0, 3) == 0:
                 ent[: n // 3] = ent[0]
